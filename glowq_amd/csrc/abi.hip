@@ -1,0 +1,289 @@
+// C ABI of the library: argument validation, route selection, launches.  No torch types, no
+// allocation, no synchronisation; see include/glowq_w4a16.h for the contract of each entry point.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace glowq {
+// gemv.hip
+hipError_t launch_wave_dot(GroupDev& g, int rows_per_task, int num_cus, hipStream_t stream);
+hipError_t launch_generic(GroupDev& g, int num_cus, hipStream_t stream);
+int wave_dot_rows(long total_rows);
+size_t wave_dot_lds_bytes(int M, int K, int rank, bool has_r);
+// misc.hip
+hipError_t launch_dequant(const int32_t*, const half_t*, const int32_t*, half_t*, int, int, int, int, int, int, int,
+                          hipStream_t);
+hipError_t launch_unpack(const int32_t*, uint8_t*, int, int, int, int, hipStream_t);
+hipError_t launch_shared_proj_small(const half_t*, const half_t*, half_t*, int, int, int, hipStream_t);
+// skinny.hip / gemm.hip
+bool skinny_supported(const GroupDev& g);
+hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream);
+bool gemm_supported(const GroupDev& g);
+hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream);
+hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t);
+}  // namespace glowq
+
+using namespace glowq;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int num_cus() {
+  // one value per device; the current device is the one the caller's tensors live on
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3;
+constexpr int kWaveDotMaxM = 4;
+constexpr size_t kLdsLimit = 160 * 1024;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+// The fast routes read weights in 16-byte units of 32 codes: a unit must not straddle a
+// quantisation group and every row must start 16-byte aligned.
+bool fast_layout(const GroupDev& g) {
+  if ((g.K & 31) != 0 || (g.group_size & 31) != 0) return false;
+  if (!aligned16(g.x)) return false;
+  for (int i = 0; i < g.n_members; ++i) {
+    const MemberDev& m = g.mem[i];
+    if (!aligned16(m.qweight) || (m.ldw & 3) != 0) return false;
+    if (m.L && !aligned4(m.L)) return false;
+  }
+  if (g.r && !aligned4(g.r)) return false;
+  return true;
+}
+
+int check_common(const void* x, int M, int K, int group_size) {
+  if (x == nullptr) return fail(GLOWQ_EINVAL, "inputs must be a device pointer (got NULL)");
+  if (M <= 0 || K <= 0) return fail(GLOWQ_EINVAL, "inputs must be [M, IC] with M > 0 and IC > 0 (got M=%d, IC=%d)", M, K);
+  if (group_size <= 0) return fail(GLOWQ_EINVAL, "group_size must be > 0");
+  if (group_size % 8 != 0) return fail(GLOWQ_EINVAL, "group_size must be a multiple of 8");
+  return GLOWQ_OK;
+}
+
+int check_member(const glowq_member_t& m, int K, int group_size, int idx) {
+  const int groups = (K + group_size - 1) / group_size;
+  const int packed_iters = (K + 7) / 8;
+  if (m.qweight == nullptr || m.scales == nullptr || m.qzeros == nullptr || m.y == nullptr)
+    return fail(GLOWQ_EINVAL, "member %d: qweight, scales, qzeros and y must be device pointers", idx);
+  if (m.N <= 0) return fail(GLOWQ_EINVAL, "member %d: OC must be > 0", idx);
+  if (m.lds < groups) return fail(GLOWQ_ESHAPE, "member %d: scales groups mismatch (%d < %d)", idx, m.lds, groups);
+  if (m.ldw_i32 < packed_iters)
+    return fail(GLOWQ_ESHAPE, "member %d: qweight packed cols too small (%d < %d)", idx, m.ldw_i32, packed_iters);
+  if (m.ldz_i32 < (groups + 7) / 8)
+    return fail(GLOWQ_ESHAPE, "member %d: qzeros packed cols too small (%d < %d)", idx, m.ldz_i32, (groups + 7) / 8);
+  if (m.ldy < m.N) return fail(GLOWQ_ESHAPE, "member %d: output row stride %d < OC %d", idx, m.ldy, m.N);
+  return GLOWQ_OK;
+}
+
+void to_dev(const glowq_member_t& s, MemberDev& d) {
+  d.qweight = s.qweight;
+  d.scales = static_cast<const half_t*>(s.scales);
+  d.qzeros = s.qzeros;
+  d.L = static_cast<const half_t*>(s.L);
+  d.bias = static_cast<const half_t*>(s.bias);
+  d.y = static_cast<half_t*>(s.y);
+  d.N = s.N;
+  d.ldw = s.ldw_i32;
+  d.lds = s.lds;
+  d.ldz = s.ldz_i32;
+  d.ldy = s.ldy;
+}
+
+int pick_route(const GroupDev& g, int force) {
+  if (!fast_layout(g)) return kRouteGeneric;
+  if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
+  if (g.M <= kWaveDotMaxM && force != kRouteSkinny &&
+      wave_dot_lds_bytes(g.M, g.K, g.rank, g.r != nullptr) <= kLdsLimit)
+    return kRouteWaveDot;
+  if (skinny_supported(g)) return kRouteSkinny;
+  if (gemm_supported(g)) return kRouteGemm;
+  return kRouteGeneric;
+}
+
+// Runs one group through the chosen route.  Routes with a row capacity smaller than M walk the
+// token rows in chunks (weights are re-read once per chunk).
+int run_group(GroupDev g, int route, hipStream_t stream) {
+  const int cus = num_cus();
+  hipError_t e = hipSuccess;
+  if (route == kRouteGemm) {
+    e = launch_gemm(g, cus, stream);
+  } else if (route == kRouteSkinny) {
+    e = launch_skinny(g, cus, stream);
+  } else {
+    const int cap = (route == kRouteWaveDot) ? kWaveDotMaxM : 65535;
+    long rows = 0;
+    for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
+    const int M = g.M;
+    const half_t* x0 = g.x;
+    const half_t* r0 = g.r;
+    half_t* y0[GLOWQ_MAX_MEMBERS];
+    for (int i = 0; i < g.n_members; ++i) y0[i] = g.mem[i].y;
+    for (int m0 = 0; m0 < M && e == hipSuccess; m0 += cap) {
+      g.M = (M - m0 < cap) ? M - m0 : cap;
+      g.x = x0 + (size_t)m0 * g.K;
+      g.r = r0 ? r0 + (size_t)m0 * g.rank : nullptr;
+      for (int i = 0; i < g.n_members; ++i) g.mem[i].y = y0[i] + (size_t)m0 * g.mem[i].ldy;
+      e = (route == kRouteWaveDot) ? launch_wave_dot(g, wave_dot_rows(rows), cus, stream) : launch_generic(g, cus, stream);
+    }
+  }
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int forward_single(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros, void* y, int M,
+                   int K, int N, int group_size, int ldw, int lds, int ldz, int force, void* stream) {
+  int rc = check_common(x, M, K, group_size);
+  if (rc) return rc;
+  glowq_member_t mem;
+  memset(&mem, 0, sizeof(mem));
+  mem.qweight = qweight;
+  mem.scales = scales;
+  mem.qzeros = qzeros;
+  mem.y = y;
+  mem.N = N;
+  mem.ldw_i32 = ldw;
+  mem.lds = lds;
+  mem.ldz_i32 = ldz;
+  mem.ldy = N;
+  rc = check_member(mem, K, group_size, 0);
+  if (rc) return rc;
+  GroupDev g;
+  memset(&g, 0, sizeof(g));
+  g.x = static_cast<const half_t*>(x);
+  g.n_members = 1;
+  g.M = M;
+  g.K = K;
+  g.group_size = group_size;
+  to_dev(mem, g.mem[0]);
+  return run_group(g, pick_route(g, force), static_cast<hipStream_t>(stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+int glowq_version(void) { return 100; }
+
+const char* glowq_last_error(void) { return g_err; }
+
+int glowq_w4a16_gemv_forward(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                             void* y, int M, int K, int N, int group_size, int ldw_i32, int lds, int ldz_i32,
+                             void* stream) {
+  return forward_single(x, qweight, scales, qzeros, y, M, K, N, group_size, ldw_i32, lds, ldz_i32, -1, stream);
+}
+
+int glowq_w4a16_gemm_forward(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                             void* y, int M, int K, int N, int group_size, int split_k_iters, int ldw_i32, int lds,
+                             int ldz_i32, void* stream) {
+  (void)split_k_iters;
+  return forward_single(x, qweight, scales, qzeros, y, M, K, N, group_size, ldw_i32, lds, ldz_i32, kRouteGemm, stream);
+}
+
+int glowq_w4a16_dequant(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out, int N, int K,
+                        int group_size, int ldw_i32, int lds, int ldz_i32, void* stream) {
+  if (!qweight || !scales || !qzeros || !out) return fail(GLOWQ_EINVAL, "dequant: NULL pointer");
+  if (N <= 0 || K <= 0) return fail(GLOWQ_EINVAL, "dequant: N and K must be > 0");
+  if (group_size <= 0 || group_size % 8 != 0) return fail(GLOWQ_EINVAL, "group_size must be a multiple of 8");
+  const int groups = (K + group_size - 1) / group_size;
+  if (lds < groups) return fail(GLOWQ_ESHAPE, "scales groups mismatch");
+  if (ldw_i32 < (K + 7) / 8) return fail(GLOWQ_ESHAPE, "qweight packed cols too small");
+  if (ldz_i32 < (groups + 7) / 8) return fail(GLOWQ_ESHAPE, "qzeros packed cols too small");
+  hipError_t e = launch_dequant(qweight, static_cast<const half_t*>(scales), qzeros, static_cast<half_t*>(out), N, K,
+                                group_size, ldw_i32, lds, ldz_i32, num_cus(), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "dequant launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int glowq_unpack_int4(const int32_t* packed, uint8_t* codes, int rows, int total_vals, int ld_i32, void* stream) {
+  if (!packed || !codes) return fail(GLOWQ_EINVAL, "unpack: NULL pointer");
+  if (rows <= 0 || total_vals <= 0) return fail(GLOWQ_EINVAL, "unpack: rows and total_vals must be > 0");
+  if (ld_i32 < (total_vals + 7) / 8) return fail(GLOWQ_ESHAPE, "unpack: packed cols too small");
+  hipError_t e = launch_unpack(packed, codes, rows, total_vals, ld_i32, num_cus(), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "unpack launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int rank, void* stream) {
+  if (!x || !R || !r) return fail(GLOWQ_EINVAL, "shared_proj: NULL pointer");
+  if (M <= 0 || K <= 0 || rank <= 0) return fail(GLOWQ_EINVAL, "shared_proj: M, K and rank must be > 0");
+  const half_t* xp = static_cast<const half_t*>(x);
+  const half_t* Rp = static_cast<const half_t*>(R);
+  half_t* rp = static_cast<half_t*>(r);
+  hipError_t e;
+  if (M > 16 && (K & 31) == 0 && (rank & 15) == 0 && aligned16(x) && aligned16(R)) {
+    e = launch_shared_proj_mfma(xp, Rp, rp, M, K, rank, num_cus(), static_cast<hipStream_t>(stream));
+  } else {
+    if ((K & 7) == 0 && (!aligned16(x) || !aligned16(R)))
+      return fail(GLOWQ_EUNSUPPORTED, "shared_proj: x and R must be 16-byte aligned");
+    e = launch_shared_proj_small(xp, Rp, rp, M, K, rank, static_cast<hipStream_t>(stream));
+  }
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
+                              int K, int group_size, int rank, float alpha, void* stream) {
+  int rc = check_common(x, M, K, group_size);
+  if (rc) return rc;
+  if (members == nullptr || n_members < 1 || n_members > GLOWQ_MAX_MEMBERS)
+    return fail(GLOWQ_EINVAL, "group_forward: n_members must be 1..%d", GLOWQ_MAX_MEMBERS);
+  GroupDev g;
+  memset(&g, 0, sizeof(g));
+  bool any_L = false;
+  for (int i = 0; i < n_members; ++i) {
+    rc = check_member(members[i], K, group_size, i);
+    if (rc) return rc;
+    to_dev(members[i], g.mem[i]);
+    any_L = any_L || members[i].L != nullptr;
+  }
+  if (any_L && alpha != 0.0f) {
+    if (r == nullptr) return fail(GLOWQ_EINVAL, "group_forward: a member has L but r is NULL");
+    if (rank <= 0) return fail(GLOWQ_EINVAL, "group_forward: rank must be > 0 when a correction is applied");
+    g.r = static_cast<const half_t*>(r);
+    g.rank = rank;
+    g.alpha = alpha;
+  } else {
+    for (int i = 0; i < n_members; ++i) g.mem[i].L = nullptr;  // alpha == 0: the reference returns z untouched
+  }
+  g.x = static_cast<const half_t*>(x);
+  g.n_members = n_members;
+  g.M = M;
+  g.K = K;
+  g.group_size = group_size;
+  return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
+}
+
+int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
+  GroupDev g;
+  memset(&g, 0, sizeof(g));
+  g.n_members = 1;
+  g.M = M;
+  g.K = K;
+  g.group_size = group_size;
+  g.mem[0].N = N;
+  g.mem[0].ldw = ldw_i32;
+  return pick_route(g, -1);
+}
+
+}  // extern "C"

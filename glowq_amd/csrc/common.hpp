@@ -1,0 +1,80 @@
+// Shared device helpers for the gfx950 W4A16 + GlowQ kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/glowq_w4a16.h"
+
+namespace glowq {
+
+typedef _Float16 half_t;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// Device-side copy of one group member (pointers already typed).
+struct MemberDev {
+  const int32_t* qweight;
+  const half_t* scales;
+  const int32_t* qzeros;
+  const half_t* L;
+  const half_t* bias;
+  half_t* y;
+  int N, ldw, lds, ldz, ldy;
+};
+
+struct GroupDev {
+  const half_t* x;  // [M, K]
+  const half_t* r;  // [M, rank] or nullptr
+  MemberDev mem[GLOWQ_MAX_MEMBERS];
+  int task_end[GLOWQ_MAX_MEMBERS];  // exclusive prefix of per-member task counts
+  int n_members;
+  int M, K, group_size, rank;
+  float alpha;
+};
+
+__device__ __forceinline__ uint32_t nibble(uint32_t word, int idx) { return (word >> (4 * idx)) & 0xFu; }
+
+template <typename T>
+__device__ __forceinline__ T bitcast_u32(uint32_t v) {
+  return __builtin_bit_cast(T, v);
+}
+
+// Sum over the 64 lanes of a wave; every lane gets the total.  Four DPP steps reduce each row of
+// 16 lanes, the four row totals are then combined through scalar lane reads.
+__device__ __forceinline__ float wave_sum(float v) {
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true);  // row_half_mirror
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true);  // row_mirror
+  v += __builtin_bit_cast(float, t);
+  const int iv = __builtin_bit_cast(int, v);
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+  return (a + b) + (c + d);
+}
+
+// Sum over the 4 lanes of a quad; every lane of the quad gets the total.
+__device__ __forceinline__ float quad_sum(float v) {
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true);
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true);
+  v += __builtin_bit_cast(float, t);
+  return v;
+}
+
+}  // namespace glowq

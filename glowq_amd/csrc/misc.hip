@@ -1,0 +1,135 @@
+// Small kernels around the main path: dequantisation to fp16, nibble unpacking, and the shared
+// right-factor projection r = x R^T for few token rows.
+#include "common.hpp"
+
+namespace glowq {
+
+// out[n, k] = fp16((code - zero) * scale): fp32 multiply, one rounding.  One thread per int32 word.
+__global__ __launch_bounds__(256) void dequant_kernel(const int32_t* __restrict__ qweight,
+                                                      const half_t* __restrict__ scales,
+                                                      const int32_t* __restrict__ qzeros, half_t* __restrict__ out,
+                                                      int N, int K, int group_size, int ldw, int lds, int ldz) {
+  const int words = (K + 7) >> 3;
+  const long total = (long)N * words;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int n = (int)(idx / words);
+    const int w = (int)(idx - (long)n * words);
+    const int k0 = w << 3;
+    const int grp = k0 / group_size;  // a word never straddles groups: group_size is a multiple of 8
+    const float s = (float)scales[(size_t)n * lds + grp];
+    const float z = (float)nibble((uint32_t)qzeros[(size_t)n * ldz + (grp >> 3)], grp & 7);
+    const uint32_t pw = (uint32_t)qweight[(size_t)n * ldw + w];
+    half_t* o = out + (size_t)n * K + k0;
+    if (k0 + 8 <= K && (K & 7) == 0) {
+      h8 v;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = (half_t)(((float)nibble(pw, i) - z) * s);
+      *reinterpret_cast<h8*>(o) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (k0 + i < K) o[i] = (half_t)(((float)nibble(pw, i) - z) * s);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void unpack_kernel(const int32_t* __restrict__ packed, uint8_t* __restrict__ codes,
+                                                     int rows, int total_vals, int ld) {
+  const long total = (long)rows * total_vals;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int rrow = (int)(idx / total_vals);
+    const int k = (int)(idx - (long)rrow * total_vals);
+    codes[idx] = (uint8_t)nibble((uint32_t)packed[(size_t)rrow * ld + (k >> 3)], k & 7);
+  }
+}
+
+// r[m, j] = fp16(sum_k x[m,k] R[j,k]).  One workgroup per (row j of R, chunk of kM token rows): the
+// 256 threads stride over the row in 16-byte pieces and reduce through DPP and LDS.
+template <int kM>
+__global__ __launch_bounds__(256) void shared_proj_kernel(const half_t* __restrict__ x, const half_t* __restrict__ R,
+                                                          half_t* __restrict__ r, int M, int K, int rank) {
+  __shared__ float part[4][kM];
+  const int j = blockIdx.x;
+  const int m0 = blockIdx.y * kM;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  float acc[kM];
+#pragma unroll
+  for (int m = 0; m < kM; ++m) acc[m] = 0.f;
+  const half_t* Rrow = R + (size_t)j * K;
+  if ((K & 7) == 0) {
+    const int words = K >> 3;
+    for (int w = threadIdx.x; w < words; w += blockDim.x) {
+      const h8 rv = reinterpret_cast<const h8*>(Rrow)[w];
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+        const int mm = min(m0 + m, M - 1);
+        const h8 xv = reinterpret_cast<const h8*>(x + (size_t)mm * K)[w];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const h2 a = {rv[2 * i], rv[2 * i + 1]};
+          const h2 b = {xv[2 * i], xv[2 * i + 1]};
+          acc[m] = __builtin_amdgcn_fdot2(a, b, acc[m], false);
+        }
+      }
+    }
+  } else {
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+      const float rv = (float)Rrow[k];
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+        const int mm = min(m0 + m, M - 1);
+        acc[m] = __builtin_fmaf(rv, (float)x[(size_t)mm * K + k], acc[m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < kM; ++m) {
+    const float v = wave_sum(acc[m]);
+    if (lane == 0) part[wave][m] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < kM) {
+    const int m = m0 + threadIdx.x;
+    if (m < M) {
+      const float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+      r[(size_t)m * rank + j] = (half_t)v;
+    }
+  }
+}
+
+hipError_t launch_dequant(const int32_t* qw, const half_t* sc, const int32_t* qz, half_t* out, int N, int K, int gs,
+                          int ldw, int lds, int ldz, int num_cus, hipStream_t stream) {
+  const long total = (long)N * ((K + 7) >> 3);
+  long blocks = (total + 255) / 256;
+  const long cap = (long)num_cus * 32;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, qw, sc, qz, out, N, K, gs, ldw, lds, ldz);
+  return hipGetLastError();
+}
+
+hipError_t launch_unpack(const int32_t* packed, uint8_t* codes, int rows, int total_vals, int ld, int num_cus,
+                         hipStream_t stream) {
+  const long total = (long)rows * total_vals;
+  long blocks = (total + 255) / 256;
+  const long cap = (long)num_cus * 32;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, packed, codes, rows, total_vals, ld);
+  return hipGetLastError();
+}
+
+hipError_t launch_shared_proj_small(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank,
+                                    hipStream_t stream) {
+  if (M == 1) {
+    hipLaunchKernelGGL(shared_proj_kernel<1>, dim3(rank, 1), dim3(256), 0, stream, x, R, r, M, K, rank);
+  } else if (M == 2) {
+    hipLaunchKernelGGL(shared_proj_kernel<2>, dim3(rank, 1), dim3(256), 0, stream, x, R, r, M, K, rank);
+  } else {
+    hipLaunchKernelGGL(shared_proj_kernel<4>, dim3(rank, (M + 3) / 4), dim3(256), 0, stream, x, R, r, M, K, rank);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace glowq

@@ -1,0 +1,262 @@
+"""Loader and tensor-level front end of libglowq_w4a16.so (hand-written HIP for gfx950).
+
+Mirrors the reference's extension loader (src/cuda_w4a16/kernels.py:16-59) and the three functions
+its pybind module exports (src/cuda_w4a16/csrc/pybind.cpp:19-34):
+
+    ext = load_w4a16_extension()
+    y = ext.w4a16_gemv_forward_cuda(x, qweight, scales, qzeros, group_size)
+    y = ext.w4a16_gemm_forward_cuda(x, qweight, scales, qzeros, group_size, split_k_iters)
+    y = ext.gemv_w4a16_asym(...)                      # alias of the GEMV entry
+
+plus the group-level entry points this implementation adds (`shared_proj`, `group_forward`,
+`dequant`, `unpack_int4`).  The library itself is a plain C ABI (include/glowq_w4a16.h); torch is used
+only for device memory and the current HIP stream.  There is no CPU or eager fallback: a missing
+library raises, as the reference's loader does (kernels.py:24-32).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import List, Optional, Sequence
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libglowq_w4a16.so")
+MAX_MEMBERS = 4
+
+_ext = None
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+
+
+class _Member(ctypes.Structure):
+    _fields_ = [
+        ("qweight", _P), ("scales", _P), ("qzeros", _P), ("L", _P), ("bias", _P), ("y", _P),
+        ("N", ctypes.c_int32), ("ldw_i32", ctypes.c_int32), ("lds", ctypes.c_int32),
+        ("ldz_i32", ctypes.c_int32), ("ldy", ctypes.c_int32), ("reserved", ctypes.c_int32),
+    ]
+
+
+_SIGNATURES = {
+    "glowq_version": (ctypes.c_int, []),
+    "glowq_last_error": (ctypes.c_char_p, []),
+    "glowq_w4a16_gemv_forward": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "glowq_w4a16_gemm_forward": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "glowq_w4a16_dequant": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "glowq_unpack_int4": (_I, [_P, _P, _I, _I, _I, _P]),
+    "glowq_shared_proj": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
+}
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+class W4A16Extension:
+    """Tensor-level wrappers over the C ABI.  Every call launches on torch's current stream."""
+
+    def __init__(self, lib: ctypes.CDLL):
+        self.lib = lib
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        self.version = lib.glowq_version()
+
+    # ------------------------------------------------------------------ helpers
+    def _raise(self, rc: int, what: str):
+        msg = self.lib.glowq_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what}: {msg} (code {rc})")
+
+    @staticmethod
+    def _stream(dev: torch.device) -> int:
+        return torch.cuda.current_stream(dev).cuda_stream
+
+    @staticmethod
+    def _check_quant(x, qweight, scales, qzeros, group_size):
+        _check(x.is_cuda, "inputs must be CUDA")
+        _check(qweight.is_cuda, "qweight must be CUDA")
+        _check(scales.is_cuda, "scales must be CUDA")
+        _check(qzeros.is_cuda, "qzeros must be CUDA")
+        _check(x.dtype == torch.float16, "inputs must be fp16")
+        _check(qweight.dtype == torch.int32, "qweight must be int32 (8x int4 packed)")
+        _check(scales.dtype == torch.float16, "scales must be fp16")
+        _check(qzeros.dtype == torch.int32, "qzeros must be int32 (8x int4 packed)")
+        _check(x.dim() == 2, "inputs must be [M, IC]")
+        _check(qweight.dim() == 2, "qweight must be [OC, packed_i32]")
+        _check(scales.dim() == 2, "scales must be [OC, groups]")
+        _check(qzeros.dim() == 2, "qzeros must be [OC, groups_packed]")
+        _check(group_size > 0, "group_size must be > 0")
+        _check(group_size % 8 == 0, "group_size must be a multiple of 8")
+        _check(scales.size(0) == qweight.size(0), "scales OC mismatch")
+        _check(qzeros.size(0) == qweight.size(0), "qzeros OC mismatch")
+
+    # ------------------------------------------------------------------ reference-named entry points
+    def w4a16_gemv_forward_cuda(self, x, qweight, scales, qzeros, group_size: int) -> torch.Tensor:
+        self._check_quant(x, qweight, scales, qzeros, group_size)
+        x, qweight, scales, qzeros = x.contiguous(), qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+        M, K = x.shape
+        N = qweight.size(0)
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+        if M == 0 or N == 0:
+            return out
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_w4a16_gemv_forward(
+                x.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
+                M, K, N, int(group_size), qweight.size(1), scales.size(1), qzeros.size(1), self._stream(x.device))
+        if rc:
+            self._raise(rc, "w4a16_gemv_forward")
+        return out
+
+    gemv_w4a16_asym = w4a16_gemv_forward_cuda
+
+    def w4a16_gemm_forward_cuda(self, x, qweight, scales, qzeros, group_size: int, split_k_iters: int = 1) -> torch.Tensor:
+        self._check_quant(x, qweight, scales, qzeros, group_size)
+        x, qweight, scales, qzeros = x.contiguous(), qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+        M, K = x.shape
+        N = qweight.size(0)
+        out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+        if M == 0 or N == 0:
+            return out
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_w4a16_gemm_forward(
+                x.data_ptr(), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(),
+                M, K, N, int(group_size), int(split_k_iters), qweight.size(1), scales.size(1), qzeros.size(1),
+                self._stream(x.device))
+        if rc:
+            self._raise(rc, "w4a16_gemm_forward")
+        return out
+
+    # ------------------------------------------------------------------ additional entry points
+    def dequant(self, qweight, scales, qzeros, in_features: int, group_size: int) -> torch.Tensor:
+        _check(qweight.is_cuda and scales.is_cuda and qzeros.is_cuda, "dequant: tensors must be CUDA")
+        _check(qweight.dtype == torch.int32 and qzeros.dtype == torch.int32 and scales.dtype == torch.float16,
+               "dequant: qweight/qzeros must be int32 and scales fp16")
+        qweight, scales, qzeros = qweight.contiguous(), scales.contiguous(), qzeros.contiguous()
+        N = qweight.size(0)
+        out = torch.empty((N, in_features), dtype=torch.float16, device=qweight.device)
+        with torch.cuda.device(qweight.device):
+            rc = self.lib.glowq_w4a16_dequant(
+                qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(), N, int(in_features),
+                int(group_size), qweight.size(1), scales.size(1), qzeros.size(1), self._stream(qweight.device))
+        if rc:
+            self._raise(rc, "w4a16_dequant")
+        return out
+
+    def unpack_int4(self, packed, total_vals: int) -> torch.Tensor:
+        _check(packed.is_cuda and packed.dtype == torch.int32 and packed.dim() == 2, "unpack: packed must be CUDA int32 [rows, W]")
+        packed = packed.contiguous()
+        rows = packed.size(0)
+        out = torch.empty((rows, total_vals), dtype=torch.uint8, device=packed.device)
+        with torch.cuda.device(packed.device):
+            rc = self.lib.glowq_unpack_int4(packed.data_ptr(), out.data_ptr(), rows, int(total_vals), packed.size(1),
+                                            self._stream(packed.device))
+        if rc:
+            self._raise(rc, "unpack_int4")
+        return out
+
+    def shared_proj(self, x, R, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """r = fp16(x @ R^T); x [M, K] fp16, R [rank, K] fp16."""
+        _check(x.is_cuda and R.is_cuda, "shared_proj: tensors must be CUDA")
+        _check(x.dtype == torch.float16 and R.dtype == torch.float16, "shared_proj: tensors must be fp16")
+        _check(x.dim() == 2 and R.dim() == 2 and x.size(1) == R.size(1), "shared_proj: x [M, K] and R [rank, K] must agree on K")
+        x, R = x.contiguous(), R.contiguous()
+        M, K = x.shape
+        rank = R.size(0)
+        if out is None:
+            out = torch.empty((M, rank), dtype=torch.float16, device=x.device)
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_shared_proj(x.data_ptr(), R.data_ptr(), out.data_ptr(), M, K, rank, self._stream(x.device))
+        if rc:
+            self._raise(rc, "shared_proj")
+        return out
+
+    def group_forward(self, x, r, members: Sequence[dict], group_size: int, alpha: float,
+                      outs: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
+        """One launch for a group.  Each member is a dict with `qweight`, `scales`, `qzeros` and optional
+        `L` ([N, rank] fp16 or None) and `bias` ([N] fp16 or None).  Returns the [M, N_i] fp16 outputs."""
+        _check(1 <= len(members) <= MAX_MEMBERS, f"group_forward: 1..{MAX_MEMBERS} members")
+        _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2, "inputs must be CUDA fp16 [M, IC]")
+        x = x.contiguous()
+        M, K = x.shape
+        arr = (_Member * len(members))()
+        keep = []
+        rank = 0
+        if r is not None:
+            _check(r.is_cuda and r.dtype == torch.float16 and r.dim() == 2 and r.size(0) == M and r.is_contiguous(),
+                   "group_forward: r must be a contiguous CUDA fp16 [M, rank] tensor")
+            rank = r.size(1)
+        result = []
+        for i, m in enumerate(members):
+            qw, sc, qz = m["qweight"], m["scales"], m["qzeros"]
+            self._check_quant(x, qw, sc, qz, group_size)
+            _check(qw.is_contiguous() and sc.is_contiguous() and qz.is_contiguous(), "group_forward: buffers must be contiguous")
+            N = qw.size(0)
+            L = m.get("L")
+            bias = m.get("bias")
+            if L is not None:
+                _check(r is not None, "group_forward: a member has L but no r was given")
+                _check(L.is_cuda and L.dtype == torch.float16 and L.is_contiguous() and tuple(L.shape) == (N, rank),
+                       "group_forward: L must be a contiguous CUDA fp16 [OC, rank] tensor")
+            if bias is not None:
+                _check(bias.is_cuda and bias.dtype == torch.float16 and bias.is_contiguous() and bias.numel() == N,
+                       "group_forward: bias must be a contiguous CUDA fp16 [OC] tensor")
+            y = outs[i] if outs is not None else torch.empty((M, N), dtype=torch.float16, device=x.device)
+            _check(y.is_cuda and y.dtype == torch.float16 and tuple(y.shape) == (M, N) and y.stride(1) == 1,
+                   "group_forward: output must be CUDA fp16 [M, OC]")
+            keep.append((qw, sc, qz, L, bias, y))
+            e = arr[i]
+            e.qweight, e.scales, e.qzeros = qw.data_ptr(), sc.data_ptr(), qz.data_ptr()
+            e.L = L.data_ptr() if L is not None else None
+            e.bias = bias.data_ptr() if bias is not None else None
+            e.y = y.data_ptr()
+            e.N, e.ldw_i32, e.lds, e.ldz_i32, e.ldy = N, qw.size(1), sc.size(1), qz.size(1), y.stride(0)
+            result.append(y)
+        if M == 0:
+            return result
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_w4a16_group_forward(
+                x.data_ptr(), r.data_ptr() if r is not None else None, arr, len(members), M, K, int(group_size),
+                int(rank), float(alpha), self._stream(x.device))
+        if rc:
+            self._raise(rc, "w4a16_group_forward")
+        return result
+
+    def route(self, M: int, K: int, N: int, group_size: int = 128) -> str:
+        names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic"}
+        return names[self.lib.glowq_w4a16_route(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
+
+
+def library_path() -> str:
+    return LIB_PATH
+
+
+def load_w4a16_extension(verbose: Optional[bool] = None) -> W4A16Extension:
+    """Loads the prebuilt in-tree library (python -m glowq_amd.build).  Raises RuntimeError when it is
+    missing or does not load; nothing is compiled at run time and nothing falls back to torch."""
+    global _ext
+    if _ext is not None:
+        return _ext
+    want_verbose = bool(verbose) or os.environ.get("W4A16_VERBOSE", os.environ.get("CUDA_MIXED_VERBOSE", "")).lower() in {
+        "1", "true", "yes", "y", "on"}
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+        ext = W4A16Extension(lib)
+    except (OSError, AttributeError) as exc:
+        raise RuntimeError(
+            "Failed to load the prebuilt glowq W4A16 HIP library "
+            f"({LIB_PATH}). Build it first with:\n  python -m glowq_amd.build\n"
+            "There is no CPU or torch fallback for this path."
+        ) from exc
+    if want_verbose:
+        print(f"[glowq_amd] loaded {LIB_PATH} (version {ext.version})")
+    _ext = ext
+    return _ext
+
+
+__all__ = ["load_w4a16_extension", "W4A16Extension", "library_path", "LIB_PATH", "MAX_MEMBERS"]

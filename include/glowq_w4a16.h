@@ -1,0 +1,126 @@
+/*
+ * glowq_w4a16.h - C ABI of the MI355X (gfx950) implementation of GlowQ's Step-3 inference hot
+ * path: the W4A16 quantised linear (int4 codes packed 8 per int32, asymmetric per-group scale and
+ * zero-point, fp16 activations) fused with the group-shared low-rank correction.
+ *
+ * All pointers are DEVICE pointers unless stated otherwise.  fp16 tensors are passed as
+ * `const void*` (IEEE binary16, row-major).  Every entry point launches asynchronously on
+ * `stream` (a hipStream_t passed as void*; NULL = the default stream), never synchronises and never
+ * allocates.  Return value: GLOWQ_OK (0) or a negative GLOWQ_E* code; `glowq_last_error()` returns
+ * the message of the calling thread's last failure.
+ *
+ * Tensor conventions (identical to the reference's buffers, src/cuda_w4a16/linear.py:104-106):
+ *   x        [M, K]            fp16, row stride K
+ *   qweight  [N, ldw_i32]      int32, element k of row n is nibble (k & 7) of word (k >> 3)
+ *   scales   [N, lds]          fp16, one per group of `group_size` input columns
+ *   qzeros   [N, ldz_i32]      int32, zero-point of group g is nibble (g & 7) of word (g >> 3)
+ *   y        [M, N]            fp16, row stride ldy
+ * Naming of the low-rank factors: R is the shared right factor [rank, K] (the reference's
+ * `B_shared` / wrapper argument `B_q`); L is a module's left factor [N, rank] (the reference's
+ * `{group}.{module}.A` / wrapper argument `A_q`), src/step3_eval_dataset.py:484,506.
+ */
+#ifndef GLOWQ_W4A16_H_
+#define GLOWQ_W4A16_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GLOWQ_OK 0
+#define GLOWQ_EINVAL (-1)     /* bad argument (null pointer, non-positive size, bad group_size) */
+#define GLOWQ_ESHAPE (-2)     /* leading dimensions too small for the stated shape */
+#define GLOWQ_ELAUNCH (-3)    /* the HIP runtime reported a launch error */
+#define GLOWQ_EUNSUPPORTED (-4)
+
+#define GLOWQ_MAX_MEMBERS 4
+
+/* One module of a QKV / MLP group (q, k, v or gate, up), or a solo module (o_proj, down_proj). */
+typedef struct glowq_member {
+  const int32_t* qweight; /* [N, ldw_i32] */
+  const void* scales;     /* [N, lds] fp16 */
+  const int32_t* qzeros;  /* [N, ldz_i32] */
+  const void* L;          /* [N, rank] fp16 left factor, or NULL: no correction (GlowQ-S unselected) */
+  const void* bias;       /* [N] fp16 or NULL */
+  void* y;                /* [M, N] fp16 output, row stride ldy */
+  int32_t N;
+  int32_t ldw_i32;
+  int32_t lds;
+  int32_t ldz_i32;
+  int32_t ldy;
+  int32_t reserved;
+} glowq_member_t;
+
+/* Library / device information. */
+int glowq_version(void);
+const char* glowq_last_error(void);
+
+/*
+ * y = fp16( sum_k (code - zero) * scale * x ), fp32 accumulate, weights never rounded to fp16.
+ * Replaces `w4a16_gemv_forward_cuda` (src/cuda_w4a16/csrc/gemv_w4a16.cu:146-214; pybind
+ * src/cuda_w4a16/csrc/pybind.cpp:19-23).  Any M is accepted; all M rows share one pass over the
+ * weights in chunks of the kernel's row capacity.
+ */
+int glowq_w4a16_gemv_forward(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                             void* y, int M, int K, int N, int group_size, int ldw_i32, int lds, int ldz_i32,
+                             void* stream);
+
+/*
+ * Same contract for the large-M route: replaces `w4a16_gemm_forward_cuda`
+ * (src/cuda_w4a16/csrc/gemm_w4a16.cu:76-135; pybind src/cuda_w4a16/csrc/pybind.cpp:24-27).  The
+ * reference dequantises the whole weight to fp16 in HBM and calls a library GEMM; here the int4 codes
+ * are dequantised on the fly ( fp16((code - zero) * scale), the same single rounding ) and fed to
+ * fp16 MFMA with fp32 accumulate.  `split_k_iters` is accepted and ignored, as in the reference
+ * (gemm_w4a16.cu:83).
+ */
+int glowq_w4a16_gemm_forward(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                             void* y, int M, int K, int N, int group_size, int split_k_iters, int ldw_i32,
+                             int lds, int ldz_i32, void* stream);
+
+/*
+ * out[n, k] = fp16( (code - zero) * scale ), out is [N, K] with row stride K.  Replaces
+ * `dequant_w4a16_asym_i32_kernel` (src/cuda_w4a16/csrc/gemm_w4a16.cu:19-50) and is the device twin of
+ * `CudaW4A16Linear._dequant_chunk` (src/cuda_w4a16/linear.py:248-253).
+ */
+int glowq_w4a16_dequant(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out, int N, int K,
+                        int group_size, int ldw_i32, int lds, int ldz_i32, void* stream);
+
+/*
+ * codes[n, k] = nibble (k & 7) of word (k >> 3), as uint8.  Device twin of `_unpack_int4_i32`
+ * (src/cuda_w4a16/linear.py:49-54; device form src/cuda_w4a16/csrc/gemv_w4a16.cu:16-25).
+ */
+int glowq_unpack_int4(const int32_t* packed, uint8_t* codes, int rows, int total_vals, int ld_i32, void* stream);
+
+/*
+ * r[m, j] = fp16( sum_k x[m, k] * R[j, k] ): the shared right-factor projection, computed once per
+ * group and reused by every member.  Replaces `F.linear(x, B_q)` in `AddSVDCorrection.forward`
+ * (src/step3_eval_dataset.py:484,497,501,504).  r is [M, rank], row stride rank.
+ */
+int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int rank, void* stream);
+
+/*
+ * One launch for a whole group: for every member i
+ *     y_i = fp16( W4A16(x; member i) + bias_i + alpha * r @ L_i^T )
+ * with r = the [M, rank] fp16 result of glowq_shared_proj (may be NULL when no member has L).
+ * Members with L == NULL get no correction (the GlowQ-S selective path).  Replaces, per member, the
+ * sequence inner(x) -> F.linear(r, A_q) -> z.add_(svd_raw, alpha) of `AddSVDCorrection.forward`
+ * (src/step3_eval_dataset.py:470-511) and the selective wrapping of
+ * `patch_svd_correction_wrappers_cumulative` (src/restoration/step4_evaluate_cumulative.py:99-154).
+ * `members` is a HOST pointer to `n_members` (1..GLOWQ_MAX_MEMBERS) descriptors; it is copied
+ * into the launch and may be reused as soon as the call returns.
+ */
+int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
+                              int K, int group_size, int rank, float alpha, void* stream);
+
+/*
+ * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
+ * 2 = tiled MFMA GEMM, 3 = generic (odd shapes).
+ */
+int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* GLOWQ_W4A16_H_ */
