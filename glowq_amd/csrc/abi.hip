@@ -11,7 +11,7 @@ namespace glowq {
 hipError_t launch_wave_dot(GroupDev& g, int rows_per_task, int num_cus, hipStream_t stream);
 hipError_t launch_generic(GroupDev& g, int num_cus, hipStream_t stream);
 int wave_dot_rows(long total_rows);
-size_t wave_dot_lds_bytes(int M, int K, int rank, bool has_r);
+bool wave_dot_supported(int M, int K, int rank, bool has_r);
 // misc.hip
 hipError_t launch_dequant(const int32_t*, const half_t*, const int32_t*, half_t*, int, int, int, int, int, int, int,
                           hipStream_t);
@@ -54,7 +54,6 @@ int num_cus() {
 
 constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3;
 constexpr int kWaveDotMaxM = 4;
-constexpr size_t kLdsLimit = 160 * 1024;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
@@ -63,13 +62,14 @@ bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0
 // quantisation group and every row must start 16-byte aligned.
 bool fast_layout(const GroupDev& g) {
   if ((g.K & 31) != 0 || (g.group_size & 31) != 0) return false;
+  if (((g.group_size >> 5) & ((g.group_size >> 5) - 1)) != 0) return false;  // units per group: a power of two
   if (!aligned16(g.x)) return false;
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
     if (!aligned16(m.qweight) || (m.ldw & 3) != 0) return false;
     if (m.L && !aligned4(m.L)) return false;
   }
-  if (g.r && !aligned4(g.r)) return false;
+  if (g.r && (g.rank & 1) != 0) return false;  // the L rows are read two halves at a time
   return true;
 }
 
@@ -113,8 +113,7 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
-  if (g.M <= kWaveDotMaxM && force != kRouteSkinny &&
-      wave_dot_lds_bytes(g.M, g.K, g.rank, g.r != nullptr) <= kLdsLimit)
+  if (g.M <= kWaveDotMaxM && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr))
     return kRouteWaveDot;
   if (skinny_supported(g)) return kRouteSkinny;
   if (gemm_supported(g)) return kRouteGemm;

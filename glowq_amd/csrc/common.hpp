@@ -35,6 +35,7 @@ struct GroupDev {
   const half_t* r;  // [M, rank] or nullptr
   MemberDev mem[GLOWQ_MAX_MEMBERS];
   int task_end[GLOWQ_MAX_MEMBERS];  // exclusive prefix of per-member task counts
+  int wg_end[GLOWQ_MAX_MEMBERS];    // exclusive prefix of the workgroups assigned to each member
   int n_members;
   int M, K, group_size, rank;
   float alpha;

@@ -11,6 +11,8 @@
 // with a zero exponent field is the subnormal c * 2^-24 (c * 2^-20 for the nibble four bits higher),
 // exact, and v_dot2_f32_f16 multiplies it by x with fp32 accumulation.  Two accumulators keep the two
 // scalings apart; the common 2^24 is applied once per output.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace glowq {
@@ -19,6 +21,18 @@ namespace glowq {
 //   xs  [M][4][U] units of 8 halves: quarter j of unit u holds x[32u + 8j + {0,4,1,5,2,6,3,7}]
 //   sig [M][U]    float: 2^-24 * sum of the 32 activations of unit u
 //   rs  [M][rank] halves (only when a correction is applied)
+// LDS layout of the wave-dot route: x tiles, per-unit sums, then r at a 16-byte aligned offset.
+__host__ __device__ inline size_t wave_dot_r_offset(int M, int K) {
+  const size_t off = (size_t)M * K * sizeof(half_t) + (size_t)M * (K >> 5) * sizeof(float);
+  return (off + 15) & ~(size_t)15;
+}
+
+// partial sums of the slice waves: [2 parities][row blocks per workgroup][slices][rows x tokens] floats;
+
+__host__ __device__ inline size_t wave_dot_part_offset(int M, int K, int rank) {
+  return (wave_dot_r_offset(M, K) + (size_t)M * rank * sizeof(half_t) + 15) & ~(size_t)15;
+}
+
 template <int kM>
 __device__ __forceinline__ void stage_activations(const GroupDev& g, int U, h8* xs, float* sig, half_t* rs) {
   const int words = g.K >> 3;  // 8 halves each
@@ -59,131 +73,180 @@ __device__ __forceinline__ void dot_word(uint32_t w, const h8& xq, float& accA, 
   accB = __builtin_amdgcn_fdot2(c37, x37, accB, false);
 }
 
-template <int kM, int kRows>
-__global__ __launch_bounds__(256) void gemv_wave_dot_kernel(const GroupDev g) {
+// What a wave loads for one row block, all of it issued before anything is used: per row one
+// 16-byte unit of 32 int4 codes, the raw scale and zero-point word of the unit's quantisation group,
+// and kLW dwords (two halves each) of the row of the left factor L.
+template <int kRows, int kLW>
+struct Prefetch {
+  u32x4 w[kRows];
+  half_t sc[kRows];
+  uint32_t zw[kRows];
+  uint32_t l[kRows][kLW > 0 ? kLW : 1];
+};
+
+// Work decomposition.  A row block is kRows consecutive output rows of one member; a wave owns whole
+// row blocks, so no partial sums ever cross waves and the only barrier of the kernel is the one after
+// the activations are staged.  The K extent is cut into `kit` slices of 2048 columns (64 units, one per
+// lane); a step is one slice of one row block and always has the same static shape: kRows coalesced
+// 1 KB loads plus the small loads that go with them, all issued one step ahead of their use.
+// The correction rides along as a K-extension, y = [deq(W) | L] . [x ; alpha r], the L row being spread
+// over the kit steps of its row block (kLW dwords per lane and step).
+// Every workgroup serves ONE member for its whole life (the host splits the grid between the members in
+// proportion to their row blocks), so the member's pointers and strides are loop invariants held in
+// scalar registers and nothing is looked up in memory between two prefetches.
+template <int kM, int kRows, int kLW>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(((kM >= 2 || kRows >= 4) ? 4 : 6), 8)))
+void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int U = g.K >> 5;                 // 16-byte units per row
-  const int upg = g.group_size >> 5;      // units per quantisation group
+  const int U = g.K >> 5;                                  // 16-byte units per weight row
+  const int upg_shift = __builtin_ctz(g.group_size >> 5);  // units per quantisation group = 1 << upg_shift
   h8* xs = reinterpret_cast<h8*>(smem);
   float* sig = reinterpret_cast<float*>(smem + (size_t)kM * g.K * sizeof(half_t));
-  half_t* rs = reinterpret_cast<half_t*>(sig + kM * U);
+  half_t* rs = reinterpret_cast<half_t*>(smem + wave_dot_r_offset(kM, g.K));
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int waves_per_block = blockDim.x >> 6;
-  const int total_tasks = g.task_end[g.n_members - 1];
-  int task = blockIdx.x * waves_per_block + wave;
+
+  // member of this workgroup: every candidate field comes from a fixed kernel-argument offset and is
+  // picked with scalar selects, so the whole lookup costs one round trip to the argument buffer
+  MemberDev mem = g.mem[0];
+  int wg_begin = 0, wg_stop = g.wg_end[0], total_blocks = g.task_end[0];
+#define GLOWQ_PICK(i)                                            \
+  if (g.n_members > i && (int)blockIdx.x >= g.wg_end[i - 1]) {  \
+    mem = g.mem[i];                                              \
+    wg_begin = g.wg_end[i - 1];                                  \
+    wg_stop = g.wg_end[i];                                       \
+    total_blocks = g.task_end[i] - g.task_end[i - 1];            \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
+  const int stride = (wg_stop - wg_begin) * waves_per_block;  // waves serving this member
+  const int ldw_half = g.rank >> 1;                                // dwords per L row
+  const float alpha_scaled = (mem.L != nullptr ? g.alpha : 0.f) * 0x1p-24f;  // accumulators carry 2^-24
+
+  // (row block, slice) of a step; a cursor that ran past the end keeps prefetching the last valid
+  // block (valid addresses) and its steps are never computed
+  struct Cursor {
+    int blk, it;
+  };
+  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW>& p) {
+    const int n0 = min(c.blk, total_blocks - 1) * kRows;
+    const int u = min(lane + c.it * kWave, U - 1);
+    const int grp = u >> upg_shift;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int n = min(n0 + r, mem.N - 1);
+      p.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw) + u);
+      p.sc[r] = mem.scales[(size_t)n * mem.lds + grp];
+      p.zw[r] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (grp >> 3)];
+      if constexpr (kLW > 0) {
+        // a member without L reads r itself (valid memory) and is weighted by zero
+        const uint32_t* lrow = mem.L ? reinterpret_cast<const uint32_t*>(mem.L + (size_t)n * g.rank)
+                                     : reinterpret_cast<const uint32_t*>(g.r);
+#pragma unroll
+        for (int j = 0; j < kLW; ++j) p.l[r][j] = lrow[min((c.it * kLW + j) * kWave + lane, ldw_half - 1)];
+      }
+    }
+  };
+  auto advance = [&](Cursor& c) {
+    if (++c.it == kit) {
+      c.it = 0;
+      c.blk += stride;
+    }
+  };
+
+  float tot[kRows][kM];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r)
+#pragma unroll
+    for (int m = 0; m < kM; ++m) tot[r][m] = 0.f;
+
+  auto compute = [&](const Cursor& c, const Prefetch<kRows, kLW>& p) {
+    const int uraw = lane + c.it * kWave;
+    const bool active = uraw < U;
+    const int u = active ? uraw : U - 1;
+    const int grp = u >> upg_shift;
+    float sc[kRows], zp[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      sc[r] = active ? (float)p.sc[r] : 0.f;
+      zp[r] = (float)nibble(p.zw[r], grp & 7);
+    }
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+      h8 xq[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xq[j] = xs[((size_t)m * 4 + j) * U + u];
+      const float sg = sig[m * U + u];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        float accA = 0.f, accB = 0.f;
+        dot_word(p.w[r].x, xq[0], accA, accB);
+        dot_word(p.w[r].y, xq[1], accA, accB);
+        dot_word(p.w[r].z, xq[2], accA, accB);
+        dot_word(p.w[r].w, xq[3], accA, accB);
+        float v = __builtin_fmaf(accB, 0.0625f, accA);
+        v = __builtin_fmaf(-zp[r], sg, v);
+        tot[r][m] = __builtin_fmaf(sc[r], v, tot[r][m]);
+      }
+    }
+    if constexpr (kLW > 0) {
+#pragma unroll
+      for (int j = 0; j < kLW; ++j) {
+        const int idx = (c.it * kLW + j) * kWave + lane;
+        const float a = idx < ldw_half ? alpha_scaled : 0.f;
+        const int ic = min(idx, ldw_half - 1);
+#pragma unroll
+        for (int m = 0; m < kM; ++m) {
+          const h2 rv = reinterpret_cast<const h2*>(rs + m * g.rank)[ic];
+#pragma unroll
+          for (int r = 0; r < kRows; ++r)
+            tot[r][m] = __builtin_fmaf(a, __builtin_amdgcn_fdot2(bitcast_u32<h2>(p.l[r][j]), rv, 0.f, false), tot[r][m]);
+        }
+      }
+    }
+    if (c.it == kit - 1) {
+      const int n0 = c.blk * kRows;
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+#pragma unroll
+        for (int m = 0; m < kM; ++m) {
+          const float v = wave_sum(tot[r][m]);
+          tot[r][m] = 0.f;
+          const int n = n0 + r;
+          if (lane == 0 && n < mem.N) {
+            const float b = mem.bias ? (float)mem.bias[n] : 0.f;
+            mem.y[(size_t)m * mem.ldy + n] = (half_t)(__builtin_fmaf(v, 0x1p24f, b));
+          }
+        }
+      }
+    }
+  };
+
+  // Software pipeline: the loads of step s+1 are in flight while step s is computed.  The first
+  // loads go out before the activations are staged, so the staging hides behind HBM latency.
+  Cursor ahead;
+  ahead.blk = ((int)blockIdx.x - wg_begin) * waves_per_block + wave;
+  ahead.it = 0;
+  Prefetch<kRows, kLW> buf0, buf1;
+  issue(ahead, buf0);
 
   stage_activations<kM>(g, U, xs, sig, rs);
   __syncthreads();
 
-  const int iters = (U + kWave - 1) / kWave;
-  for (; task < total_tasks; task += gridDim.x * waves_per_block) {
-    int mi = 0;
-    while (mi + 1 < g.n_members && task >= g.task_end[mi]) ++mi;
-    const MemberDev& mem = g.mem[mi];
-    const int n0 = (task - (mi ? g.task_end[mi - 1] : 0)) * kRows;
-
-    float tot[kRows][kM];
-#pragma unroll
-    for (int r = 0; r < kRows; ++r)
-#pragma unroll
-      for (int m = 0; m < kM; ++m) tot[r][m] = 0.f;
-
-    const int32_t* wrow[kRows];
-    const half_t* srow[kRows];
-    const int32_t* zrow[kRows];
-#pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      const int n = min(n0 + r, mem.N - 1);
-      wrow[r] = mem.qweight + (size_t)n * mem.ldw;
-      srow[r] = mem.scales + (size_t)n * mem.lds;
-      zrow[r] = mem.qzeros + (size_t)n * mem.ldz;
-    }
-
-#pragma unroll 2
-    for (int it = 0; it < iters; ++it) {
-      const int uraw = lane + it * kWave;
-      const bool active = uraw < U;
-      const int u = active ? uraw : U - 1;
-      const int grp = u / upg;
-
-      u32x4 wv[kRows];
-      float sc[kRows];
-      float zp[kRows];
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        wv[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[r]) + u);
-        const float s = (float)srow[r][grp];
-        sc[r] = active ? s : 0.f;
-        zp[r] = (float)nibble((uint32_t)zrow[r][grp >> 3], grp & 7);
-      }
-
-#pragma unroll
-      for (int m = 0; m < kM; ++m) {
-        h8 xq[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xq[j] = xs[((size_t)m * 4 + j) * U + u];
-        const float sg = sig[m * U + u];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-          float accA = 0.f, accB = 0.f;
-          dot_word(wv[r].x, xq[0], accA, accB);
-          dot_word(wv[r].y, xq[1], accA, accB);
-          dot_word(wv[r].z, xq[2], accA, accB);
-          dot_word(wv[r].w, xq[3], accA, accB);
-          float v = __builtin_fmaf(accB, 0.0625f, accA);
-          v = __builtin_fmaf(-zp[r], sg, v);
-          tot[r][m] = __builtin_fmaf(sc[r], v, tot[r][m]);
-        }
-      }
-    }
-
-    // undo the 2^-24 of the subnormal trick, then the rank-r correction: alpha * L[n,:] . r[m,:]
-#pragma unroll
-    for (int r = 0; r < kRows; ++r)
-#pragma unroll
-      for (int m = 0; m < kM; ++m) tot[r][m] *= 0x1p24f;
-
-    if (mem.L != nullptr && g.r != nullptr) {
-#pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        const int n = min(n0 + r, mem.N - 1);
-        const half_t* lrow = mem.L + (size_t)n * g.rank;
-        float corr[kM];
-#pragma unroll
-        for (int m = 0; m < kM; ++m) corr[m] = 0.f;
-        if ((g.rank & 1) == 0) {
-          for (int jj = lane; jj < (g.rank >> 1); jj += kWave) {
-            const h2 lp = reinterpret_cast<const h2*>(lrow)[jj];
-#pragma unroll
-            for (int m = 0; m < kM; ++m)
-              corr[m] = __builtin_amdgcn_fdot2(lp, reinterpret_cast<const h2*>(rs + m * g.rank)[jj], corr[m], false);
-          }
-        } else {
-          for (int jj = lane; jj < g.rank; jj += kWave) {
-            const float lv = (float)lrow[jj];
-#pragma unroll
-            for (int m = 0; m < kM; ++m) corr[m] = __builtin_fmaf(lv, (float)rs[m * g.rank + jj], corr[m]);
-          }
-        }
-#pragma unroll
-        for (int m = 0; m < kM; ++m) tot[r][m] = __builtin_fmaf(g.alpha, corr[m], tot[r][m]);
-      }
-    }
-
-#pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-#pragma unroll
-      for (int m = 0; m < kM; ++m) {
-        const float v = wave_sum(tot[r][m]);
-        const int n = n0 + r;
-        if (lane == 0 && n < mem.N) {
-          const float b = mem.bias ? (float)mem.bias[n] : 0.f;
-          mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
-        }
-      }
-    }
+  while (ahead.blk < total_blocks) {
+    Cursor cur = ahead;
+    advance(ahead);
+    issue(ahead, buf1);
+    compute(cur, buf0);
+    if (ahead.blk >= total_blocks) break;
+    cur = ahead;
+    advance(ahead);
+    issue(ahead, buf0);
+    compute(cur, buf1);
   }
 }
 
@@ -235,51 +298,110 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const GroupDev g) {
 
 // ---- host launchers ---------------------------------------------------------------------
 size_t wave_dot_lds_bytes(int M, int K, int rank, bool has_r) {
-  const size_t U = (size_t)K >> 5;
-  return (size_t)M * K * sizeof(half_t) + (size_t)M * U * sizeof(float) + (has_r ? (size_t)M * rank * sizeof(half_t) : 0);
+  return wave_dot_part_offset(M, K, has_r ? rank : 0);
 }
 
-template <int kM, int kRows>
-static hipError_t launch_wave_dot_t(const GroupDev& g, int grid, size_t lds, hipStream_t stream) {
-  auto kern = gemv_wave_dot_kernel<kM, kRows>;
+static int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : fallback;
+}
+
+// Launch tuning knobs (rows per row block, waves per workgroup, cap on workgroups per CU); the
+// environment overrides exist for tuning runs and are read once.
+struct WaveDotTuning {
+  int rows, waves, max_wg_per_cu;
+};
+static const WaveDotTuning& tuning_override() {
+  static const WaveDotTuning t = {env_int("GLOWQ_GEMV_ROWS", 0), env_int("GLOWQ_GEMV_WAVES", 0),
+                                  env_int("GLOWQ_GEMV_WG_PER_CU", 0)};
+  return t;
+}
+
+template <int kM, int kRows, int kLW>
+static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int max_wg_per_cu, int num_cus, size_t lds,
+                                    hipStream_t stream) {
+  auto kern = gemv_wave_dot_kernel<kM, kRows, kLW>;
+  const int threads = waves * kWave;
   static size_t configured = 48 * 1024;  // largest dynamic LDS size this instantiation was raised to
   if (lds > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     configured = lds;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, stream, g);
+  // resident workgroups per CU for this block size and LDS footprint; the last answer is remembered
+  static int last_threads = 0, last_occ = 0;
+  static size_t last_lds = 0;
+  int occ = last_occ;
+  if (last_occ == 0 || last_threads != threads || last_lds != lds) {
+    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), threads, lds);
+    if (e != hipSuccess) return e;
+    if (occ < 1) occ = 1;
+    last_threads = threads;
+    last_lds = lds;
+    last_occ = occ;
+  }
+  if (max_wg_per_cu > 0 && occ > max_wg_per_cu) occ = max_wg_per_cu;
+  // Split the grid between the members in proportion to their row blocks; when everything does not
+  // fit on the chip at once the waves become persistent and walk an equal number of row blocks.
+  const int resident = num_cus * occ;
+  int wgs_needed = 0;
+  for (int i = 0; i < g.n_members; ++i) {
+    const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
+    wgs_needed += (blocks + waves - 1) / waves;
+  }
+  const int rounds = wgs_needed > resident ? (wgs_needed + resident - 1) / resident : 1;
+  GroupDev gl = g;
+  int grid = 0;
+  for (int i = 0; i < g.n_members; ++i) {
+    const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
+    const int wg_i = ((blocks + waves - 1) / waves + rounds - 1) / rounds;
+    grid += wg_i < 1 ? 1 : wg_i;
+    gl.wg_end[i] = grid;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl, kit);
   return hipGetLastError();
 }
 
-// Rows per wave task for the wave-dot route: enough tasks to put several waves on every SIMD while
-// keeping a few independent rows per wave for load-level parallelism.
-int wave_dot_rows(long total_rows) {
-  if (total_rows >= 16384) return 4;
-  if (total_rows >= 4096) return 2;
-  return 1;
+// The wave-dot route covers K up to 16 slices of 2048 columns and ranks up to 2 dwords per lane
+// and slice wave.
+bool wave_dot_supported(int M, int K, int rank, bool has_r) {
+  const int kit = (K / 32 + kWave - 1) / kWave;
+  if (M < 1 || M > 4 || kit > 16) return false;
+  if (has_r && (rank & 1)) return false;
+  if (has_r && rank > 2 * 128 * kit) return false;
+  return wave_dot_lds_bytes(M, K, rank, has_r) <= 160 * 1024;
 }
 
-hipError_t launch_wave_dot(GroupDev& g, int rows_per_task, int num_cus, hipStream_t stream) {
+int wave_dot_rows(long total_rows) {
+  const int o = tuning_override().rows;
+  if (o == 1 || o == 2 || o == 4) return o;
+  return total_rows >= 8192 ? 4 : 2;
+}
+
+hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStream_t stream) {
+  // register budget: rows x tokens held to 4 accumulators per lane
+  while (rows_per_block * g.M > 4) rows_per_block >>= 1;
   int total = 0;
   for (int i = 0; i < g.n_members; ++i) {
-    total += (g.mem[i].N + rows_per_task - 1) / rows_per_task;
+    total += (g.mem[i].N + rows_per_block - 1) / rows_per_block;
     g.task_end[i] = total;
   }
-  const size_t lds = wave_dot_lds_bytes(g.M, g.K, g.rank, g.r != nullptr);
-  const int blocks_needed = (total + 3) / 4;
-  // resident workgroups per CU: bounded by LDS (160 KB) and by 8 waves per SIMD
-  int per_cu = (int)((160 * 1024) / (lds + 256));
-  if (per_cu > 8) per_cu = 8;
-  if (per_cu < 1) per_cu = 1;
-  int grid = blocks_needed < num_cus * per_cu ? blocks_needed : num_cus * per_cu;
-  if (grid < 1) grid = 1;
-#define GLOWQ_CASE(MM, RR) \
-  if (g.M == MM && rows_per_task == RR) return launch_wave_dot_t<MM, RR>(g, grid, lds, stream);
-  GLOWQ_CASE(1, 1) GLOWQ_CASE(1, 2) GLOWQ_CASE(1, 4)
-  GLOWQ_CASE(2, 1) GLOWQ_CASE(2, 2) GLOWQ_CASE(2, 4)
-  GLOWQ_CASE(3, 1) GLOWQ_CASE(3, 2) GLOWQ_CASE(3, 4)
-  GLOWQ_CASE(4, 1) GLOWQ_CASE(4, 2) GLOWQ_CASE(4, 4)
+  const int kit = (g.K / 32 + kWave - 1) / kWave;
+  const bool has_r = g.r != nullptr;
+  const int lw = has_r ? (g.rank + 128 * kit - 1) / (128 * kit) : 0;
+  const size_t lds = wave_dot_lds_bytes(g.M, g.K, g.rank, has_r);
+  int waves = tuning_override().waves;
+  if (waves < 1 || waves > 16) waves = 8;
+  const int max_wg = tuning_override().max_wg_per_cu;
+#define GLOWQ_CASE(MM, RR, LL) \
+  if (g.M == MM && rows_per_block == RR && lw == LL) \
+    return launch_wave_dot_t<MM, RR, LL>(g, kit, waves, max_wg, num_cus, lds, stream);
+#define GLOWQ_CASES(MM, RR) GLOWQ_CASE(MM, RR, 0) GLOWQ_CASE(MM, RR, 1) GLOWQ_CASE(MM, RR, 2)
+  GLOWQ_CASES(1, 1) GLOWQ_CASES(1, 2) GLOWQ_CASES(1, 4)
+  GLOWQ_CASES(2, 1) GLOWQ_CASES(2, 2)
+  GLOWQ_CASES(3, 1)
+  GLOWQ_CASES(4, 1)
+#undef GLOWQ_CASES
 #undef GLOWQ_CASE
   return hipErrorInvalidValue;
 }
