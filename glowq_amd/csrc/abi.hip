@@ -230,7 +230,7 @@ int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int r
   const half_t* Rp = static_cast<const half_t*>(R);
   half_t* rp = static_cast<half_t*>(r);
   hipError_t e;
-  if (M > 16 && (K & 31) == 0 && (rank & 15) == 0 && aligned16(x) && aligned16(R)) {
+  if (M > 16 && (K & 63) == 0 && aligned16(x) && aligned16(R)) {
     e = launch_shared_proj_mfma(xp, Rp, rp, M, K, rank, num_cus(), static_cast<hipStream_t>(stream));
   } else {
     if ((K & 7) == 0 && (!aligned16(x) || !aligned16(R)))

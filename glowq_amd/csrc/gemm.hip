@@ -1,7 +1,360 @@
-// placeholder: tiled MFMA GEMM route not built yet
+// Prefill GEMM for gfx950: y[M,N] = x[M,K] . deq(W)[N,K]^T (+ alpha * r[M,rank] . L[N,rank]^T) on fp16 MFMA
+// with fp32 accumulation.
+//
+// A workgroup of 4 waves owns a BM x BN output tile (BM = 32*kMT rows, BN = 128*kNT columns); the waves
+// split the columns, each holding kMT x kNT accumulator tiles of 32x32 (v_mfma_f32_32x32x16_f16).
+//   * Activations go global -> registers -> LDS (double-buffered, rows padded to 144 bytes so that the
+//     16-byte fragment reads of 32 consecutive rows fall into distinct banks) and are read back as MFMA
+//     A fragments by all four waves.
+//   * Weights never touch LDS or HBM as fp16: the B operand of the 32x32x16 MFMA wants, per lane, 8
+//     consecutive k of one output column -- exactly one int32 word of 8 int4 codes.  A lane loads 16 bytes
+//     (4 words = the 4 MFMA k-steps of a 64-deep block) and dequantises them in registers to
+//     fp16((code - zero) * scale): the codes are masked into the mantissa of 1024.0 / 64.0, the offset
+//     and zero-point are removed by one exact packed subtraction, and one packed multiply rounds once,
+//     which is bit-identical to the reference's dequantisation.  Every weight is dequantised exactly once.
+//   * The masks deliver the codes of a word in the order (0,4,1,5,2,6,3,7); the activations are permuted
+//     the same way on their way into LDS, so no instruction is spent on reordering weights.
+//   * The rank-r correction is a K-extension that runs first: acc = r . L^T on the same pipeline with an
+//     fp16 B operand, acc *= alpha, then the quantised K loop accumulates on top.
 #include "common.hpp"
+
 namespace glowq {
-bool gemm_supported(const GroupDev&) { return false; }
-hipError_t launch_gemm(GroupDev&, int, hipStream_t) { return hipErrorNotSupported; }
-hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t) { return hipErrorNotSupported; }
+
+constexpr int kBK = 64;              // k depth of one pipeline step
+constexpr int kARow = kBK + 8;       // padded LDS row, in halves (144 bytes)
+
+struct GemmArgs {
+  const half_t* x;        // [M, K]
+  const half_t* r;        // [M, rank] or nullptr
+  const int32_t* qweight; // [N, ldw] (quantised B) or nullptr
+  const half_t* scales;
+  const int32_t* qzeros;
+  const half_t* bmat;     // [N, ldb] fp16 B operand: L for the correction, or the whole B of a plain GEMM
+  const half_t* bias;
+  half_t* y;              // [M, ldy]
+  int M, N, K, group_size, rank;
+  int ldw, lds, ldz, ldb, ldy;
+  float alpha;
+};
+
+__device__ __forceinline__ h8 permute_for_nibble_order(const h8& v) {
+  h8 p;
+  p[0] = v[0]; p[1] = v[4]; p[2] = v[1]; p[3] = v[5];
+  p[4] = v[2]; p[5] = v[6]; p[6] = v[3]; p[7] = v[7];
+  return p;
+}
+
+// 8 codes of one word -> fp16((code - zero) * scale), in nibble order (0,4,1,5,2,6,3,7).
+// zb_lo = -(1024 + zero), zb_hi = -(64 + zero), both exact in fp16.
+__device__ __forceinline__ h8 dequant_word(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2) {
+  const uint32_t hi = w >> 8;
+  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | 0x64006400u);
+  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | 0x54005400u);
+  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | 0x64006400u);
+  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | 0x54005400u);
+  const h2 d0 = (q0 + zb_lo) * s2;
+  const h2 d1 = (q1 + zb_hi) * s2;
+  const h2 d2 = (q2 + zb_lo) * s2;
+  const h2 d3 = (q3 + zb_hi) * s2;
+  h8 out;
+  out[0] = d0[0]; out[1] = d0[1]; out[2] = d1[0]; out[3] = d1[1];
+  out[4] = d2[0]; out[5] = d2[1]; out[6] = d3[0]; out[7] = d3[1];
+  return out;
+}
+
+// kQuant: B is the int4 weight (with the optional correction phase in front); otherwise B is plain fp16.
+template <int kMT, int kNT, bool kQuant>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const int m_blocks) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int BM = 32 * kMT;
+  constexpr int BN = 128 * kNT;
+  half_t* lds_a = reinterpret_cast<half_t*>(smem);  // [2][BM][kARow]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int bm = blockIdx.x % m_blocks;  // row blocks vary fastest: neighbouring workgroups share weight columns
+  const int bn = blockIdx.x / m_blocks;
+  const int m0 = bm * BM;
+  const int ln = lane & 31;  // column inside a 32-wide tile (B operand, accumulator) / row inside a tile (A operand)
+  const int lh = lane >> 5;  // which half of the k range of an MFMA step this lane feeds
+
+  int ncol[kNT];  // weight row (= output column) this lane feeds, clamped for loads
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) ncol[tn] = min(bn * BN + wave * (32 * kNT) + tn * 32 + ln, a.N - 1);
+
+  f16v acc[kMT][kNT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
+
+  // ---- activation tile: global -> registers -> LDS ------------------------------------------------
+  // BM rows x 8 octets (16 bytes); thread t takes octets t, t+256, ...: 8 consecutive threads read the
+  // 128 contiguous bytes of one row.
+  h8 areg[kMT];
+  auto load_a = [&](const half_t* src, int ld, int kb) {
+#pragma unroll
+    for (int i = 0; i < kMT; ++i) {
+      const int q = tid + 256 * i;
+      const int row = min(m0 + (q >> 3), a.M - 1);
+      areg[i] = *reinterpret_cast<const h8*>(src + (size_t)row * ld + kb + (q & 7) * 8);
+    }
+  };
+  auto store_a = [&](int stage, bool permute) {
+#pragma unroll
+    for (int i = 0; i < kMT; ++i) {
+      const int q = tid + 256 * i;
+      half_t* dst = lds_a + ((size_t)stage * BM + (q >> 3)) * kARow + (q & 7) * 8;
+      *reinterpret_cast<h8*>(dst) = permute ? permute_for_nibble_order(areg[i]) : areg[i];
+    }
+  };
+  // A fragment of MFMA step t for row tile tm: octet (4*lh + t) of row tm*32 + ln
+  auto read_a = [&](int stage, int tm, int t) {
+    const half_t* src = lds_a + ((size_t)stage * BM + tm * 32 + ln) * kARow + (4 * lh + t) * 8;
+    return *reinterpret_cast<const h8*>(src);
+  };
+  auto mma_step = [&](int stage, const h8 (&bfrag)[kNT][4]) {
+    constexpr int kChunk = kMT < 4 ? kMT : 4;  // row tiles whose A fragments are live at once
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int c = 0; c < kMT; c += kChunk) {
+        h8 af[kChunk];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) af[i] = read_a(stage, c + i, t);
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < kChunk; ++i)
+            acc[c + i][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bfrag[tn][t], acc[c + i][tn], 0, 0, 0);
+      }
+    }
+  };
+
+  int stage = 0;
+
+  // ---- phase 1: the correction as a K-extension, acc = r . L^T, fp16 B operand ----------------------
+  if (kQuant && a.r != nullptr) {
+    const int steps = a.rank / kBK;
+    load_a(a.r, a.rank, 0);
+    store_a(stage, false);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ++ks) {
+      h8 bfrag[kNT][4];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + ks * kBK + 32 * lh + 8 * t);
+      if (ks + 1 < steps) load_a(a.r, a.rank, (ks + 1) * kBK);
+      mma_step(stage, bfrag);
+      if (ks + 1 < steps) store_a(stage ^ 1, false);
+      __syncthreads();
+      stage ^= 1;
+    }
+    if (a.alpha != 1.0f) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= a.alpha;
+    }
+  }
+
+  // ---- phase 2: the main K loop ---------------------------------------------------------------------
+  const int steps = a.K / kBK;
+  const int gs_shift = __builtin_ctz(a.group_size);  // group sizes on this route are powers of two
+  if constexpr (kQuant) {
+    // quantised B: per step and column tile one 16-byte load of codes, one scale, one zero-point word
+    u32x4 wq[kNT], wq_next[kNT];
+    half_t sc[kNT], sc_next[kNT];
+    uint32_t zw[kNT], zw_next[kNT];
+    auto load_w = [&](int kb, u32x4 (&w)[kNT], half_t (&s)[kNT], uint32_t (&z)[kNT]) {
+      const int grp = (kb + 32 * lh) >> gs_shift;
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        w[tn] = *reinterpret_cast<const u32x4*>(a.qweight + (size_t)ncol[tn] * a.ldw + (kb >> 3) + 4 * lh);
+        s[tn] = a.scales[(size_t)ncol[tn] * a.lds + grp];
+        z[tn] = (uint32_t)a.qzeros[(size_t)ncol[tn] * a.ldz + (grp >> 3)];
+      }
+    };
+    load_a(a.x, a.K, 0);
+    load_w(0, wq, sc, zw);
+    store_a(stage, true);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ++ks) {
+      const int kb = ks * kBK;
+      if (ks + 1 < steps) {
+        load_a(a.x, a.K, kb + kBK);
+        load_w(kb + kBK, wq_next, sc_next, zw_next);
+      }
+      h8 bfrag[kNT][4];
+      const int grp = (kb + 32 * lh) >> gs_shift;
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        const half_t z = (half_t)(float)nibble(zw[tn], grp & 7);
+        const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
+        const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh}, s2 = {sc[tn], sc[tn]};
+        bfrag[tn][0] = dequant_word(wq[tn].x, zb_lo, zb_hi, s2);
+        bfrag[tn][1] = dequant_word(wq[tn].y, zb_lo, zb_hi, s2);
+        bfrag[tn][2] = dequant_word(wq[tn].z, zb_lo, zb_hi, s2);
+        bfrag[tn][3] = dequant_word(wq[tn].w, zb_lo, zb_hi, s2);
+      }
+      mma_step(stage, bfrag);
+      if (ks + 1 < steps) {
+        store_a(stage ^ 1, true);
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) {
+          wq[tn] = wq_next[tn];
+          sc[tn] = sc_next[tn];
+          zw[tn] = zw_next[tn];
+        }
+      }
+      __syncthreads();
+      stage ^= 1;
+    }
+  } else {
+    // plain fp16 B (the shared projection r = x R^T for many rows)
+    load_a(a.x, a.K, 0);
+    store_a(stage, false);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ++ks) {
+      h8 bfrag[kNT][4];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + ks * kBK + 32 * lh + 8 * t);
+      if (ks + 1 < steps) load_a(a.x, a.K, (ks + 1) * kBK);
+      mma_step(stage, bfrag);
+      if (ks + 1 < steps) store_a(stage ^ 1, false);
+      __syncthreads();
+      stage ^= 1;
+    }
+  }
+
+  // ---- epilogue: accumulator register i of a 32x32 tile is row 8*(i/4) + 4*lh + i%4, column ln ---------
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) {
+    const int n = bn * BN + wave * (32 * kNT) + tn * 32 + ln;
+    if (n >= a.N) continue;
+    const float b = a.bias ? (float)a.bias[n] : 0.f;
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + tm * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+        if (m < a.M) a.y[(size_t)m * a.ldy + n] = (half_t)(acc[tm][tn][i] + b);
+      }
+    }
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+template <int kMT, int kNT, bool kQuant>
+static hipError_t launch_gemm_t(const GemmArgs& a, hipStream_t stream) {
+  constexpr int BM = 32 * kMT, BN = 128 * kNT;
+  auto kern = gemm_mfma_kernel<kMT, kNT, kQuant>;
+  const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t);
+  static bool configured = false;
+  if (!configured && lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  const int m_blocks = (a.M + BM - 1) / BM;
+  const int n_blocks = (a.N + BN - 1) / BN;
+  hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks), dim3(256), lds, stream, a, m_blocks);
+  return hipGetLastError();
+}
+
+static hipError_t launch_gemm_args(const GemmArgs& a, hipStream_t stream) {
+  // row tiles per workgroup: the largest that M fills; column tiles: 2 per wave unless N is small
+  const int nt = a.N > 128 ? 2 : 1;
+  int mt = a.M > 128 ? 8 : (a.M > 64 ? 4 : (a.M > 32 ? 2 : 1));
+#define GLOWQ_GEMM_CASE(MT, NT) \
+  if (mt == MT && nt == NT) return launch_gemm_t<MT, NT, true>(a, stream);
+  GLOWQ_GEMM_CASE(8, 2) GLOWQ_GEMM_CASE(4, 2) GLOWQ_GEMM_CASE(2, 2) GLOWQ_GEMM_CASE(1, 2)
+  GLOWQ_GEMM_CASE(8, 1) GLOWQ_GEMM_CASE(4, 1) GLOWQ_GEMM_CASE(2, 1) GLOWQ_GEMM_CASE(1, 1)
+#undef GLOWQ_GEMM_CASE
+  return hipErrorInvalidValue;
+}
+
+// The MFMA route needs 64-deep k blocks that stay inside one quantisation group per 32-column half and
+// 16-byte aligned rows everywhere.
+bool gemm_supported(const GroupDev& g) {
+  if ((g.K % kBK) != 0 || (g.group_size % 32) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
+  if (g.r != nullptr && (g.rank % kBK) != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
+  if (g.r != nullptr && (reinterpret_cast<uintptr_t>(g.r) & 15u) != 0) return false;
+  for (int i = 0; i < g.n_members; ++i) {
+    const MemberDev& m = g.mem[i];
+    if ((reinterpret_cast<uintptr_t>(m.qweight) & 15u) != 0 || (m.ldw & 3) != 0) return false;
+    if (m.L != nullptr && (reinterpret_cast<uintptr_t>(m.L) & 15u) != 0) return false;
+  }
+  return true;
+}
+
+hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
+  (void)num_cus;
+  for (int i = 0; i < g.n_members; ++i) {
+    const MemberDev& m = g.mem[i];
+    GemmArgs a;
+    a.x = g.x;
+    a.r = (m.L != nullptr) ? g.r : nullptr;
+    a.qweight = m.qweight;
+    a.scales = m.scales;
+    a.qzeros = m.qzeros;
+    a.bmat = m.L;
+    a.bias = m.bias;
+    a.y = m.y;
+    a.M = g.M;
+    a.N = m.N;
+    a.K = g.K;
+    a.group_size = g.group_size;
+    a.rank = g.rank;
+    a.ldw = m.ldw;
+    a.lds = m.lds;
+    a.ldz = m.ldz;
+    a.ldb = g.rank;
+    a.ldy = m.ldy;
+    a.alpha = g.alpha;
+    hipError_t e = launch_gemm_args(a, stream);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+// r[M, rank] = fp16(x[M, K] . R[rank, K]^T) on the same kernel with an fp16 B operand.
+hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int num_cus,
+                                   hipStream_t stream) {
+  (void)num_cus;
+  if ((K % kBK) != 0) return hipErrorInvalidValue;
+  GemmArgs a;
+  a.x = x;
+  a.r = nullptr;
+  a.qweight = nullptr;
+  a.scales = nullptr;
+  a.qzeros = nullptr;
+  a.bmat = R;
+  a.bias = nullptr;
+  a.y = r;
+  a.M = M;
+  a.N = rank;
+  a.K = K;
+  a.group_size = 128;
+  a.rank = 0;
+  a.ldw = a.lds = a.ldz = 0;
+  a.ldb = K;
+  a.ldy = rank;
+  a.alpha = 1.0f;
+  // small row tiles: N is tiny here, the parallelism has to come from M
+  if (rank > 128) return launch_gemm_t<2, 2, false>(a, stream);
+  return launch_gemm_t<2, 1, false>(a, stream);
+}
+
 }  // namespace glowq

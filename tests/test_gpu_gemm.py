@@ -1,0 +1,74 @@
+"""GPU parity of the MFMA GEMM route (large M) and of the shared projection, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import glowq_oracle as oracle
+from helpers import assert_close, dev, make_group
+
+pytestmark = pytest.mark.gpu
+
+
+def test_identity_input_reproduces_dequantised_weight_exactly(ext):
+    """x = I_K: y[m, n] = fp16((code - zero) * scale) of weight element [n, m], so the in-kernel
+    dequantisation (every nibble position, zero-point and scale path) is checked bit for bit."""
+    K, N, gs = 256, 320, 128
+    _, (m,), _ = make_group(21, 1, K, [N], 0, group_size=gs)
+    x = np.eye(K, dtype=np.float16)
+    y = ext.w4a16_gemm_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs, 1).cpu().numpy()
+    want = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], K, gs).T
+    np.testing.assert_array_equal(y.view(np.uint16), np.ascontiguousarray(want).view(np.uint16))
+
+
+@pytest.mark.parametrize("M,K,N,gs", [
+    (256, 512, 256, 128), (200, 1024, 300, 128), (33, 256, 64, 64), (2048, 1024, 512, 128), (129, 2048, 1000, 128),
+    (64, 3584, 512, 128), (17, 512, 1024, 32),
+])
+def test_gemm_matches_oracle(ext, M, K, N, gs):
+    print(f"case M={M} K={K} N={N} gs={gs}", flush=True)
+    x, (m,), _ = make_group(31 + M + N, M, K, [N], 0, group_size=gs)
+    y = ext.w4a16_gemm_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs, 1)
+    torch.cuda.synchronize()
+    # yardstick: the reference's GEMM semantics (weights rounded to fp16 once) in float64
+    w = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], K, gs).astype(np.float64)
+    want = x.astype(np.float64) @ w.T
+    assert_close(y.cpu().numpy(), want, f"gemm M={M} K={K} N={N}")
+
+
+def test_gemm_route_falls_back_on_odd_shapes(ext):
+    M, K, N, gs = 70, 200, 37, 40
+    x, (m,), _ = make_group(77, M, K, [N], 0, group_size=gs)
+    y = ext.w4a16_gemm_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs, 1)
+    want = oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], gs)
+    assert_close(y.cpu().numpy(), want, "generic from gemm entry")
+
+
+@pytest.mark.parametrize("M,K,rank", [(1, 2048, 64), (3, 4096, 128), (8, 1024, 256), (300, 1024, 128), (2048, 512, 64),
+                                      (70, 3584, 256), (5, 200, 24)])
+def test_shared_proj(ext, M, K, rank):
+    g = torch.Generator().manual_seed(M + K + rank)
+    x = torch.randn(M, K, generator=g).half().numpy()
+    R = (torch.randn(rank, K, generator=g) * K ** -0.5).half().numpy()
+    r = ext.shared_proj(dev(x), dev(R)).cpu().numpy()
+    want = x.astype(np.float64) @ R.astype(np.float64).T
+    assert_close(r, want, f"shared_proj M={M}")
+
+
+@pytest.mark.parametrize("M,K,Ns,rank,alpha", [(256, 1024, [256, 128], 128, 1.0), (100, 512, [300], 64, 0.5),
+                                               (40, 1024, [128, 128, 64], 128, 1.0), (16, 2048, [256], 64, 1.0)])
+def test_group_forward_large_m(ext, M, K, Ns, rank, alpha):
+    """Rows above the GEMV capacity: MFMA route with the correction as a K-extension."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(57 + M, M, K, Ns, rank, with_bias=True)
+    r = ext.shared_proj(dev(x), dev(R))
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]),
+            "L": dev(m["L"]) if i != 1 else None, "bias": dev(m["bias"])} for i, m in enumerate(members)]
+    outs = ext.group_forward(dev(x), r, mem, 128, alpha)
+    torch.cuda.synchronize()
+    for i, (m, y) in enumerate(zip(members, outs)):
+        if i == 1:
+            want = oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)
+        else:
+            want = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha)
+        want = want + m["bias"].astype(np.float64)[None, :]
+        assert_close(y.cpu().numpy(), want, f"group large M member {i}")
