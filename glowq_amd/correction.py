@@ -36,7 +36,7 @@ class MiniGroupCache:
     """One-slot, use-counted cache of the shared projection r (step3_eval_dataset.py:417-444), extended
     with the member outputs of the fused group launch."""
 
-    __slots__ = ("r", "valid", "uses_left", "members", "outputs", "x_key")
+    __slots__ = ("r", "valid", "uses_left", "members", "outputs", "x_key", "x_hold")
 
     def __init__(self):
         self.r: Optional[torch.Tensor] = None
@@ -45,6 +45,7 @@ class MiniGroupCache:
         self.members: List["AddSVDCorrection"] = []
         self.outputs: Dict[int, torch.Tensor] = {}
         self.x_key = None
+        self.x_hold = None  # the leader's input, kept alive so that its address cannot be reused meanwhile
 
     def set(self, r: torch.Tensor, uses: int):
         self.r = r
@@ -59,6 +60,7 @@ class MiniGroupCache:
                 self.valid = False
                 self.r = None
                 self.x_key = None
+                self.x_hold = None
             return out, True
         return None, False
 
@@ -68,6 +70,7 @@ class MiniGroupCache:
         self.uses_left = 0
         self.outputs = {}
         self.x_key = None
+        self.x_hold = None
 
     # -- extensions ---------------------------------------------------------------------------------
     def register(self, wrapper: "AddSVDCorrection") -> None:
@@ -173,6 +176,7 @@ class AddSVDCorrection(nn.Module):
             cache.clear()
             cache.set(r, _LEADER_USES[self.role])
             cache.x_key = _x_key(x2d)
+            cache.x_hold = x2d
             for w, y in zip(group[1:], outs[1:]):
                 cache.outputs[id(w)] = y
             return self._finish(outs[0], lead_shape)

@@ -1,0 +1,224 @@
+"""Pins the CPU oracle: golden vectors written by the reference's own functions, exhaustive brute
+force on the packing, and mathematical invariants chosen so that a dropped term, a wrong sign or a
+transposed operand fails.  CPU only."""
+import numpy as np
+import pytest
+import torch
+
+import c_oracle
+import glowq_oracle as oracle
+import torch_cpu_path as tp
+from helpers import make_group
+
+
+# ---------------------------------------------------------------- golden vectors (tests/golden)
+def test_pack_unpack_golden(golden):
+    np.testing.assert_array_equal(oracle.pack_int4_to_int32(golden["pack_codes"]), golden["pack_words"])
+    np.testing.assert_array_equal(oracle.unpack_int4_i32(golden["pack_words"], 50), golden["unpack_vals_50"])
+    np.testing.assert_array_equal(oracle.unpack_int4_i32(golden["pack_words"], 56), golden["unpack_vals_56"])
+
+
+@pytest.mark.parametrize("name", list("abcde"))
+def test_quantizer_golden_bit_exact(golden, name):
+    gs, kp = (int(v) for v in golden[f"q_{name}_gs"])
+    qw, qz, sc, kp2 = oracle.quantize_per_group_w4(golden[f"q_{name}_w"], gs)
+    assert kp2 == kp
+    np.testing.assert_array_equal(qw, golden[f"q_{name}_qweight"])
+    np.testing.assert_array_equal(qz, golden[f"q_{name}_qzeros"])
+    np.testing.assert_array_equal(sc.view(np.uint16), golden[f"q_{name}_scales"].view(np.uint16))
+
+
+@pytest.mark.parametrize("name", ["m1", "m2"])
+def test_dequant_and_forward_golden(golden, name):
+    gs = int(golden[f"{name}_gs"][0])
+    x, w = golden[f"{name}_x"], golden[f"{name}_w"]
+    K = x.shape[1]
+    qw, qz, sc, _ = oracle.quantize_per_group_w4(w, gs)
+    np.testing.assert_array_equal(qw, golden[f"{name}_qweight"])
+    np.testing.assert_array_equal(qz, golden[f"{name}_qzeros"])
+    d = oracle.dequant(qw, qz, sc, K, gs)
+    np.testing.assert_array_equal(d.view(np.uint16), golden[f"{name}_deq"].view(np.uint16))
+    np.testing.assert_array_equal(c_oracle.dequant(qw, sc, qz, K, gs).view(np.uint16), golden[f"{name}_deq"].view(np.uint16))
+    y = oracle.gemm_ref(x, qw, qz, sc, gs).astype(np.float32)
+    if name == "m2":
+        y = (y + golden["m2_bias"].astype(np.float32)).astype(np.float16).astype(np.float32)
+    # the reference's CPU matmul accumulates in its own order: one fp16 ulp at |y| < 2
+    assert np.abs(y - golden[f"{name}_y"].astype(np.float32)).max() <= 2e-3
+    assert list(golden[f"{name}_state_keys"]) == sorted(
+        ["qweight_i32", "qzeros_i32", "scales_f16"] + (["bias"] if name == "m2" else []))
+
+
+# ---------------------------------------------------------------- brute force / closed forms
+def test_pack_every_value_every_position():
+    for pos in range(8):
+        for val in range(16):
+            codes = np.zeros((1, 8), dtype=np.uint8)
+            codes[0, pos] = val
+            word = oracle.pack_int4_to_int32(codes)
+            want = (val << (4 * pos)) & 0xFFFFFFFF
+            want = want - (1 << 32) if want >= (1 << 31) else want
+            assert int(word[0]) == want
+            assert int(oracle.unpack_int4_i32(word.reshape(1, 1), 8)[0, pos]) == val
+            # the device kernels' form of the same lookup: (word >> 4*(k&7)) & 0xF
+            assert ((int(word[0]) & 0xFFFFFFFF) >> (4 * pos)) & 0xF == val
+
+
+def test_pack_unpack_round_trip_random():
+    rng = np.random.default_rng(0)
+    codes = rng.integers(0, 16, size=(13, 9, 8), dtype=np.uint8)
+    words = oracle.pack_int4_to_int32(codes)
+    np.testing.assert_array_equal(oracle.unpack_int4_i32(words, 72), codes.reshape(13, 72))
+    out = np.empty((13, 72), dtype=np.uint8)
+    lib = c_oracle.load()
+    lib.oracle_unpack_u4(words.ctypes.data, 13, 9, 72, out.ctypes.data)
+    np.testing.assert_array_equal(out, codes.reshape(13, 72))
+
+
+def test_dequant_all_code_zero_pairs():
+    """(code - zero) * scale for all 16 x 16 pairs and a sweep of scales, against exact arithmetic."""
+    scales = np.array([2.0 ** -10, 0.00731, 0.0125, 1.0, 3.0003, 1e-4], dtype=np.float16)
+    for s in scales:
+        for z in range(16):
+            codes = np.arange(16, dtype=np.uint8).repeat(8).reshape(1, 128)  # every code, every nibble slot
+            qw = oracle.pack_int4_to_int32(codes.reshape(1, 16, 8))
+            qz = oracle.pack_int4_to_int32(np.array([[[z, 8, 8, 8, 8, 8, 8, 8]]], dtype=np.uint8))
+            sc = np.array([[s]], dtype=np.float16)
+            d = oracle.dequant(qw, qz, sc, 128, 128)
+            want = ((codes.astype(np.float64) - z) * float(s)).astype(np.float16)  # exact product, one rounding
+            np.testing.assert_array_equal(d.view(np.uint16), want.view(np.uint16))
+
+
+def test_quantizer_invariants():
+    x, (m,), _ = make_group(0, 1, 512, [64], 0)
+    w = m["w"].astype(np.float32).reshape(64, 4, 128)
+    codes, zeros, sc, gid = oracle.codes_and_params(m["qweight"], m["qzeros"], m["scales"], 512, 128)
+    assert codes.max() <= 15 and zeros.max() <= 15
+    s = sc.astype(np.float32)
+    # scale is (max - min) / 15 up to fp16 rounding; the extremes map to the ends of the code range
+    np.testing.assert_allclose(s, (w.max(-1) - w.min(-1)) / 15.0, rtol=2e-3)
+    c = codes.reshape(64, 4, 128)
+    assert np.all(np.take_along_axis(c, w.argmin(-1)[..., None], -1) <= 1)
+    assert np.all(np.take_along_axis(c, w.argmax(-1)[..., None], -1) >= 14)
+    # reconstruction error of an unclipped element is at most half a step (plus fp16 rounding slack)
+    deq = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], 512, 128).astype(np.float32).reshape(64, 4, 128)
+    unclipped = (c > 0) & (c < 15)
+    assert np.all(np.abs(deq - w)[unclipped] <= 0.5 * s[..., None].repeat(128, -1)[unclipped] * 1.02 + 1e-4)
+    # unused zero-point nibbles hold code 8 (4 groups -> nibbles 4..7 of the single word)
+    znib = oracle.unpack_int4_i32(m["qzeros"], 8)
+    assert np.all(znib[:, 4:] == 8)
+
+
+def test_quantizer_recovers_exact_grid():
+    """A group whose values are exactly s * (c - z) for integer codes c reproduces those codes."""
+    s, z = np.float16(0.015625), 6  # power-of-two step: every product is exact in fp16
+    rng = np.random.default_rng(3)
+    c = rng.integers(0, 16, size=(4, 128)).astype(np.int64)
+    c[:, 0], c[:, 1] = 0, 15
+    w = ((c - z) * float(s)).astype(np.float16)
+    qw, qz, sc, _ = oracle.quantize_per_group_w4(w, 128)
+    np.testing.assert_array_equal(oracle.unpack_int4_i32(qw, 128), c.astype(np.uint8))
+    assert np.all(oracle.unpack_int4_i32(qz, 1) == z) and np.all(sc == s)
+
+
+def test_quantizer_pads_k_to_group_multiple():
+    w = (np.random.default_rng(1).standard_normal((3, 200)) * 0.02).astype(np.float16)
+    qw, qz, sc, kp = oracle.quantize_per_group_w4(w, 64)
+    assert kp == 256 and qw.shape == (3, 32) and sc.shape == (3, 4) and qz.shape == (3, 1)
+    codes, zeros, _, _ = oracle.codes_and_params(qw, qz, sc, 256, 64)
+    # padded columns hold value 0 and quantise to the group's zero-point (or its clipped neighbour)
+    np.testing.assert_array_equal(codes[:, 200:], np.repeat(zeros[:, 3:4], 56, axis=1))
+
+
+# ---------------------------------------------------------------- linear / correction semantics
+def test_gemv_reduces_to_library_matmul():
+    x, (m,), _ = make_group(5, 3, 384, [40], 0)
+    deq = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], 384, 128).astype(np.float64)
+    exact = oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)
+    # the GEMV semantics never round the weight, the GEMM semantics round it once to fp16
+    assert np.abs(exact - x.astype(np.float64) @ deq.T).max() < 5e-3
+    np.testing.assert_array_equal(oracle.gemm_ref(x, m["qweight"], m["qzeros"], m["scales"], 128),
+                                  (x.astype(np.float64) @ deq.T).astype(np.float16))
+    for fn in (c_oracle.gemv_f32acc, c_oracle.gemm_deq_f32acc):
+        y = fn(x, m["qweight"], m["scales"], m["qzeros"], 128).astype(np.float64)
+        assert np.all(np.abs(y - exact) <= 1e-2 + 1e-3 * np.abs(exact))
+    np.testing.assert_allclose(c_oracle.linear_f64(x, m["qweight"], m["scales"], m["qzeros"], 128), exact, rtol=1e-12, atol=1e-12)
+
+
+def test_one_hot_input_selects_one_dequantised_column():
+    _, (m,), _ = make_group(9, 1, 256, [16], 0)
+    deq = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], 256, 128)
+    for k in (0, 1, 7, 8, 127, 128, 255):
+        x = np.zeros((1, 256), dtype=np.float16)
+        x[0, k] = 1
+        np.testing.assert_array_equal(oracle.gemv_ref(x, m["qweight"], m["qzeros"], m["scales"], 128)[0], deq[:, k])
+        np.testing.assert_array_equal(c_oracle.gemv_f32acc(x, m["qweight"], m["scales"], m["qzeros"], 128)[0], deq[:, k])
+
+
+def test_correction_closed_form_and_linearity():
+    x, members, R = make_group(12, 2, 256, [24, 8], 32)
+    m = members[0]
+    z = oracle.gemv_ref(x, m["qweight"], m["qzeros"], m["scales"], 128)
+    r = oracle.shared_proj(x, R)
+    # alpha = 0 leaves z untouched; the correction is linear in alpha up to the fp16 roundings
+    np.testing.assert_array_equal(oracle.correction(z, r, m["L"], 0.0), z)
+    full = x.astype(np.float64) @ R.astype(np.float64).T @ m["L"].astype(np.float64).T
+    for alpha in (1.0, 0.5, -2.0):
+        got = oracle.correction(z, r, m["L"], alpha).astype(np.float64)
+        assert np.abs(got - (z.astype(np.float64) + alpha * full)).max() < 4e-3
+        exact = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha)
+        assert np.abs(got - exact).max() < 6e-3
+    # transposing either factor would not even have the right shape; a zero L gives z back
+    np.testing.assert_array_equal(oracle.correction(z, r, np.zeros_like(m["L"]), 1.0), z)
+    # C restatement agrees
+    np.testing.assert_array_equal(c_oracle.shared_proj(x, R), r)
+    assert np.abs(c_oracle.add_correction(z, r, m["L"], 1.0).astype(np.float32) - oracle.correction(z, r, m["L"], 1.0).astype(np.float32)).max() <= 1e-3
+
+
+def test_group_equals_independent_solo_results():
+    x, members, R = make_group(14, 1, 256, [16, 8, 8], 16)
+    outs = oracle.group_forward(x, members, R, 1.0)
+    for m, y in zip(members, outs):
+        solo = oracle.group_forward(x, [m], R, 1.0)[0]
+        np.testing.assert_array_equal(y, solo)
+    members[1]["L"] = None  # an unselected member is exactly the plain linear
+    outs = oracle.group_forward(x, members, R, 1.0)
+    np.testing.assert_array_equal(outs[1], oracle.gemv_ref(x, members[1]["qweight"], members[1]["qzeros"], members[1]["scales"], 128))
+
+
+def test_torch_cpu_path_matches_numpy_oracle():
+    x, members, R = make_group(15, 2, 256, [24, 8], 32)
+    tm = [{"qweight": torch.from_numpy(m["qweight"]), "qzeros": torch.from_numpy(m["qzeros"]),
+           "scales": torch.from_numpy(m["scales"]), "L": torch.from_numpy(m["L"]), "group_size": 128} for m in members]
+    outs = tp.corrected_group(torch.from_numpy(x), tm, torch.from_numpy(R), 1.0, chunk=16)
+    for m, y in zip(members, outs):
+        want = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0)
+        assert np.abs(y.numpy().astype(np.float64) - want).max() < 8e-3
+    gid = torch.arange(256) // 128
+    d = tp.dequant_chunk(tm[0]["qweight"], tm[0]["qzeros"], tm[0]["scales"], gid, 256, 2, 0, 24).numpy()
+    np.testing.assert_array_equal(d.view(np.uint16), oracle.dequant(members[0]["qweight"], members[0]["qzeros"], members[0]["scales"], 256, 128).view(np.uint16))
+
+
+def test_cache_state_machine():
+    c = oracle.MiniGroupCacheModel()
+    assert c.consume() == (None, False)
+    c.set("r", 2)
+    assert c.consume() == ("r", True) and c.valid
+    assert c.consume() == ("r", True) and not c.valid and c.r is None
+    assert c.consume() == (None, False)
+    c.set("s", 1)
+    c.clear()
+    assert c.consume() == (None, False)
+
+
+def test_fp16_conversions_of_c_oracle():
+    lib = c_oracle.load()
+    rng = np.random.default_rng(0)
+    bits = np.concatenate([rng.integers(0, 1 << 16, 4000), np.array([0, 1, 0x3FF, 0x400, 0x7BFF, 0x8000, 0x8001, 0xFBFF])]).astype(np.uint16)
+    for b in bits:
+        h = np.array([b], dtype=np.uint16).view(np.float16)[0]
+        if np.isnan(h) or np.isinf(h):
+            continue
+        assert lib.oracle_h2f(int(b)) == float(h)
+    vals = np.concatenate([rng.standard_normal(4000) * 10 ** rng.uniform(-8, 5, 4000), [65519.9, 65520.0, 2.0 ** -25, 2.0 ** -25 * 1.0001, 0.0]]).astype(np.float32)
+    for v in vals:
+        assert lib.oracle_f2h(float(v)) == int(np.array([v], dtype=np.float32).astype(np.float16).view(np.uint16)[0])
