@@ -69,7 +69,8 @@ bool fast_layout(const GroupDev& g) {
     if (!aligned16(m.qweight) || (m.ldw & 3) != 0) return false;
     if (m.L && !aligned4(m.L)) return false;
   }
-  if (g.r && (g.rank & 1) != 0) return false;  // the L rows are read two halves at a time
+  if ((g.r || g.R) && (g.rank & 1) != 0) return false;  // the L rows are read two halves at a time
+  if (g.R && (!aligned16(g.R) || (g.K & 7) != 0)) return false;
   return true;
 }
 
@@ -113,7 +114,7 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
-  if (g.M <= kWaveDotMaxM && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr))
+  if (g.M <= kWaveDotMaxM && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
     return kRouteWaveDot;
   if (skinny_supported(g)) return kRouteSkinny;
   if (gemm_supported(g)) return kRouteGemm;
@@ -125,6 +126,17 @@ int pick_route(const GroupDev& g, int force) {
 int run_group(GroupDev g, int route, hipStream_t stream) {
   const int cus = num_cus();
   hipError_t e = hipSuccess;
+  if (g.R != nullptr) {
+    // r = x R^T goes ahead as a launch of its own.  (Folding it into the group kernel was measured: the
+    // R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch costs.)
+    if (g.M > 16 && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
+      e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream);
+    else
+      e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
+    if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
+    g.r = g.r_out;
+    g.R = nullptr;
+  }
   if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
   } else if (route == kRouteSkinny) {
@@ -270,6 +282,37 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
   g.M = M;
   g.K = K;
   g.group_size = group_size;
+  return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
+}
+
+int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                    int n_members, int M, int K, int group_size, int rank, float alpha, void* stream) {
+  int rc = check_common(x, M, K, group_size);
+  if (rc) return rc;
+  if (members == nullptr || n_members < 1 || n_members > GLOWQ_MAX_MEMBERS)
+    return fail(GLOWQ_EINVAL, "group_forward_fused: n_members must be 1..%d", GLOWQ_MAX_MEMBERS);
+  if (R == nullptr || r_out == nullptr || rank <= 0)
+    return fail(GLOWQ_EINVAL, "group_forward_fused: R, r_out and a positive rank are required");
+  if ((K & 7) == 0 && (!aligned16(x) || !aligned16(R)))
+    return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused: x and R must be 16-byte aligned");
+  GroupDev g;
+  memset(&g, 0, sizeof(g));
+  for (int i = 0; i < n_members; ++i) {
+    rc = check_member(members[i], K, group_size, i);
+    if (rc) return rc;
+    to_dev(members[i], g.mem[i]);
+  }
+  g.x = static_cast<const half_t*>(x);
+  g.R = static_cast<const half_t*>(R);
+  g.r_out = static_cast<half_t*>(r_out);
+  g.rank = rank;
+  g.alpha = alpha;
+  g.n_members = n_members;
+  g.M = M;
+  g.K = K;
+  g.group_size = group_size;
+  if (alpha == 0.0f)
+    for (int i = 0; i < n_members; ++i) g.mem[i].L = nullptr;  // r is still produced: callers cache it
   return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
 }
 

@@ -33,6 +33,9 @@ struct MemberDev {
 struct GroupDev {
   const half_t* x;  // [M, K]
   const half_t* r;  // [M, rank] or nullptr
+  // set by the entry point that also produces r: the projection r_out = x R^T is launched ahead of the group
+  const half_t* R;  // [rank, K] or nullptr
+  half_t* r_out;
   MemberDev mem[GLOWQ_MAX_MEMBERS];
   int task_end[GLOWQ_MAX_MEMBERS];  // exclusive prefix of per-member task counts
   int wg_end[GLOWQ_MAX_MEMBERS];    // exclusive prefix of the workgroups assigned to each member

@@ -58,18 +58,34 @@ __global__ __launch_bounds__(256) void shared_proj_kernel(const half_t* __restri
   for (int m = 0; m < kM; ++m) acc[m] = 0.f;
   const half_t* Rrow = R + (size_t)j * K;
   if ((K & 7) == 0) {
+    // batches of 4 pieces per thread: all loads of a batch are issued before the first is used, so a long
+    // row costs one memory latency per 8192 columns, not one per 2048
     const int words = K >> 3;
-    for (int w = threadIdx.x; w < words; w += blockDim.x) {
-      const h8 rv = reinterpret_cast<const h8*>(Rrow)[w];
+    constexpr int kBatch = 4;
+    for (int w0 = threadIdx.x; w0 < words; w0 += kBatch * blockDim.x) {
+      h8 rv[kBatch], xv[kM][kBatch];
+      float live[kBatch];
 #pragma unroll
-      for (int m = 0; m < kM; ++m) {
-        const int mm = min(m0 + m, M - 1);
-        const h8 xv = reinterpret_cast<const h8*>(x + (size_t)mm * K)[w];
+      for (int b = 0; b < kBatch; ++b) {
+        const int w = w0 + b * blockDim.x;
+        live[b] = w < words ? 1.f : 0.f;
+        const int wc = min(w, words - 1);
+        rv[b] = reinterpret_cast<const h8*>(Rrow)[wc];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const h2 a = {rv[2 * i], rv[2 * i + 1]};
-          const h2 b = {xv[2 * i], xv[2 * i + 1]};
-          acc[m] = __builtin_amdgcn_fdot2(a, b, acc[m], false);
+        for (int m = 0; m < kM; ++m) xv[m][b] = reinterpret_cast<const h8*>(x + (size_t)min(m0 + m, M - 1) * K)[wc];
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+#pragma unroll
+        for (int m = 0; m < kM; ++m) {
+          float d = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const h2 a = {rv[b][2 * i], rv[b][2 * i + 1]};
+            const h2 c = {xv[m][b][2 * i], xv[m][b][2 * i + 1]};
+            d = __builtin_amdgcn_fdot2(a, c, d, false);
+          }
+          acc[m] = __builtin_fmaf(live[b], d, acc[m]);
         }
       }
     }

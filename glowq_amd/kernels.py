@@ -48,6 +48,7 @@ _SIGNATURES = {
     "glowq_unpack_int4": (_I, [_P, _P, _I, _I, _I, _P]),
     "glowq_shared_proj": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
 }
 
@@ -177,9 +178,11 @@ class W4A16Extension:
         return out
 
     def group_forward(self, x, r, members: Sequence[dict], group_size: int, alpha: float,
-                      outs: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
+                      outs: Optional[List[torch.Tensor]] = None, R: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
         """One launch for a group.  Each member is a dict with `qweight`, `scales`, `qzeros` and optional
-        `L` ([N, rank] fp16 or None) and `bias` ([N] fp16 or None).  Returns the [M, N_i] fp16 outputs."""
+        `L` ([N, rank] fp16 or None) and `bias` ([N] fp16 or None).  Returns the [M, N_i] fp16 outputs.
+        With `R` ([rank, K] fp16) the launch computes r = x R^T itself and writes it into `r` (an
+        [M, rank] fp16 buffer) for the caller's cache; without it `r` is an input."""
         _check(1 <= len(members) <= MAX_MEMBERS, f"group_forward: 1..{MAX_MEMBERS} members")
         _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2, "inputs must be CUDA fp16 [M, IC]")
         x = x.contiguous()
@@ -187,6 +190,10 @@ class W4A16Extension:
         arr = (_Member * len(members))()
         keep = []
         rank = 0
+        if R is not None:
+            _check(R.is_cuda and R.dtype == torch.float16 and R.dim() == 2 and R.size(1) == K and R.is_contiguous(),
+                   "group_forward: R must be a contiguous CUDA fp16 [rank, K] tensor")
+            _check(r is not None and tuple(r.shape) == (M, R.size(0)), "group_forward: r must be an [M, rank] output buffer when R is given")
         if r is not None:
             _check(r.is_cuda and r.dtype == torch.float16 and r.dim() == 2 and r.size(0) == M and r.is_contiguous(),
                    "group_forward: r must be a contiguous CUDA fp16 [M, rank] tensor")
@@ -220,9 +227,14 @@ class W4A16Extension:
         if M == 0:
             return result
         with torch.cuda.device(x.device):
-            rc = self.lib.glowq_w4a16_group_forward(
-                x.data_ptr(), r.data_ptr() if r is not None else None, arr, len(members), M, K, int(group_size),
-                int(rank), float(alpha), self._stream(x.device))
+            if R is not None:
+                rc = self.lib.glowq_w4a16_group_forward_fused(
+                    x.data_ptr(), R.data_ptr(), r.data_ptr(), arr, len(members), M, K, int(group_size),
+                    int(rank), float(alpha), self._stream(x.device))
+            else:
+                rc = self.lib.glowq_w4a16_group_forward(
+                    x.data_ptr(), r.data_ptr() if r is not None else None, arr, len(members), M, K, int(group_size),
+                    int(rank), float(alpha), self._stream(x.device))
         if rc:
             self._raise(rc, "w4a16_group_forward")
         return result

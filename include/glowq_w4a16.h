@@ -114,6 +114,14 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
                               int K, int group_size, int rank, float alpha, void* stream);
 
 /*
+ * Projection and group in one call: r_out = fp16(x R^T) ([M, rank], for the caller's group cache) followed by
+ * the group launch that consumes it.  Replaces the whole body of `AddSVDCorrection.forward` for a group
+ * (src/step3_eval_dataset.py:470-511) with one library call (two launches on `stream`).
+ */
+int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                    int n_members, int M, int K, int group_size, int rank, float alpha, void* stream);
+
+/*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
  * 2 = tiled MFMA GEMM, 3 = generic (odd shapes).
  */
