@@ -16,6 +16,8 @@
 //     the same way on their way into LDS, so no instruction is spent on reordering weights.
 //   * The rank-r correction is a K-extension that runs first: acc = r . L^T on the same pipeline with an
 //     fp16 B operand, acc *= alpha, then the quantised K loop accumulates on top.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace glowq {
@@ -35,6 +37,13 @@ struct GemmArgs {
   int M, N, K, group_size, rank;
   int ldw, lds, ldz, ldb, ldy;
   float alpha;
+};
+
+// One launch covers every member of a group: workgroup b serves member i for blk_end[i-1] <= b < blk_end[i].
+struct GemmGroup {
+  GemmArgs m[GLOWQ_MAX_MEMBERS];
+  int blk_end[GLOWQ_MAX_MEMBERS];
+  int n;
 };
 
 __device__ __forceinline__ h8 permute_for_nibble_order(const h8& v) {
@@ -64,7 +73,20 @@ __device__ __forceinline__ h8 dequant_word(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2
 
 // kQuant: B is the int4 weight (with the optional correction phase in front); otherwise B is plain fp16.
 template <int kMT, int kNT, bool kQuant>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const int m_blocks) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
+void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
+  // member of this workgroup, picked with scalar selects from fixed kernel-argument offsets
+  GemmArgs a = gg.m[0];
+  int blk_base = 0;
+#define GLOWQ_PICK(i)                                         \
+  if (gg.n > i && (int)blockIdx.x >= gg.blk_end[i - 1]) {    \
+    a = gg.m[i];                                              \
+    blk_base = gg.blk_end[i - 1];                             \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int BM = 32 * kMT;
   constexpr int BN = 128 * kNT;
@@ -73,8 +95,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int bm = blockIdx.x % m_blocks;  // row blocks vary fastest: neighbouring workgroups share weight columns
-  const int bn = blockIdx.x / m_blocks;
+  const int blk = (int)blockIdx.x - blk_base;
+  const int bm = blk % m_blocks;  // row blocks vary fastest: neighbouring workgroups share weight columns
+  const int bn = blk / m_blocks;
   const int m0 = bm * BM;
   const int ln = lane & 31;  // column inside a 32-wide tile (B operand, accumulator) / row inside a tile (A operand)
   const int lh = lane >> 5;  // which half of the k range of an MFMA step this lane feeds
@@ -94,23 +117,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const 
   // ---- activation tile: global -> registers -> LDS ------------------------------------------------
   // BM rows x 8 octets (16 bytes); thread t takes octets t, t+256, ...: 8 consecutive threads read the
   // 128 contiguous bytes of one row.
-  h8 areg[kMT];
-  auto load_a = [&](const half_t* src, int ld, int kb) {
+  struct ARegs {
+    u32x4 v[kMT];
+  };
+  ARegs areg, areg1;
+  auto load_a_to = [&](ARegs& dst, const half_t* src, int ld, int kb) {
 #pragma unroll
     for (int i = 0; i < kMT; ++i) {
       const int q = tid + 256 * i;
       const int row = min(m0 + (q >> 3), a.M - 1);
-      areg[i] = *reinterpret_cast<const h8*>(src + (size_t)row * ld + kb + (q & 7) * 8);
+      dst.v[i] = *reinterpret_cast<const u32x4*>(src + (size_t)row * ld + kb + (q & 7) * 8);
     }
   };
-  auto store_a = [&](int stage, bool permute) {
+  auto store_a_from = [&](const ARegs& srcr, int stage, bool permute) {
 #pragma unroll
     for (int i = 0; i < kMT; ++i) {
       const int q = tid + 256 * i;
       half_t* dst = lds_a + ((size_t)stage * BM + (q >> 3)) * kARow + (q & 7) * 8;
-      *reinterpret_cast<h8*>(dst) = permute ? permute_for_nibble_order(areg[i]) : areg[i];
+      const h8 v = __builtin_bit_cast(h8, srcr.v[i]);
+      *reinterpret_cast<h8*>(dst) = permute ? permute_for_nibble_order(v) : v;
     }
   };
+  auto load_a = [&](const half_t* src, int ld, int kb) { load_a_to(areg, src, ld, kb); };
+  auto store_a = [&](int stage, bool permute) { store_a_from(areg, stage, permute); };
   // A fragment of MFMA step t for row tile tm: octet (4*lh + t) of row tm*32 + ln
   auto read_a = [&](int stage, int tm, int t) {
     const half_t* src = lds_a + ((size_t)stage * BM + tm * 32 + ln) * kARow + (4 * lh + t) * 8;
@@ -169,71 +198,101 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const 
   const int steps = a.K / kBK;
   const int gs_shift = __builtin_ctz(a.group_size);  // group sizes on this route are powers of two
   if constexpr (kQuant) {
-    // quantised B: per step and column tile one 16-byte load of codes, one scale, one zero-point word
-    u32x4 wq[kNT], wq_next[kNT];
-    half_t sc[kNT], sc_next[kNT];
-    uint32_t zw[kNT], zw_next[kNT];
-    auto load_w = [&](int kb, u32x4 (&w)[kNT], half_t (&s)[kNT], uint32_t (&z)[kNT]) {
+    // quantised B: per step and column tile one 16-byte load of codes, one scale, one zero-point word.
+    // Two register sets alternate (no copies), and the prefetch of the next step is unconditional (the
+    // last step re-reads its own block): a uniform number of loads per step keeps the wait counts exact,
+    // so the loads issued at the top of a step stay in flight under that step's MFMAs.
+    struct WRegs {  // all members 32-bit wide: the struct stays in registers
+      u32x4 w[kNT];
+      uint32_t s[kNT];  // fp16 bits of the scale
+      uint32_t z[kNT];
+    };
+    auto load_w = [&](int kb, WRegs& wr) {
       const int grp = (kb + 32 * lh) >> gs_shift;
 #pragma unroll
       for (int tn = 0; tn < kNT; ++tn) {
-        w[tn] = *reinterpret_cast<const u32x4*>(a.qweight + (size_t)ncol[tn] * a.ldw + (kb >> 3) + 4 * lh);
-        s[tn] = a.scales[(size_t)ncol[tn] * a.lds + grp];
-        z[tn] = (uint32_t)a.qzeros[(size_t)ncol[tn] * a.ldz + (grp >> 3)];
+        wr.w[tn] = *reinterpret_cast<const u32x4*>(a.qweight + (size_t)ncol[tn] * a.ldw + (kb >> 3) + 4 * lh);
+        wr.s[tn] = reinterpret_cast<const unsigned short*>(a.scales)[(size_t)ncol[tn] * a.lds + grp];
+        wr.z[tn] = (uint32_t)a.qzeros[(size_t)ncol[tn] * a.ldz + (grp >> 3)];
       }
     };
-    load_a(a.x, a.K, 0);
-    load_w(0, wq, sc, zw);
-    store_a(stage, true);
-    __syncthreads();
-    for (int ks = 0; ks < steps; ++ks) {
+    // Step s: dequantise W(s) out of its register set, refill that set with W(s+2) and the matching
+    // activation set with A(s+2), run the MFMAs of step s on LDS stage s%2, then move A(s+1) (loaded one
+    // step ago, so it has had a whole step to arrive) into the other LDS stage.  Loads are unconditional
+    // (clamped to the last block) so that every step issues the same number of them.
+    auto step = [&](int ks, WRegs& wr, ARegs& a_fill, const ARegs& a_store) {
       const int kb = ks * kBK;
-      if (ks + 1 < steps) {
-        load_a(a.x, a.K, kb + kBK);
-        load_w(kb + kBK, wq_next, sc_next, zw_next);
-      }
       h8 bfrag[kNT][4];
       const int grp = (kb + 32 * lh) >> gs_shift;
 #pragma unroll
       for (int tn = 0; tn < kNT; ++tn) {
-        const half_t z = (half_t)(float)nibble(zw[tn], grp & 7);
+        const half_t z = (half_t)(float)nibble(wr.z[tn], grp & 7);
         const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
-        const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh}, s2 = {sc[tn], sc[tn]};
-        bfrag[tn][0] = dequant_word(wq[tn].x, zb_lo, zb_hi, s2);
-        bfrag[tn][1] = dequant_word(wq[tn].y, zb_lo, zb_hi, s2);
-        bfrag[tn][2] = dequant_word(wq[tn].z, zb_lo, zb_hi, s2);
-        bfrag[tn][3] = dequant_word(wq[tn].w, zb_lo, zb_hi, s2);
+        const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh};
+        const h2 s2 = bitcast_u32<h2>(wr.s[tn] | (wr.s[tn] << 16));
+        bfrag[tn][0] = dequant_word(wr.w[tn].x, zb_lo, zb_hi, s2);
+        bfrag[tn][1] = dequant_word(wr.w[tn].y, zb_lo, zb_hi, s2);
+        bfrag[tn][2] = dequant_word(wr.w[tn].z, zb_lo, zb_hi, s2);
+        bfrag[tn][3] = dequant_word(wr.w[tn].w, zb_lo, zb_hi, s2);
       }
+      const int kb2 = min(ks + 2, steps - 1) * kBK;
+      load_w(kb2, wr);
+      load_a_to(a_fill, a.x, a.K, kb2);
       mma_step(stage, bfrag);
-      if (ks + 1 < steps) {
-        store_a(stage ^ 1, true);
-#pragma unroll
-        for (int tn = 0; tn < kNT; ++tn) {
-          wq[tn] = wq_next[tn];
-          sc[tn] = sc_next[tn];
-          zw[tn] = zw_next[tn];
-        }
-      }
+      store_a_from(a_store, stage ^ 1, true);
       __syncthreads();
       stage ^= 1;
+    };
+    WRegs w0, w1;
+    load_a_to(areg, a.x, a.K, 0);
+    load_w(0, w0);
+    load_a_to(areg1, a.x, a.K, min(1, steps - 1) * kBK);
+    load_w(min(1, steps - 1) * kBK, w1);
+    store_a_from(areg, stage, true);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ks += 2) {
+      step(ks, w0, areg, areg1);
+      if (ks + 1 >= steps) break;
+      step(ks + 1, w1, areg1, areg);
     }
   } else {
-    // plain fp16 B (the shared projection r = x R^T for many rows)
-    load_a(a.x, a.K, 0);
-    store_a(stage, false);
-    __syncthreads();
-    for (int ks = 0; ks < steps; ++ks) {
-      h8 bfrag[kNT][4];
+    // plain fp16 B (the shared projection r = x R^T for many rows): same two-deep pipeline, the B
+    // fragments are loaded as they are (4 x 16 bytes per lane, column tile and step)
+    struct BRegs {
+      u32x4 v[kNT][4];
+    };
+    auto load_b = [&](int kb, BRegs& br) {
 #pragma unroll
       for (int tn = 0; tn < kNT; ++tn)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + ks * kBK + 32 * lh + 8 * t);
-      if (ks + 1 < steps) load_a(a.x, a.K, (ks + 1) * kBK);
+          br.v[tn][t] = *reinterpret_cast<const u32x4*>(a.bmat + (size_t)ncol[tn] * a.ldb + kb + 32 * lh + 8 * t);
+    };
+    auto step = [&](int ks, BRegs& br, ARegs& a_fill, const ARegs& a_store) {
+      h8 bfrag[kNT][4];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bfrag[tn][t] = __builtin_bit_cast(h8, br.v[tn][t]);
+      const int kb2 = min(ks + 2, steps - 1) * kBK;
+      load_b(kb2, br);
+      load_a_to(a_fill, a.x, a.K, kb2);
       mma_step(stage, bfrag);
-      if (ks + 1 < steps) store_a(stage ^ 1, false);
+      store_a_from(a_store, stage ^ 1, false);
       __syncthreads();
       stage ^= 1;
+    };
+    BRegs b0, b1;
+    load_a_to(areg, a.x, a.K, 0);
+    load_b(0, b0);
+    load_a_to(areg1, a.x, a.K, min(1, steps - 1) * kBK);
+    load_b(min(1, steps - 1) * kBK, b1);
+    store_a_from(areg, stage, false);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ks += 2) {
+      step(ks, b0, areg, areg1);
+      if (ks + 1 >= steps) break;
+      step(ks + 1, b1, areg1, areg);
     }
   }
 
@@ -256,7 +315,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const GemmArgs a, const 
 
 // ---- host side ------------------------------------------------------------------------------------
 template <int kMT, int kNT, bool kQuant>
-static hipError_t launch_gemm_t(const GemmArgs& a, hipStream_t stream) {
+static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
   auto kern = gemm_mfma_kernel<kMT, kNT, kQuant>;
   const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t);
@@ -266,18 +325,28 @@ static hipError_t launch_gemm_t(const GemmArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     configured = true;
   }
-  const int m_blocks = (a.M + BM - 1) / BM;
-  const int n_blocks = (a.N + BN - 1) / BN;
-  hipLaunchKernelGGL(kern, dim3(m_blocks * n_blocks), dim3(256), lds, stream, a, m_blocks);
+  const int m_blocks = (gg.m[0].M + BM - 1) / BM;
+  int total = 0;
+  for (int i = 0; i < gg.n; ++i) {
+    total += m_blocks * ((gg.m[i].N + BN - 1) / BN);
+    gg.blk_end[i] = total;
+  }
+  hipLaunchKernelGGL(kern, dim3(total), dim3(256), lds, stream, gg, m_blocks);
   return hipGetLastError();
 }
 
-static hipError_t launch_gemm_args(const GemmArgs& a, hipStream_t stream) {
-  // row tiles per workgroup: the largest that M fills; column tiles: 2 per wave unless N is small
-  const int nt = a.N > 128 ? 2 : 1;
-  int mt = a.M > 128 ? 8 : (a.M > 64 ? 4 : (a.M > 32 ? 2 : 1));
+static hipError_t launch_gemm_group(GemmGroup& gg, hipStream_t stream) {
+  // row tiles per workgroup: the largest that M fills (capped: 4 keeps two workgroups per CU resident);
+  // column tiles: 2 per wave unless every member is narrow
+  int n_max = 0;
+  for (int i = 0; i < gg.n; ++i) n_max = gg.m[i].N > n_max ? gg.m[i].N : n_max;
+  const int nt = n_max > 128 ? 2 : 1;
+  const int M = gg.m[0].M;
+  static const int mt_max = getenv("GLOWQ_GEMM_MT") ? atoi(getenv("GLOWQ_GEMM_MT")) : 4;
+  int mt = M > 128 ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
+  if (mt > mt_max) mt = mt_max;
 #define GLOWQ_GEMM_CASE(MT, NT) \
-  if (mt == MT && nt == NT) return launch_gemm_t<MT, NT, true>(a, stream);
+  if (mt == MT && nt == NT) return launch_gemm_t<MT, NT, true>(gg, stream);
   GLOWQ_GEMM_CASE(8, 2) GLOWQ_GEMM_CASE(4, 2) GLOWQ_GEMM_CASE(2, 2) GLOWQ_GEMM_CASE(1, 2)
   GLOWQ_GEMM_CASE(8, 1) GLOWQ_GEMM_CASE(4, 1) GLOWQ_GEMM_CASE(2, 1) GLOWQ_GEMM_CASE(1, 1)
 #undef GLOWQ_GEMM_CASE
@@ -301,9 +370,11 @@ bool gemm_supported(const GroupDev& g) {
 
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
   (void)num_cus;
+  GemmGroup gg;
+  gg.n = g.n_members;
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
-    GemmArgs a;
+    GemmArgs& a = gg.m[i];
     a.x = g.x;
     a.r = (m.L != nullptr) ? g.r : nullptr;
     a.qweight = m.qweight;
@@ -323,10 +394,8 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
     a.ldb = g.rank;
     a.ldy = m.ldy;
     a.alpha = g.alpha;
-    hipError_t e = launch_gemm_args(a, stream);
-    if (e != hipSuccess) return e;
   }
-  return hipSuccess;
+  return launch_gemm_group(gg, stream);
 }
 
 // r[M, rank] = fp16(x[M, K] . R[rank, K]^T) on the same kernel with an fp16 B operand.
@@ -334,7 +403,9 @@ hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, 
                                    hipStream_t stream) {
   (void)num_cus;
   if ((K % kBK) != 0) return hipErrorInvalidValue;
-  GemmArgs a;
+  GemmGroup gg;
+  gg.n = 1;
+  GemmArgs& a = gg.m[0];
   a.x = x;
   a.r = nullptr;
   a.qweight = nullptr;
@@ -353,8 +424,8 @@ hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, 
   a.ldy = rank;
   a.alpha = 1.0f;
   // small row tiles: N is tiny here, the parallelism has to come from M
-  if (rank > 128) return launch_gemm_t<2, 2, false>(a, stream);
-  return launch_gemm_t<2, 1, false>(a, stream);
+  if (rank > 128) return launch_gemm_t<1, 2, false>(gg, stream);
+  return launch_gemm_t<1, 1, false>(gg, stream);
 }
 
 }  // namespace glowq
