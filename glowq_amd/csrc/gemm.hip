@@ -398,34 +398,156 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
   return launch_gemm_group(gg, stream);
 }
 
-// r[M, rank] = fp16(x[M, K] . R[rank, K]^T) on the same kernel with an fp16 B operand.
+// ---- shared projection for many rows: r[M, rank] = fp16(x[M, K] . R[rank, K]^T) ---------------------------
+// N = rank is tiny, so the parallelism has to come from M and K: a workgroup owns 32 rows of x and up to 128
+// columns of r, and its four waves split K -- wave w takes the 64-deep slice w of every 256-deep block, with
+// its own A fragments (x, staged in LDS for all four slices at once) and its own B fragments (R, straight
+// from global memory, prefetched one block ahead).  There is no barrier-bound dependency between the waves
+// inside a block beyond the staging of x; the four partial tiles meet in LDS once, at the end.
+constexpr int kPK = 256;           // k depth of one block (4 waves x 64)
+constexpr int kPRow = kPK + 8;     // padded LDS row in halves
+
+template <int kNT>
+__global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict__ x, const half_t* __restrict__ R,
+                                                        half_t* __restrict__ r, int M, int K, int rank) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  half_t* lds_x = reinterpret_cast<half_t*>(smem);  // [2][32][kPRow]; reused for the final reduction
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+  const int m0 = blockIdx.x * 32;
+  const int n0 = blockIdx.y * (32 * kNT);
+  const int blocks = (K + kPK - 1) / kPK;  // K is a multiple of 64; the last block may be partial
+
+  int ncol[kNT];
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) ncol[tn] = min(n0 + tn * 32 + ln, rank - 1);
+
+  f16v acc[kNT];
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[tn][i] = 0.f;
+
+  // x tile of a block: 32 rows x 32 octets; thread t takes octets t, t+256, t+512, t+768
+  struct XRegs {
+    u32x4 v[4];
+  };
+  auto load_x = [&](int kb, XRegs& xr) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = tid + 256 * i;
+      const int row = min(m0 + (q >> 5), M - 1);
+      const int k = min(kb + (q & 31) * 8, K - 8);
+      xr.v[i] = *reinterpret_cast<const u32x4*>(x + (size_t)row * K + k);
+    }
+  };
+  auto store_x = [&](int stage, const XRegs& xr) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = tid + 256 * i;
+      *reinterpret_cast<u32x4*>(lds_x + ((size_t)stage * 32 + (q >> 5)) * kPRow + (q & 31) * 8) = xr.v[i];
+    }
+  };
+  struct BRegs {
+    u32x4 v[kNT][4];
+  };
+  // this wave's slice of a block: columns kb + 64*wave .. +63; a slice past the end of K is weighted by zero
+  auto load_b = [&](int kb, BRegs& br) {
+    const int ks = min(kb + 64 * wave, K - 64);
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        br.v[tn][t] = *reinterpret_cast<const u32x4*>(R + (size_t)ncol[tn] * K + ks + 32 * lh + 8 * t);
+  };
+  auto mma_block = [&](int stage, int kb, const BRegs& br) {
+    if (kb + 64 * wave >= K) return;  // wave-uniform: nothing of this slice lies inside K
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const h8 af = *reinterpret_cast<const h8*>(lds_x + ((size_t)stage * 32 + ln) * kPRow + 64 * wave + (4 * lh + t) * 8);
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+        acc[tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, __builtin_bit_cast(h8, br.v[tn][t]), acc[tn], 0, 0, 0);
+    }
+  };
+
+  int stage = 0;
+  // Block s: copy B(s) out of its register set, refill that set with B(s+2) and the matching x set with
+  // x(s+2), run the MFMAs of block s on LDS stage s%2, then move x(s+1) (loaded one block ago) into the other
+  // stage.  Two blocks of loads are in flight at any time.
+  auto block = [&](int blk, BRegs& br, XRegs& x_fill, const XRegs& x_store) {
+    BRegs cur = br;
+    const int kn = min(blk + 2, blocks - 1) * kPK;
+    load_b(kn, br);
+    load_x(kn, x_fill);
+    mma_block(stage, blk * kPK, cur);
+    store_x(stage ^ 1, x_store);
+    __syncthreads();
+    stage ^= 1;
+  };
+  XRegs x0, x1;
+  BRegs b0, b1;
+  load_x(0, x0);
+  load_b(0, b0);
+  load_x(min(1, blocks - 1) * kPK, x1);
+  load_b(min(1, blocks - 1) * kPK, b1);
+  store_x(0, x0);
+  __syncthreads();
+  for (int blk = 0; blk < blocks; blk += 2) {
+    block(blk, b0, x0, x1);
+    if (blk + 1 >= blocks) break;
+    block(blk + 1, b1, x1, x0);
+  }
+
+  // the four K slices meet in LDS: [wave][tile][16 regs][64 lanes] floats
+  float* red = reinterpret_cast<float*>(smem);
+  __syncthreads();
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[((wave * kNT + tn) * 16 + i) * 64 + lane] = acc[tn][i];
+  __syncthreads();
+  // wave w finishes registers 4w .. 4w+3 of every tile
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) {
+    const int n = n0 + tn * 32 + ln;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int i = wave * 4 + ii;
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v += red[((w * kNT + tn) * 16 + i) * 64 + lane];
+      const int m = m0 + 8 * (i >> 2) + 4 * lh + (i & 3);
+      if (m < M && n < rank) r[(size_t)m * rank + n] = (half_t)v;
+    }
+  }
+}
+
 hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int num_cus,
                                    hipStream_t stream) {
   (void)num_cus;
-  if ((K % kBK) != 0) return hipErrorInvalidValue;
-  GemmGroup gg;
-  gg.n = 1;
-  GemmArgs& a = gg.m[0];
-  a.x = x;
-  a.r = nullptr;
-  a.qweight = nullptr;
-  a.scales = nullptr;
-  a.qzeros = nullptr;
-  a.bmat = R;
-  a.bias = nullptr;
-  a.y = r;
-  a.M = M;
-  a.N = rank;
-  a.K = K;
-  a.group_size = 128;
-  a.rank = 0;
-  a.ldw = a.lds = a.ldz = 0;
-  a.ldb = K;
-  a.ldy = rank;
-  a.alpha = 1.0f;
-  // small row tiles: N is tiny here, the parallelism has to come from M
-  if (rank > 128) return launch_gemm_t<1, 2, false>(gg, stream);
-  return launch_gemm_t<1, 1, false>(gg, stream);
+  if ((K % kBK) != 0 || K < kBK) return hipErrorInvalidValue;
+  const int m_blocks = (M + 31) / 32;
+  const size_t lds_x = (size_t)2 * 32 * kPRow * sizeof(half_t);
+  static const bool wide = getenv("GLOWQ_PROJ_WIDE") != nullptr;
+  if (rank > 64 && wide) {
+    constexpr int NT = 4;
+    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
+    static bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 127) / 128), dim3(256), lds, stream, x, R, r, M, K, rank);
+  } else {
+    constexpr int NT = 2;
+    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
+    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 63) / 64), dim3(256), lds, stream, x, R, r, M, K, rank);
+  }
+  return hipGetLastError();
 }
 
 }  // namespace glowq
