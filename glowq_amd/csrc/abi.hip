@@ -2,6 +2,7 @@
 // allocation, no synchronisation; see include/glowq_w4a16.h for the contract of each entry point.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "common.hpp"
@@ -53,7 +54,13 @@ int num_cus() {
 }
 
 constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3;
-constexpr int kWaveDotMaxM = 4;
+constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
+
+// rows up to which the wave-dot GEMV is preferred over the skinny MFMA kernel (tuning override: GLOWQ_WAVEDOT_M)
+int wave_dot_pref_m() {
+  static const int v = getenv("GLOWQ_WAVEDOT_M") ? atoi(getenv("GLOWQ_WAVEDOT_M")) : kWaveDotMaxM;
+  return v < 0 ? 0 : (v > kWaveDotMaxM ? kWaveDotMaxM : v);
+}
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
@@ -114,7 +121,7 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
-  if (g.M <= kWaveDotMaxM && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
+  if (g.M <= wave_dot_pref_m() && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
     return kRouteWaveDot;
   if (skinny_supported(g)) return kRouteSkinny;
   if (gemm_supported(g)) return kRouteGemm;

@@ -1,6 +1,311 @@
-// placeholder: skinny MFMA route not built yet
+// Skinny MFMA route for a handful of token rows (5 <= M <= 64): the weights are streamed once, like in the
+// GEMV, but the multiply-accumulate work goes to the matrix cores.
+//
+// A workgroup owns 32*kNT output columns of one member and all M rows; its waves split K: wave w takes the
+// a contiguous range of 64-deep blocks and keeps a private 32*kMT x 32*kNT accumulator tile
+// (v_mfma_f32_32x32x16_f16).  Nothing is shared between the waves while they stream, so there is no
+// barrier in the loop and every wave runs its own three-deep prefetch:
+//   * B operand: one 16-byte load of int4 codes per lane, block and column tile, dequantised in registers to
+//     fp16((code - zero) * scale) exactly as in the tiled GEMM;
+//   * A operand: the lane's 8 activations per MFMA step straight from global memory (x is a few hundred KB at
+//     most and lives in L2), permuted in registers into the order the nibble masks deliver the codes.  With
+//     kNT >= 2 every A fragment feeds two MFMAs, which keeps the L1 traffic per weight byte low enough.
+// The correction is a K-extension in front: the rank/64 blocks of [r | L] are dealt to the waves first,
+// acc *= alpha, then the weight blocks accumulate on top.  The waves' partial tiles meet in LDS once.
+#include <cstdlib>
+
 #include "common.hpp"
+
 namespace glowq {
-bool skinny_supported(const GroupDev&) { return false; }
-hipError_t launch_skinny(GroupDev&, int, hipStream_t) { return hipErrorNotSupported; }
+
+struct SkinnyMember {
+  const int32_t* qweight;
+  const half_t* scales;
+  const int32_t* qzeros;
+  const half_t* L;
+  const half_t* bias;
+  half_t* y;
+  int N, ldw, lds, ldz, ldy;
+};
+
+struct SkinnyArgs {
+  const half_t* x;  // [M, K]
+  const half_t* r;  // [M, rank] or nullptr
+  SkinnyMember mem[GLOWQ_MAX_MEMBERS];
+  int blk_end[GLOWQ_MAX_MEMBERS];
+  int n_members;
+  int M, K, rank, gs_shift;
+  float alpha;
+};
+
+__device__ __forceinline__ h8 nibble_order(const u32x4& v) {
+  // halves (0..7) -> (0,4,1,5,2,6,3,7): two byte permutes per output dword
+  u32x4 o;
+  o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (h0, h4)
+  o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (h1, h5)
+  o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (h2, h6)
+  o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (h3, h7)
+  return __builtin_bit_cast(h8, o);
+}
+
+__device__ __forceinline__ h8 dequant_word_sk(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2) {
+  const uint32_t hi = w >> 8;
+  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | 0x64006400u);
+  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | 0x54005400u);
+  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | 0x64006400u);
+  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | 0x54005400u);
+  const h2 d0 = (q0 + zb_lo) * s2;
+  const h2 d1 = (q1 + zb_hi) * s2;
+  const h2 d2 = (q2 + zb_lo) * s2;
+  const h2 d3 = (q3 + zb_hi) * s2;
+  h8 out;
+  out[0] = d0[0]; out[1] = d0[1]; out[2] = d1[0]; out[3] = d1[1];
+  out[4] = d2[0]; out[5] = d2[1]; out[6] = d3[0]; out[7] = d3[1];
+  return out;
+}
+
+// What one block needs: per column tile 16 bytes of codes (or 4 x 16 bytes of L), scale and zero-point word,
+// and per row tile the four A fragments.
+template <int kMT, int kNT>
+struct SkinnyRegs {
+  u32x4 a[kMT][4];
+  u32x4 b[kNT];
+  uint32_t s[kNT];
+  uint32_t z[kNT];
+};
+
+template <int kMT, int kNT>
+__global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves = blockDim.x >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+
+  SkinnyMember mem = g.mem[0];
+  int blk_base = 0;
+#define GLOWQ_PICK(i)                                          \
+  if (g.n_members > i && (int)blockIdx.x >= g.blk_end[i - 1]) { \
+    mem = g.mem[i];                                            \
+    blk_base = g.blk_end[i - 1];                               \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
+  const int n0 = ((int)blockIdx.x - blk_base) * (32 * kNT);
+
+  int ncol[kNT];
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) ncol[tn] = min(n0 + tn * 32 + ln, mem.N - 1);
+  int mrow[kMT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm) mrow[tm] = min(tm * 32 + ln, g.M - 1);
+
+  f16v acc[kMT][kNT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
+
+  // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
+  const bool corrected = mem.L != nullptr && g.r != nullptr;
+  if (corrected) {
+    const int lblocks = g.rank >> 6;
+    for (int jb = wave; jb < lblocks; jb += waves) {
+      const int kb = jb * 64;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        h8 af[kMT];
+#pragma unroll
+        for (int tm = 0; tm < kMT; ++tm)
+          af[tm] = *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kb + 32 * lh + 8 * t);
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) {
+          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kb + 32 * lh + 8 * t);
+#pragma unroll
+          for (int tm = 0; tm < kMT; ++tm) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf, acc[tm][tn], 0, 0, 0);
+        }
+      }
+    }
+    if (g.alpha != 1.0f) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= g.alpha;
+    }
+  }
+
+  // ---- phase 2: weight blocks, three register sets in rotation ------------------------------------------
+  // Wave w walks the contiguous block range [w*per, (w+1)*per): consecutive steps of a wave touch
+  // consecutive 32-byte pieces of the same 128-byte lines of its 32 weight rows, so every line is fetched
+  // from HBM once and re-used out of L2.
+  const int kblocks = g.K >> 6;
+  const int per = (kblocks + waves - 1) / waves;
+  const int first_blk = wave * per;
+  const int my_blocks = max(0, min(per, kblocks - first_blk));
+  auto issue = [&](int i, SkinnyRegs<kMT, kNT>& rg) {
+    const int blk = min(first_blk + i, kblocks - 1);  // past-the-end prefetches re-read the last block
+    const int kb = blk * 64;
+    const int grp = (kb + 32 * lh) >> g.gs_shift;
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      rg.b[tn] = *reinterpret_cast<const u32x4*>(mem.qweight + (size_t)ncol[tn] * mem.ldw + (kb >> 3) + 4 * lh);
+      rg.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
+      rg.z[tn] = (uint32_t)mem.qzeros[(size_t)ncol[tn] * mem.ldz + (grp >> 3)];
+    }
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        rg.a[tm][t] = *reinterpret_cast<const u32x4*>(g.x + (size_t)mrow[tm] * g.K + kb + 32 * lh + 8 * t);
+  };
+  auto compute = [&](int i, const SkinnyRegs<kMT, kNT>& rg) {
+    const int kb = (first_blk + i) * 64;
+    const int grp = (kb + 32 * lh) >> g.gs_shift;
+    h8 bf[kNT][4];
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      const half_t z = (half_t)(float)nibble(rg.z[tn], grp & 7);
+      const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
+      const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh};
+      const h2 s2 = bitcast_u32<h2>(rg.s[tn] | (rg.s[tn] << 16));
+      bf[tn][0] = dequant_word_sk(rg.b[tn].x, zb_lo, zb_hi, s2);
+      bf[tn][1] = dequant_word_sk(rg.b[tn].y, zb_lo, zb_hi, s2);
+      bf[tn][2] = dequant_word_sk(rg.b[tn].z, zb_lo, zb_hi, s2);
+      bf[tn][3] = dequant_word_sk(rg.b[tn].w, zb_lo, zb_hi, s2);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm) {
+        const h8 af = nibble_order(rg.a[tm][t]);
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf[tn][t], acc[tm][tn], 0, 0, 0);
+      }
+    }
+  };
+
+  // The fences pin the loads where they are written: with no barrier in this loop the compiler is otherwise
+  // free to sink them down to their uses, which would collapse the three-deep pipeline into none.
+#define GLOWQ_PIN_LOADS() asm volatile("" ::: "memory")
+  SkinnyRegs<kMT, kNT> r0, r1, r2;
+  issue(0, r0);
+  issue(1, r1);
+  GLOWQ_PIN_LOADS();
+  for (int i = 0; i < my_blocks; i += 3) {
+    issue(i + 2, r2);
+    GLOWQ_PIN_LOADS();
+    compute(i, r0);
+    if (i + 1 >= my_blocks) break;
+    issue(i + 3, r0);
+    GLOWQ_PIN_LOADS();
+    compute(i + 1, r1);
+    if (i + 2 >= my_blocks) break;
+    issue(i + 4, r1);
+    GLOWQ_PIN_LOADS();
+    compute(i + 2, r2);
+  }
+#undef GLOWQ_PIN_LOADS
+
+  // ---- the waves' partial tiles meet in LDS: [wave][tm][tn][16 regs][64 lanes] floats, in rounds of 8 waves
+  float* red = reinterpret_cast<float*>(smem);
+  constexpr int kTile = kMT * kNT * 16 * 64;
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) red[(size_t)wave * kTile + ((tm * kNT + tn) * 16 + i) * 64 + lane] = acc[tm][tn][i];
+  __syncthreads();
+  // every thread finishes a share of the (tile, register, lane) slots
+  const int slots = kMT * kNT * 16 * 64;
+  for (int sidx = threadIdx.x; sidx < slots; sidx += blockDim.x) {
+    float v = 0.f;
+    for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + sidx];
+    const int l = sidx & 63;
+    const int i = (sidx >> 6) & 15;
+    const int tt = sidx >> 10;
+    const int tm = tt / kNT, tn = tt - tm * kNT;
+    const int n = n0 + tn * 32 + (l & 31);
+    const int m = tm * 32 + 8 * (i >> 2) + 4 * (l >> 5) + (i & 3);
+    if (m < g.M && n < mem.N) {
+      const float b = mem.bias ? (float)mem.bias[n] : 0.f;
+      mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
+    }
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------
+bool skinny_supported(const GroupDev& g) {
+  if (g.M < 1 || g.M > 64) return false;
+  if ((g.K & 63) != 0 || (g.group_size & 31) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
+  if (g.r != nullptr && (g.rank & 63) != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
+  if (g.r != nullptr && (reinterpret_cast<uintptr_t>(g.r) & 15u) != 0) return false;
+  for (int i = 0; i < g.n_members; ++i) {
+    const MemberDev& m = g.mem[i];
+    if ((reinterpret_cast<uintptr_t>(m.qweight) & 15u) != 0 || (m.ldw & 3) != 0) return false;
+    if (m.L != nullptr && (reinterpret_cast<uintptr_t>(m.L) & 15u) != 0) return false;
+  }
+  return true;
+}
+
+template <int kMT, int kNT>
+static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) {
+  auto kern = skinny_mfma_kernel<kMT, kNT>;
+  const size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
+  static size_t configured = 48 * 1024;
+  if (lds > configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    configured = lds;
+  }
+  int total = 0;
+  for (int i = 0; i < a.n_members; ++i) {
+    total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
+    a.blk_end[i] = total;
+  }
+  hipLaunchKernelGGL(kern, dim3(total), dim3(waves * 64), lds, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
+  (void)num_cus;
+  SkinnyArgs a;
+  a.x = g.x;
+  a.r = g.r;
+  a.n_members = g.n_members;
+  a.M = g.M;
+  a.K = g.K;
+  a.rank = g.rank;
+  a.gs_shift = __builtin_ctz(g.group_size);
+  a.alpha = g.alpha;
+  for (int i = 0; i < g.n_members; ++i) {
+    const MemberDev& m = g.mem[i];
+    SkinnyMember& s = a.mem[i];
+    s.qweight = m.qweight;
+    s.scales = m.scales;
+    s.qzeros = m.qzeros;
+    s.L = m.L;
+    s.bias = m.bias;
+    s.y = m.y;
+    s.N = m.N;
+    s.ldw = m.ldw;
+    s.lds = m.lds;
+    s.ldz = m.ldz;
+    s.ldy = m.ldy;
+  }
+  static const int env_waves = getenv("GLOWQ_SKINNY_WAVES") ? atoi(getenv("GLOWQ_SKINNY_WAVES")) : 0;
+  int waves = (env_waves >= 1 && env_waves <= 8) ? env_waves : 8;
+  const int kblocks = g.K >> 6;
+  if (waves > kblocks) waves = kblocks;
+  if (g.M <= 32) return launch_skinny_t<1, 2>(a, waves, stream);
+  return launch_skinny_t<2, 2>(a, waves, stream);
+}
+
 }  // namespace glowq
