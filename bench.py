@@ -40,6 +40,7 @@ GROUPS = {
     "down_proj": (14336, [4096]),
 }
 DOMINANT = "gate_up"
+DOMINANT_TRAFFIC_BYTES = 68708000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
 
 
 def algorithmic_bytes(M, K, N, rank, gs=GROUP_SIZE):
@@ -118,6 +119,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain device copies of known size (256 MiB read + 256 MiB written each) so that "
+                         "FETCH_SIZE / WRITE_SIZE counters of a profiling run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU execution (run with --gpus 1)", file=sys.stderr)
@@ -180,7 +184,8 @@ def main():
     # dominant kernel: the gate|up group launch alone, 32 layers of
     # distinct weights back to back in one graph, HIP events around the replays on the launch stream
     K_d, Ns_d = GROUPS[DOMINANT]
-    dom_bytes = algorithmic_bytes(M_TOKENS, K_d, sum(Ns_d), RANK)
+    # the group kernel's own bytes: the group total minus R, which the projection launch reads
+    dom_bytes = algorithmic_bytes(M_TOKENS, K_d, sum(Ns_d), RANK) - 2 * RANK * K_d
     gdom = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
         with torch.cuda.graph(gdom, stream=side):
@@ -221,6 +226,18 @@ def main():
         by = algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK)
         per_group[name] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
 
+    if args.calibrate_copy:
+        # cold sources: 8 distinct 256 MiB buffers, each copied once (the kernel shows up in a profile as
+        # torch's elementwise copy kernel with 134217728 elements)
+        srcs = [torch.full((128 * 1024 * 1024,), float(i), dtype=torch.float16, device=dev) for i in range(8)]
+        dst = torch.empty_like(srcs[0])
+        graph.replay()  # push the sources out of the last-level cache
+        torch.cuda.synchronize()
+        for s_ in srcs:
+            dst.copy_(s_)
+        torch.cuda.synchronize()
+        del srcs, dst
+
     result = {
         "metric": "W4A16+GlowQ decode linears, microseconds per layer (Llama-3.1-8B shape, batch 1)",
         "value": round(us_per_layer, 3),
@@ -255,7 +272,9 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "avg_launch_us": round(dom_us, 3),
             "algorithmic_bytes_per_launch": dom_bytes,
-            "traffic": None,
+            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by the
+            # same counters on a 256 MiB copy (x1.9998 / x1.0): profiles/decode_linears_llama8b_hbm_traffic.md
+            "traffic": DOMINANT_TRAFFIC_BYTES,
         },
     }
     if not args.no_cpu_baseline:
