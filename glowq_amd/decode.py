@@ -1,0 +1,324 @@
+"""Minimal Llama-style decoder over the W4A16 + GlowQ linears, with a HIP-graph-captured decode step.
+
+The counterpart of what the reference measures with `generate()` (`measure_generation_metrics`,
+src/step3_eval_dataset.py:705-798: TTFB = wall of a 1-token generate, tok/s = new tokens / wall) and of the manual
+greedy loop with a KV cache in test/step3_1_layerwise.py:181-210 -- without Hugging Face: random-init weights of
+the named architecture (RMSNorm, RoPE, grouped-query attention, SwiGLU), HF-style module names
+(`model.layers.N.self_attn.{q,k,v,o}_proj`, `model.layers.N.mlp.{gate,up,down}_proj`) so that
+`convert_to_cuda_w4a16` and `patch_svd_correction_wrappers` apply unchanged, and the artifact key scheme of
+src/step2_rsvd.py:487-527 for the low-rank factors.
+
+    python -m glowq_amd.decode --layers 32 --prompt 512 --new 256        # Llama-3.1-8B shape, batch 1
+
+Only the linears are this library's kernels; norms, RoPE, attention and the lm_head are plain torch ops.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import time
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .correction import patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
+from .linear import CudaW4A16Linear, convert_to_cuda_w4a16
+
+
+@dataclass
+class DecoderConfig:
+    hidden: int = 4096
+    layers: int = 32
+    heads: int = 32
+    kv_heads: int = 8
+    head_dim: int = 128
+    intermediate: int = 14336
+    vocab: int = 128256
+    rope_theta: float = 500000.0
+    rms_eps: float = 1e-5
+    max_len: int = 1024
+    group_size: int = 128
+    rank: int = 128
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim, dtype=torch.float16))
+        self.eps = eps
+
+    def forward(self, x):
+        return F.rms_norm(x, (x.size(-1),), self.weight, self.eps)
+
+
+class Attention(nn.Module):
+    def __init__(self, cfg: DecoderConfig):
+        super().__init__()
+        self.cfg = cfg
+        h, d = cfg.hidden, cfg.head_dim
+        self.q_proj = nn.Linear(h, cfg.heads * d, bias=False)
+        self.k_proj = nn.Linear(h, cfg.kv_heads * d, bias=False)
+        self.v_proj = nn.Linear(h, cfg.kv_heads * d, bias=False)
+        self.o_proj = nn.Linear(cfg.heads * d, h, bias=False)
+
+    def forward(self, x, cos, sin, cache_k, cache_v, pos_idx, mask):
+        """x [T, hidden]; cos/sin [T, head_dim]; caches [kv_heads, max_len, head_dim]; pos_idx [T] (device,
+        positions of the T tokens); mask [T, max_len] additive."""
+        cfg = self.cfg
+        T = x.size(0)
+        q = self.q_proj(x).view(T, cfg.heads, cfg.head_dim).transpose(0, 1)      # [H, T, d]
+        k = self.k_proj(x).view(T, cfg.kv_heads, cfg.head_dim).transpose(0, 1)   # [KV, T, d]
+        v = self.v_proj(x).view(T, cfg.kv_heads, cfg.head_dim).transpose(0, 1)
+        q, k = _rope(q, cos, sin), _rope(k, cos, sin)
+        cache_k.index_copy_(1, pos_idx, k.to(cache_k.dtype))
+        cache_v.index_copy_(1, pos_idx, v.to(cache_v.dtype))
+        out = F.scaled_dot_product_attention(q.to(cache_k.dtype).unsqueeze(0), cache_k.unsqueeze(0), cache_v.unsqueeze(0),
+                                             attn_mask=mask.unsqueeze(0).unsqueeze(0), enable_gqa=True)
+        out = out.squeeze(0).transpose(0, 1).reshape(T, cfg.heads * cfg.head_dim)
+        return self.o_proj(out)
+
+
+def _rope(t, cos, sin):
+    d = t.size(-1) // 2
+    rot = torch.cat((-t[..., d:], t[..., :d]), dim=-1)
+    return t * cos + rot * sin
+
+
+class MLP(nn.Module):
+    def __init__(self, cfg: DecoderConfig):
+        super().__init__()
+        self.gate_proj = nn.Linear(cfg.hidden, cfg.intermediate, bias=False)
+        self.up_proj = nn.Linear(cfg.hidden, cfg.intermediate, bias=False)
+        self.down_proj = nn.Linear(cfg.intermediate, cfg.hidden, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, cfg: DecoderConfig):
+        super().__init__()
+        self.self_attn = Attention(cfg)
+        self.mlp = MLP(cfg)
+        self.input_layernorm = RMSNorm(cfg.hidden, cfg.rms_eps)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden, cfg.rms_eps)
+
+    def forward(self, x, cos, sin, cache_k, cache_v, pos_idx, mask):
+        x = x + self.self_attn(self.input_layernorm(x), cos, sin, cache_k, cache_v, pos_idx, mask)
+        return x + self.mlp(self.post_attention_layernorm(x))
+
+
+class _Body(nn.Module):
+    def __init__(self):
+        super().__init__()
+
+
+class Decoder(nn.Module):
+    """`model.embed_tokens`, `model.layers`, `model.norm`, `lm_head`: the attribute layout HF Llama uses."""
+
+    def __init__(self, cfg: DecoderConfig):
+        super().__init__()
+        self.cfg = cfg
+        self.model = _Body()
+        self.model.embed_tokens = nn.Embedding(cfg.vocab, cfg.hidden)
+        self.model.layers = nn.ModuleList()
+        self.model.norm = RMSNorm(cfg.hidden, cfg.rms_eps)
+        self.lm_head = nn.Linear(cfg.hidden, cfg.vocab, bias=False)
+
+    def rope_tables(self, device):
+        cfg = self.cfg
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32, device=device) / cfg.head_dim))
+        ang = torch.arange(cfg.max_len, dtype=torch.float32, device=device)[:, None] * inv[None, :]
+        ang = torch.cat((ang, ang), dim=-1)
+        return ang.cos(), ang.sin()
+
+    def forward_tokens(self, tokens, pos_idx, caches, cos_t, sin_t):
+        """tokens [T] (device), pos_idx [T] (device): logits [T, vocab] after writing the KV cache at pos_idx."""
+        cfg = self.cfg
+        x = self.model.embed_tokens(tokens)
+        cos, sin = cos_t.index_select(0, pos_idx).to(x.dtype), sin_t.index_select(0, pos_idx).to(x.dtype)
+        col = torch.arange(cfg.max_len, device=tokens.device)
+        mask = torch.where(col[None, :] <= pos_idx[:, None], 0.0, float("-inf")).to(torch.float16)
+        for layer, (ck, cv) in zip(self.model.layers, caches):
+            x = layer(x, cos, sin, ck, cv, pos_idx, mask)
+        return self.lm_head(self.model.norm(x))
+
+
+def build_decoder(cfg: DecoderConfig, device="cuda", seed: int = 3, with_correction: bool = True,
+                  groups_to_patch: Optional[set] = None) -> Tuple[Decoder, Dict[str, torch.Tensor], Dict[str, str]]:
+    """Random-init weights ~ N(0, 0.02) layer by layer on the device, each layer quantised as soon as it exists
+    (an 8B model never holds more than one layer in fp16), then synthetic low-rank factors in the artifact key
+    scheme (R ~ N(0, 1/K), L ~ N(0, 0.01^2)) patched in with the reference's patcher."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    model = Decoder(cfg).half()
+    model.model.embed_tokens.to(device)
+    model.model.norm.to(device)
+    model.lm_head.to(device)
+    with torch.no_grad():
+        model.model.embed_tokens.weight.normal_(0, 0.02, generator=g)
+        model.lm_head.weight.normal_(0, 0.02, generator=g)
+    for _ in range(cfg.layers):
+        layer = DecoderLayer(cfg).half().to(device)
+        with torch.no_grad():
+            for mod in layer.modules():
+                if isinstance(mod, nn.Linear):
+                    mod.weight.normal_(0, 0.02, generator=g)
+        convert_to_cuda_w4a16(layer, cfg.group_size)
+        model.model.layers.append(layer)
+    shared: Dict[str, torch.Tensor] = {}
+    bmap: Dict[str, str] = {}
+    if with_correction:
+        def rnd(*shape, std):
+            return (torch.randn(*shape, device=device, generator=g) * std).half()
+
+        for i, layer in enumerate(model.model.layers):
+            pre = f"model.layers.{i}"
+            for gname, sub, members in (("qkv", "self_attn", ("q_proj", "k_proj", "v_proj")), ("mlp", "mlp", ("gate_proj", "up_proj"))):
+                K = getattr(getattr(layer, sub), members[0]).in_features
+                shared[f"layer{i}_{gname}.B_shared"] = rnd(cfg.rank, K, std=K ** -0.5)
+                for mname in members:
+                    N = getattr(getattr(layer, sub), mname).out_features
+                    shared[f"layer{i}_{gname}.{mname}.A"] = rnd(N, cfg.rank, std=0.01)
+                    bmap[f"{pre}.{sub}.{mname}.weight"] = f"layer{i}_{gname}.B_shared"
+            for sub, mname in (("self_attn", "o_proj"), ("mlp", "down_proj")):
+                lin = getattr(getattr(layer, sub), mname)
+                mod = f"{pre}.{sub}.{mname}"
+                shared[f"{mod}.A"] = rnd(lin.out_features, cfg.rank, std=0.01)
+                shared[f"{mod}.B"] = rnd(cfg.rank, lin.in_features, std=lin.in_features ** -0.5)
+                bmap[f"{mod}.weight"] = f"{mod}.B"
+        if groups_to_patch is None:
+            patch_svd_correction_wrappers(model, shared, bmap, alpha_svd=1.0)
+        else:
+            patch_svd_correction_wrappers_cumulative(model, shared, bmap, groups_to_patch, alpha_svd=1.0)
+    return model.eval(), shared, bmap
+
+
+def load_glowq_artifacts(shared_path: str, bmap_path: str, device="cuda"):
+    """`low_rank_shared.pt` (dict name -> fp16 tensor) and `b_ref_map.json` (weight name -> key of its right factor)
+    as written by the reference's step 2 (src/step2_rsvd.py:519-527; consumer src/step3_eval_dataset.py:1077-1080).
+    Loaded with `weights_only=True`: nothing from the file is executed."""
+    shared = torch.load(shared_path, map_location=device, weights_only=True)
+    with open(bmap_path) as f:
+        bmap = json.load(f)
+    return shared, bmap
+
+
+class GreedyDecoder:
+    """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
+
+    def __init__(self, model: Decoder, use_graph: bool = True):
+        self.model = model
+        cfg = model.cfg
+        dev = model.lm_head.weight.device
+        self.dev = dev
+        self.caches = [(torch.zeros(cfg.kv_heads, cfg.max_len, cfg.head_dim, dtype=torch.float16, device=dev),
+                        torch.zeros(cfg.kv_heads, cfg.max_len, cfg.head_dim, dtype=torch.float16, device=dev))
+                       for _ in range(cfg.layers)]
+        self.cos, self.sin = model.rope_tables(dev)
+        self.tok = torch.zeros(1, dtype=torch.long, device=dev)
+        self.pos = torch.zeros(1, dtype=torch.long, device=dev)
+        self.next_tok = torch.zeros(1, dtype=torch.long, device=dev)
+        self.use_graph = use_graph
+        self.graph = None
+
+    @torch.no_grad()
+    def _step(self):
+        """One token: logits of `tok` at `pos`, greedy pick, then advance `tok` and `pos` on the device (so a
+        replayed graph needs no host-side update between tokens)."""
+        logits = self.model.forward_tokens(self.tok, self.pos, self.caches, self.cos, self.sin)
+        self.next_tok.copy_(logits.argmax(-1))
+        self.tok.copy_(self.next_tok)
+        self.pos.add_(1)
+
+    @torch.no_grad()
+    def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
+        T = prompt.numel()
+        pos = torch.arange(T, device=self.dev)
+        logits = self.model.forward_tokens(prompt.to(self.dev), pos, self.caches, self.cos, self.sin)
+        return logits[-1].argmax().reshape(1)
+
+    @torch.no_grad()
+    def capture(self):
+        """Captures `_step`.  Its warm-up and the capture pass itself write the KV cache at `pos`, which the caller
+        must treat as scratch (generate() points `pos` at the last cache slot meanwhile)."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._step()  # outside the capture: lazy initialisation, kernel attributes
+            torch.cuda.synchronize()
+            self.pos.sub_(1)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=side):
+                self._step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+
+    @torch.no_grad()
+    def generate(self, prompt: torch.Tensor, new_tokens: int):
+        """Returns (tokens [new_tokens] on the host, ttfb_s, decode_s): TTFB = prefill + first token,
+        decode_s = wall of the remaining new_tokens - 1 steps."""
+        cfg = self.model.cfg
+        if prompt.numel() + new_tokens > cfg.max_len - 1:
+            raise ValueError("prompt + new tokens exceed the KV cache (the last slot is kept as capture scratch)")
+        if self.use_graph and self.graph is None:
+            self.tok.zero_()
+            self.pos.fill_(cfg.max_len - 1)
+            self.capture()
+        out = torch.zeros(new_tokens, dtype=torch.long, device=self.dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        first = self.prefill(prompt)
+        out[0:1].copy_(first)
+        torch.cuda.synchronize()
+        ttfb = time.perf_counter() - t0
+        self.tok.copy_(first)
+        self.pos.fill_(prompt.numel())
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(1, new_tokens):
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self._step()
+            out[i:i + 1].copy_(self.next_tok)
+        torch.cuda.synchronize()
+        decode_s = time.perf_counter() - t1
+        return out.cpu(), ttfb, decode_s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--new", type=int, default=256)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-correction", action="store_true")
+    ap.add_argument("--vocab", type=int, default=128256)
+    args = ap.parse_args()
+    import os
+
+    os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    cfg = DecoderConfig(layers=args.layers, vocab=args.vocab, max_len=max(1024, args.prompt + args.new + 8))
+    t0 = time.perf_counter()
+    model, _, _ = build_decoder(cfg, with_correction=not args.no_correction)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    dec = GreedyDecoder(model, use_graph=not args.no_graph)
+    g = torch.Generator().manual_seed(3)
+    prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=g)
+    dec.generate(prompt, 4)  # warm-up (also captures the graph)
+    _, ttfb, decode_s = dec.generate(prompt, args.new)
+    print(json.dumps({
+        "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
+                    f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + ("" if args.no_correction else f" + GlowQ r={cfg.rank}"),
+        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph,
+        "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((args.new - 1) / decode_s, 1),
+        "ms_per_token": round(decode_s * 1e3 / (args.new - 1), 3), "build_s": round(build_s, 1)}))
+
+
+if __name__ == "__main__":
+    main()
