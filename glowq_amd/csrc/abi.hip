@@ -1,5 +1,6 @@
 // C ABI of the library: argument validation, route selection, launches.  No torch types, no
 // allocation, no synchronisation; see include/glowq_w4a16.h for the contract of each entry point.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -13,6 +14,9 @@ hipError_t launch_wave_dot(GroupDev& g, int rows_per_task, int num_cus, hipStrea
 hipError_t launch_generic(GroupDev& g, int num_cus, hipStream_t stream);
 int wave_dot_rows(long total_rows);
 bool wave_dot_supported(int M, int K, int rank, bool has_r);
+// gemv_quad.hip
+int quad_capacity(int M, int K, int rank, bool has_r);
+hipError_t launch_quad(GroupDev& g, int num_cus, hipStream_t stream);
 // misc.hip
 hipError_t launch_dequant(const int32_t*, const half_t*, const int32_t*, half_t*, int, int, int, int, int, int, int,
                           hipStream_t);
@@ -53,13 +57,24 @@ int num_cus() {
   return cached[dev];
 }
 
-constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3;
+constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4;
 constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
 
-// rows up to which the wave-dot GEMV is preferred over the skinny MFMA kernel (tuning override: GLOWQ_WAVEDOT_M)
-int wave_dot_pref_m() {
-  static const int v = getenv("GLOWQ_WAVEDOT_M") ? atoi(getenv("GLOWQ_WAVEDOT_M")) : kWaveDotMaxM;
-  return v < 0 ? 0 : (v > kWaveDotMaxM ? kWaveDotMaxM : v);
+// Route limits, settable at run time (glowq_set_tuning) and initialised from the environment:
+//   wave_dot_max_m  rows up to which the wave-dot GEMV is preferred over the skinny MFMA kernel (GLOWQ_WAVEDOT_M)
+//   quad_max_m      rows up to which the 4x4x4 matrix-core GEMV is used; 0 switches it off (GLOWQ_QUAD_M)
+//   quad_min_m      rows from which it is used (GLOWQ_QUAD_MIN_M; a single row is faster on the wave-dot kernel)
+int env_or(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : fallback;
+}
+int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+std::atomic<int> g_wave_dot_max_m{clampi(env_or("GLOWQ_WAVEDOT_M", kWaveDotMaxM), 0, kWaveDotMaxM)};
+std::atomic<int> g_quad_max_m{clampi(env_or("GLOWQ_QUAD_M", 16), 0, 16)};
+std::atomic<int> g_quad_min_m{clampi(env_or("GLOWQ_QUAD_MIN_M", 2), 1, 16)};
+int wave_dot_pref_m() { return g_wave_dot_max_m.load(std::memory_order_relaxed); }
+bool quad_wanted(int M) {
+  return M >= g_quad_min_m.load(std::memory_order_relaxed) && M <= g_quad_max_m.load(std::memory_order_relaxed);
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -121,6 +136,12 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
+  if (quad_wanted(g.M) && force != kRouteSkinny && quad_capacity(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr) > 0) {
+    bool ok = true;
+    for (int i = 0; i < g.n_members; ++i)  // 16-byte L rows; 32-bit byte offsets inside every buffer of a member
+      ok = ok && (g.mem[i].L == nullptr || aligned16(g.mem[i].L)) && (long)g.mem[i].N * g.mem[i].ldw * 4 < (1L << 31);
+    if (ok) return kRouteQuad;
+  }
   if (g.M <= wave_dot_pref_m() && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
     return kRouteWaveDot;
   if (skinny_supported(g)) return kRouteSkinny;
@@ -149,7 +170,8 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   } else if (route == kRouteSkinny) {
     e = launch_skinny(g, cus, stream);
   } else {
-    const int cap = (route == kRouteWaveDot) ? kWaveDotMaxM : 65535;
+    const int cap = (route == kRouteWaveDot) ? kWaveDotMaxM
+                    : (route == kRouteQuad) ? quad_capacity(g.M, g.K, g.rank, g.r != nullptr) : 65535;
     long rows = 0;
     for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
     const int M = g.M;
@@ -162,7 +184,9 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
       g.x = x0 + (size_t)m0 * g.K;
       g.r = r0 ? r0 + (size_t)m0 * g.rank : nullptr;
       for (int i = 0; i < g.n_members; ++i) g.mem[i].y = y0[i] + (size_t)m0 * g.mem[i].ldy;
-      e = (route == kRouteWaveDot) ? launch_wave_dot(g, wave_dot_rows(rows), cus, stream) : launch_generic(g, cus, stream);
+      e = (route == kRouteWaveDot) ? launch_wave_dot(g, wave_dot_rows(rows), cus, stream)
+          : (route == kRouteQuad)  ? launch_quad(g, cus, stream)
+                                   : launch_generic(g, cus, stream);
     }
   }
   if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
@@ -335,4 +359,16 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
   return pick_route(g, -1);
 }
 
+
+int glowq_set_tuning(const char* key, int value) {
+  if (key == nullptr) return fail(GLOWQ_EINVAL, "tuning key must not be NULL");
+  std::atomic<int>* slot = nullptr;
+  int lo = 0, hi = 16;
+  if (strcmp(key, "wave_dot_max_m") == 0) { slot = &g_wave_dot_max_m; hi = kWaveDotMaxM; }
+  else if (strcmp(key, "quad_max_m") == 0) { slot = &g_quad_max_m; }
+  else if (strcmp(key, "quad_min_m") == 0) { slot = &g_quad_min_m; lo = 1; }
+  if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
+  if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
+  return slot->exchange(value);
+}
 }  // extern "C"

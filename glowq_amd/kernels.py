@@ -50,6 +50,7 @@ _SIGNATURES = {
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
+    "glowq_set_tuning": (_I, [ctypes.c_char_p, _I]),
 }
 
 
@@ -240,8 +241,15 @@ class W4A16Extension:
         return result
 
     def route(self, M: int, K: int, N: int, group_size: int = 128) -> str:
-        names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic"}
+        names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv"}
         return names[self.lib.glowq_w4a16_route(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
+
+    def set_tuning(self, key: str, value: int) -> int:
+        """Sets a route limit of the process ("quad_max_m", "quad_min_m", "wave_dot_max_m"); returns the old value."""
+        old = self.lib.glowq_set_tuning(key.encode(), int(value))
+        if old < 0:
+            raise ValueError(self.lib.glowq_last_error().decode())
+        return old
 
 
 def library_path() -> str:

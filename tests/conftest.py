@@ -25,3 +25,14 @@ def golden():
     import numpy as np
 
     return np.load(os.path.join(ROOT, "tests", "golden", "w4a16_golden.npz"))
+
+
+@pytest.fixture(params=["quad", "classic"])
+def small_m_route(request, ext):
+    """Runs a test once with the 4x4x4 matrix-core GEMV serving 1..16 token rows and once with it switched
+    off (wave-dot GEMV for 1..4 rows, skinny MFMA kernel above)."""
+    old = ext.set_tuning("quad_max_m", 16 if request.param == "quad" else 0)
+    old_min = ext.set_tuning("quad_min_m", 1)
+    yield request.param
+    ext.set_tuning("quad_max_m", old)
+    ext.set_tuning("quad_min_m", old_min)

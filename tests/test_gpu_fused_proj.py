@@ -38,11 +38,11 @@ def run_cases(ext, repeats=2):
                 assert_close(y.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"fused member {i}")
 
 
-def test_fused_projection_matches_oracle(ext):
+def test_fused_projection_matches_oracle(ext, small_m_route):
     run_cases(ext)
 
 
-def test_fused_equals_two_launch_form(ext):
+def test_fused_equals_two_launch_form(ext, small_m_route):
     M, K, Ns, rank = 1, 4096, [1024, 256, 256], 128
     x, members, R = make_group(91, M, K, Ns, rank)
     mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]), "L": dev(m["L"])} for m in members]

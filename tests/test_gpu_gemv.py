@@ -21,7 +21,7 @@ def _run_single(ext, x, m, gs=128, entry="gemv"):
     (1, 2048, 2048, 128), (1, 4096, 1024, 128), (2, 4096, 512, 128), (3, 1024, 300, 128), (4, 5120, 256, 128),
     (1, 14336, 128, 128), (1, 3584, 130, 128), (1, 4096, 4096, 128), (1, 256, 7, 64), (1, 512, 33, 32),
 ])
-def test_gemv_matches_oracle(ext, M, K, N, gs):
+def test_gemv_matches_oracle(ext, small_m_route, M, K, N, gs):
     print(f"case M={M} K={K} N={N} gs={gs}", flush=True)
     x, (m,), _ = make_group(7 + M + K + N, M, K, [N], 0, group_size=gs)
     got = _run_single(ext, x, m, gs)
@@ -41,7 +41,7 @@ def test_generic_route_odd_shapes(ext, M, K, N, gs):
     assert_close(got, want, f"generic M={M} K={K} N={N}")
 
 
-def test_one_hot_input_selects_dequantised_column(ext):
+def test_one_hot_input_selects_dequantised_column(ext, small_m_route):
     """x = e_k makes y[n] = (code - z) * s for column k: every nibble position, exactly (fp16 of an
     exactly representable product of a 5-bit integer and an fp16 is exact when it fits 11 bits)."""
     K, N, gs = 256, 64, 128
@@ -64,7 +64,7 @@ def test_dequant_and_unpack_exact(ext):
         np.testing.assert_array_equal(codes, oracle.unpack_int4_i32(m["qweight"], K))
 
 
-def test_golden_module_vectors(ext, golden):
+def test_golden_module_vectors(ext, small_m_route, golden):
     """The reference's own dequantised weights and CPU forward outputs (tests/golden)."""
     for name in ("m1", "m2"):
         gs = int(golden[f"{name}_gs"][0])
@@ -80,7 +80,7 @@ def test_golden_module_vectors(ext, golden):
         assert np.all(np.abs(y - want) <= 1e-2 + 1e-3 * np.abs(want))
 
 
-def test_group_forward_with_correction(ext):
+def test_group_forward_with_correction(ext, small_m_route):
     for (M, K, Ns, rank, alpha) in [(1, 2048, [256, 128, 128], 64, 1.0), (2, 4096, [512, 96], 128, 0.5),
                                     (1, 4096, [300], 256, 1.0), (4, 1024, [64, 64, 64, 64], 32, 2.0),
                                     (1, 1024, [128, 64], 37, 1.0)]:
@@ -100,7 +100,7 @@ def test_group_forward_with_correction(ext):
             assert_close(y.cpu().numpy(), want, f"group K={K} rank={rank}")
 
 
-def test_selective_members_skip_correction(ext):
+def test_selective_members_skip_correction(ext, small_m_route):
     """GlowQ-S: a member without L gets exactly the uncorrected result, the others the corrected one."""
     M, K, Ns, rank = 1, 2048, [128, 64, 192], 64
     x, members, R = make_group(5, M, K, Ns, rank)

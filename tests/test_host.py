@@ -293,7 +293,14 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.glowq_w4a16_group_forward(one, None, None, 0, 1, 64, 32, 0, 1.0, None) == -1
     assert lib.glowq_shared_proj(one, one, one, 0, 64, 8, None) == -1
     assert lib.glowq_w4a16_dequant(one, one, one, one, 4, 64, 32, 8, 2, 0, None) == -2
-    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(2048, 3584, 3584) == "tiled_mfma_gemm"
+    assert ext.route(2048, 3584, 3584) == "tiled_mfma_gemm"
+    old = ext.set_tuning("quad_max_m", 0)
+    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096) == "skinny_mfma"
+    ext.set_tuning("quad_max_m", 16)
+    assert ext.route(8, 4096, 4096) == "quad_mfma_gemv"
+    ext.set_tuning("quad_max_m", old)
+    with pytest.raises(ValueError):
+        ext.set_tuning("no_such_key", 1)
     assert ext.route(1, 100, 8) == "generic"
 
 
