@@ -10,9 +10,12 @@
 // apart; the zero-point is folded through per-unit activation sums, sum (c - z) s x = s (sum c x - z sum x).
 //
 // Work decomposition: a row block is 4 consecutive output rows of one member; a step is 2048 columns of a
-// row block, loaded as 4 x (16 lanes x 16 bytes) per row: lane (b, q) reads unit 16c + b of row n0 + q in
-// load c, so every row is covered 1 KB contiguous per step.  A wave owns whole row blocks; partial sums
-// never leave the wave.  The correction rides along as a K-extension with the rows of L as fp16 B operands.
+// row block.  Memory is read in the order it lies: in load c lane 16r + i reads unit 16c + i of row n0 + r
+// (16 consecutive lanes = 256 contiguous bytes), and the same lanes fetch the scale and zero-point of the
+// groups of that step, once.  The matrix core wants block b = unit, column q = row, i.e. lane 4b + q: the
+// 4 x 16 -> 16 x 4 lane transposition is done with ds_bpermute on the way into the B operand.  A wave owns
+// whole row blocks (or a K-slice of one, see `slices`).  The correction rides along as a K-extension with
+// the rows of L as fp16 B operands.
 #include <cstdlib>
 
 #include "common.hpp"
@@ -78,13 +81,19 @@ __device__ __forceinline__ void stage_quad(const GroupDev& g, const QuadLds& l, 
   }
 }
 
-template <int kLW>
+// kWide: a step holds at most 16 quantisation groups per row (group_size >= 128), so one scale and one
+// zero-point load per lane and step cover them; otherwise every 16-byte unit brings its own.
+template <int kLW, bool kWide>
 struct QuadPrefetch {
   u32x4 w[4];
-  half_t sc[4];
-  uint32_t zw[4];
+  half_t sc[kWide ? 1 : 4];
+  uint32_t zw[kWide ? 1 : 4];
   uint32_t l[kLW > 0 ? kLW : 1];
 };
+
+__device__ __forceinline__ uint32_t lane_fetch(int src_lane_bytes, uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_bytes, (int)v);
+}
 
 // sum over the 16 lanes that share lane % 4; every lane gets the total of its class
 __device__ __forceinline__ float quad_class_sum(float v, int lane) {
@@ -106,7 +115,7 @@ __device__ __forceinline__ float quad_class_sum(float v, int lane) {
 // `slices` waves of a workgroup share one row block, each taking a contiguous range of its `kit` steps; their
 // partial sums meet in LDS (one barrier per row block).  With slices == 1 a wave owns whole row blocks and the
 // only barrier is the one after staging.
-template <int kM, int kLW>
+template <int kM, int kLW, bool kWide>
 __global__ __launch_bounds__(kM > 8 ? 512 : 1024) __attribute__((amdgpu_waves_per_eu((kM > 8 ? 2 : 4), 8)))
 void gemv_quad_kernel(const GroupDev g, const int kit, const int slices) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -156,11 +165,14 @@ void gemv_quad_kernel(const GroupDev g, const int kit, const int slices) {
   struct Cursor {
     int blk, it;
   };
-  auto issue = [&](const Cursor& c, QuadPrefetch<kLW>& p) {
+  const int lr = lane >> 4, lu = lane & 15;  // row and unit-in-load this lane reads from memory
+  const int fetch_w = (16 * qj + qb) << 2;    // byte address of the lane that read (row qj, unit qb)
+  const int gps_shift = 6 - upg_shift;        // log2 of the groups per row and step
+  auto issue = [&](const Cursor& c, QuadPrefetch<kLW, kWide>& p) {
     // A cursor past the end still issues its loads (the pipeline has one static shape), but every lane then
     // reads the first 16 bytes of x: one cached request per load instead of a second pass over a row block.
     const bool valid = c.blk < total_blocks;
-    const uint32_t n = (uint32_t)min(c.blk * kQuadRows + qj, mem.N - 1);
+    const uint32_t n = (uint32_t)min(c.blk * kQuadRows + lr, mem.N - 1);
     const uint32_t w_row = valid ? n * (uint32_t)mem.ldw * 4u : 0u, s_row = valid ? n * (uint32_t)mem.lds * 2u : 0u,
                    z_row = valid ? n * (uint32_t)mem.ldz * 4u : 0u;
     const char* wb = valid ? wbase : reinterpret_cast<const char*>(g.x);
@@ -168,15 +180,23 @@ void gemv_quad_kernel(const GroupDev g, const int kit, const int slices) {
     const char* zb = valid ? zbase : reinterpret_cast<const char*>(g.x);
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc) {
-      const uint32_t u = valid ? (uint32_t)min(c.it * kWave + cc * 16 + qb, U - 1) : 0u;
-      const uint32_t grp = u >> upg_shift;
+      const uint32_t u = valid ? (uint32_t)min(c.it * kWave + cc * 16 + lu, U - 1) : 0u;
       p.w[cc] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wb + (w_row + u * 16u)));
-      p.sc[cc] = *reinterpret_cast<const half_t*>(sb + (s_row + grp * 2u));
-      p.zw[cc] = *reinterpret_cast<const uint32_t*>(zb + (z_row + (grp >> 3) * 4u));
+      if constexpr (!kWide) {
+        const uint32_t grp = u >> upg_shift;
+        p.sc[cc] = *reinterpret_cast<const half_t*>(sb + (s_row + grp * 2u));
+        p.zw[cc] = *reinterpret_cast<const uint32_t*>(zb + (z_row + (grp >> 3) * 4u));
+      }
+    }
+    if constexpr (kWide) {
+      const uint32_t grp = valid ? (uint32_t)min((c.it << gps_shift) + lu, (U - 1) >> upg_shift) : 0u;
+      p.sc[0] = *reinterpret_cast<const half_t*>(sb + (s_row + grp * 2u));
+      p.zw[0] = *reinterpret_cast<const uint32_t*>(zb + (z_row + (grp >> 3) * 4u));
     }
     if constexpr (kLW > 0) {
+      const uint32_t nq = (uint32_t)min(c.blk * kQuadRows + qj, mem.N - 1);
       const uint32_t q = valid ? (uint32_t)min(c.it * 16 + qb, l_chunks - 1) : 0u;
-      const char* lp = (valid ? lbase : reinterpret_cast<const char*>(g.x)) + ((valid ? n * l_row_bytes : 0u) + q * (4u * kLW));
+      const char* lp = (valid ? lbase : reinterpret_cast<const char*>(g.x)) + ((valid ? nq * l_row_bytes : 0u) + q * (4u * kLW));
       if constexpr (kLW == 2) {
         const u32x2 v = *reinterpret_cast<const u32x2*>(lp);
         p.l[0] = v.x; p.l[1] = v.y;
@@ -201,19 +221,37 @@ void gemv_quad_kernel(const GroupDev g, const int kit, const int slices) {
   }
   int parity = 0;
 
-  auto compute = [&](const Cursor& c, const QuadPrefetch<kLW>& p) {
+  auto compute = [&](const Cursor& c, const QuadPrefetch<kLW, kWide>& p) {
+    // scale bits and zero-point of the group(s) this lane loaded, packed for the lane exchange
+    uint32_t side[kWide ? 1 : 4];
+    if constexpr (kWide) {
+      const int grp = min((c.it << gps_shift) + lu, (U - 1) >> upg_shift);
+      side[0] = (uint32_t)__builtin_bit_cast(uint16_t, p.sc[0]) | (nibble(p.zw[0], grp & 7) << 16);
+    } else {
+#pragma unroll
+      for (int cc = 0; cc < 4; ++cc) {
+        const int grp = min(c.it * kWave + cc * 16 + lu, U - 1) >> upg_shift;
+        side[cc] = (uint32_t)__builtin_bit_cast(uint16_t, p.sc[cc]) | (nibble(p.zw[cc], grp & 7) << 16);
+      }
+    }
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc) {
       const int uraw = c.it * kWave + cc * 16 + qb;
       const bool active = uraw < U;
       const int u = active ? uraw : U - 1;
-      const int grp = u >> upg_shift;
-      const float sc = active ? (float)p.sc[cc] : 0.f;
-      const float zp = (float)nibble(p.zw[cc], grp & 7);
+      uint32_t sv;
+      if constexpr (kWide) {
+        const int grel = (u >> upg_shift) - (c.it << gps_shift);  // group of this unit within the step
+        sv = lane_fetch((16 * qj + grel) << 2, side[0]);
+      } else {
+        sv = lane_fetch(fetch_w, side[cc]);
+      }
+      const float sc = active ? (float)__builtin_bit_cast(half_t, (uint16_t)(sv & 0xFFFFu)) : 0.f;
+      const float zp = (float)(sv >> 16);
       h4 b_lo[4], b_hi[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const uint32_t w = p.w[cc][t];
+        const uint32_t w = lane_fetch(fetch_w, p.w[cc][t]);
         const uint32_t hi = w >> 8;
         b_lo[t] = __builtin_bit_cast(h4, u32x2{w & 0x000F000Fu, hi & 0x000F000Fu});  // codes 0,4,2,6 * 2^-24
         b_hi[t] = __builtin_bit_cast(h4, u32x2{w & 0x00F000F0u, hi & 0x00F000F0u});  // codes 1,5,3,7 * 2^-20
@@ -314,7 +352,7 @@ void gemv_quad_kernel(const GroupDev g, const int kit, const int slices) {
   Cursor ahead;
   ahead.blk = first_blk + local_blk;
   ahead.it = it_begin;
-  QuadPrefetch<kLW> buf0, buf1;
+  QuadPrefetch<kLW, kWide> buf0, buf1;
   issue(ahead, buf0);
 
   stage_quad<kM>(g, lay, xs, sig, rs);
@@ -356,9 +394,9 @@ bool quad_supported(int M, int K, int rank, bool has_r) {
   return quad_lds(quad_tokens(M), K, has_r ? rank : 0).total + 8192 <= 160 * 1024;
 }
 
-template <int kM, int kLW>
+template <int kM, int kLW, bool kWide>
 static hipError_t launch_quad_t(const GroupDev& g, int kit, int num_cus, size_t lds_base, hipStream_t stream) {
-  auto kern = gemv_quad_kernel<kM, kLW>;
+  auto kern = gemv_quad_kernel<kM, kLW, kWide>;
   // 16 waves per CU (8 for the widest token count), in as many workgroups as the LDS footprint allows
   static const int waves_env = quad_env("GLOWQ_QUAD_WAVES", 0);
   static const int wg_env = quad_env("GLOWQ_QUAD_WG_PER_CU", 0);
@@ -423,8 +461,11 @@ hipError_t launch_quad(GroupDev& g, int num_cus, hipStream_t stream) {
   const int lw = has_r ? quad_lw(g.rank, kit) : 0;
   const int tokens = quad_tokens(g.M);
   const size_t lds = quad_lds(tokens, g.K, has_r ? g.rank : 0).total;
-#define GLOWQ_CASE(MM, LL) \
-  if (tokens == MM && lw == LL) return launch_quad_t<MM, LL>(g, kit, num_cus, lds, stream);
+  const bool wide = g.group_size >= 128;
+#define GLOWQ_CASE(MM, LL)                                                                        \
+  if (tokens == MM && lw == LL)                                                                   \
+    return wide ? launch_quad_t<MM, LL, true>(g, kit, num_cus, lds, stream)                       \
+                : launch_quad_t<MM, LL, false>(g, kit, num_cus, lds, stream);
 #define GLOWQ_CASES(MM) GLOWQ_CASE(MM, 0) GLOWQ_CASE(MM, 2) GLOWQ_CASE(MM, 4)
   GLOWQ_CASES(1) GLOWQ_CASES(2) GLOWQ_CASES(4) GLOWQ_CASES(8) GLOWQ_CASES(16)
 #undef GLOWQ_CASES
