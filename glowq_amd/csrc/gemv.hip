@@ -76,11 +76,14 @@ __device__ __forceinline__ void dot_word(uint32_t w, const h8& xq, float& accA, 
 // What a wave loads for one row block, all of it issued before anything is used: per row one
 // 16-byte unit of 32 int4 codes, the raw scale and zero-point word of the unit's quantisation group,
 // and kLW dwords (two halves each) of the row of the left factor L.
-template <int kRows, int kLW>
+// kWide: a step holds at most 16 quantisation groups per row (group_size >= 128); then lane 16r + i loads the
+// scale and zero-point of group i of row r once per step and the lanes that need it fetch it with ds_bpermute,
+// instead of every lane loading its own copy for every row.
+template <int kRows, int kLW, bool kWide>
 struct Prefetch {
   u32x4 w[kRows];
-  half_t sc[kRows];
-  uint32_t zw[kRows];
+  half_t sc[kWide ? 1 : kRows];
+  uint32_t zw[kWide ? 1 : kRows];
   uint32_t l[kRows][kLW > 0 ? kLW : 1];
 };
 
@@ -94,7 +97,7 @@ struct Prefetch {
 // Every workgroup serves ONE member for its whole life (the host splits the grid between the members in
 // proportion to their row blocks), so the member's pointers and strides are loop invariants held in
 // scalar registers and nothing is looked up in memory between two prefetches.
-template <int kM, int kRows, int kLW>
+template <int kM, int kRows, int kLW, bool kWide>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(((kM >= 2 || kRows >= 4) ? 4 : 6), 8)))
 void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -132,7 +135,9 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   struct Cursor {
     int blk, it;
   };
-  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW>& p) {
+  const int side_row = min(lane >> 4, kRows - 1), side_idx = lane & 15;
+  const int gps_shift = 6 - upg_shift;  // log2 of the groups per row and step
+  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kWide>& p) {
     const int n0 = min(c.blk, total_blocks - 1) * kRows;
     const int u = min(lane + c.it * kWave, U - 1);
     const int grp = u >> upg_shift;
@@ -140,8 +145,10 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
     for (int r = 0; r < kRows; ++r) {
       const int n = min(n0 + r, mem.N - 1);
       p.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw) + u);
-      p.sc[r] = mem.scales[(size_t)n * mem.lds + grp];
-      p.zw[r] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (grp >> 3)];
+      if constexpr (!kWide) {
+        p.sc[r] = mem.scales[(size_t)n * mem.lds + grp];
+        p.zw[r] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (grp >> 3)];
+      }
       if constexpr (kLW > 0) {
         // a member without L reads r itself (valid memory) and is weighted by zero
         const uint32_t* lrow = mem.L ? reinterpret_cast<const uint32_t*>(mem.L + (size_t)n * g.rank)
@@ -149,6 +156,12 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
 #pragma unroll
         for (int j = 0; j < kLW; ++j) p.l[r][j] = lrow[min((c.it * kLW + j) * kWave + lane, ldw_half - 1)];
       }
+    }
+    if constexpr (kWide) {
+      const int n = min(n0 + side_row, mem.N - 1);
+      const int sg = min((c.it << gps_shift) + side_idx, (U - 1) >> upg_shift);
+      p.sc[0] = mem.scales[(size_t)n * mem.lds + sg];
+      p.zw[0] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (sg >> 3)];
     }
   };
   auto advance = [&](Cursor& c) {
@@ -164,16 +177,28 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
 #pragma unroll
     for (int m = 0; m < kM; ++m) tot[r][m] = 0.f;
 
-  auto compute = [&](const Cursor& c, const Prefetch<kRows, kLW>& p) {
+  auto compute = [&](const Cursor& c, const Prefetch<kRows, kLW, kWide>& p) {
     const int uraw = lane + c.it * kWave;
     const bool active = uraw < U;
     const int u = active ? uraw : U - 1;
     const int grp = u >> upg_shift;
     float sc[kRows], zp[kRows];
+    if constexpr (kWide) {
+      const int sg = min((c.it << gps_shift) + side_idx, (U - 1) >> upg_shift);
+      const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, p.sc[0]) | (nibble(p.zw[0], sg & 7) << 16);
+      const int grel = grp - (c.it << gps_shift);
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      sc[r] = active ? (float)p.sc[r] : 0.f;
-      zp[r] = (float)nibble(p.zw[r], grp & 7);
+      for (int r = 0; r < kRows; ++r) {
+        const uint32_t sv = (uint32_t)__builtin_amdgcn_ds_bpermute((16 * r + grel) << 2, (int)packed);
+        sc[r] = active ? (float)__builtin_bit_cast(half_t, (uint16_t)(sv & 0xFFFFu)) : 0.f;
+        zp[r] = (float)(sv >> 16);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        sc[r] = active ? (float)p.sc[r] : 0.f;
+        zp[r] = (float)nibble(p.zw[r], grp & 7);
+      }
     }
 #pragma unroll
     for (int m = 0; m < kM; ++m) {
@@ -209,19 +234,20 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
       }
     }
     if (c.it == kit - 1) {
-      const int n0 = c.blk * kRows;
+      // lane r keeps the total of row r: one store (and one bias load) per token row instead of one per output
+      const int n = c.blk * kRows + lane;
+      const bool writer = lane < kRows && n < mem.N;
+      const float b = (writer && mem.bias) ? (float)mem.bias[n] : 0.f;
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) {
+      for (int m = 0; m < kM; ++m) {
+        float mine = 0.f;
 #pragma unroll
-        for (int m = 0; m < kM; ++m) {
+        for (int r = 0; r < kRows; ++r) {
           const float v = wave_sum(tot[r][m]);
           tot[r][m] = 0.f;
-          const int n = n0 + r;
-          if (lane == 0 && n < mem.N) {
-            const float b = mem.bias ? (float)mem.bias[n] : 0.f;
-            mem.y[(size_t)m * mem.ldy + n] = (half_t)(__builtin_fmaf(v, 0x1p24f, b));
-          }
+          mine = lane == r ? v : mine;
         }
+        if (writer) mem.y[(size_t)m * mem.ldy + n] = (half_t)(__builtin_fmaf(mine, 0x1p24f, b));
       }
     }
   };
@@ -231,7 +257,7 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   Cursor ahead;
   ahead.blk = ((int)blockIdx.x - wg_begin) * waves_per_block + wave;
   ahead.it = 0;
-  Prefetch<kRows, kLW> buf0, buf1;
+  Prefetch<kRows, kLW, kWide> buf0, buf1;
   issue(ahead, buf0);
 
   stage_activations<kM>(g, U, xs, sig, rs);
@@ -317,10 +343,10 @@ static const WaveDotTuning& tuning_override() {
   return t;
 }
 
-template <int kM, int kRows, int kLW>
+template <int kM, int kRows, int kLW, bool kWide>
 static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int max_wg_per_cu, int num_cus, size_t lds,
                                     hipStream_t stream) {
-  auto kern = gemv_wave_dot_kernel<kM, kRows, kLW>;
+  auto kern = gemv_wave_dot_kernel<kM, kRows, kLW, kWide>;
   const int threads = waves * kWave;
   static size_t configured = 48 * 1024;  // largest dynamic LDS size this instantiation was raised to
   if (lds > configured) {
@@ -393,9 +419,12 @@ hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStre
   int waves = tuning_override().waves;
   if (waves < 1 || waves > 16) waves = 8;
   const int max_wg = tuning_override().max_wg_per_cu;
-#define GLOWQ_CASE(MM, RR, LL) \
-  if (g.M == MM && rows_per_block == RR && lw == LL) \
-    return launch_wave_dot_t<MM, RR, LL>(g, kit, waves, max_wg, num_cus, lds, stream);
+  // the shared scale / zero-point loads pay for single-row decode; the multi-row instantiations keep per-lane loads
+  const bool wide = g.M == 1 && g.group_size >= 128;
+#define GLOWQ_CASE(MM, RR, LL)                                                                   \
+  if (g.M == MM && rows_per_block == RR && lw == LL)                                             \
+    return (MM == 1 && wide) ? launch_wave_dot_t<MM, RR, LL, (MM == 1)>(g, kit, waves, max_wg, num_cus, lds, stream) \
+                             : launch_wave_dot_t<MM, RR, LL, false>(g, kit, waves, max_wg, num_cus, lds, stream);
 #define GLOWQ_CASES(MM, RR) GLOWQ_CASE(MM, RR, 0) GLOWQ_CASE(MM, RR, 1) GLOWQ_CASE(MM, RR, 2)
   GLOWQ_CASES(1, 1) GLOWQ_CASES(1, 2) GLOWQ_CASES(1, 4)
   GLOWQ_CASES(2, 1) GLOWQ_CASES(2, 2)
