@@ -36,6 +36,9 @@ namespace {
 
 thread_local char g_err[512] = "";
 
+}  // namespace
+
+namespace glowq {
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -56,6 +59,9 @@ int num_cus() {
   }
   return cached[dev];
 }
+}  // namespace glowq
+
+namespace {
 
 constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4;
 constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel

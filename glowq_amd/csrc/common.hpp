@@ -44,6 +44,11 @@ struct GroupDev {
   float alpha;
 };
 
+// Records the calling thread's error message (returned by glowq_last_error) and hands back `code`.
+int fail(int code, const char* fmt, ...);
+// Compute units of the current device (cached).
+int num_cus();
+
 __device__ __forceinline__ uint32_t nibble(uint32_t word, int idx) { return (word >> (4 * idx)) & 0xFu; }
 
 template <typename T>

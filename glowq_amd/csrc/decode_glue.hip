@@ -1,0 +1,337 @@
+// The operations of a Llama-style decoder layer that sit between the quantised linears, for single-token
+// decode: residual add + RMSNorm, rotary embedding + KV-cache append + attention of one query token over the
+// cache, SwiGLU gating, greedy pick.  Plain HBM/L2-latency-bound kernels; they exist so that a decode step is
+// a short chain of launches that a HIP graph can replay, not to be clever.
+#include "common.hpp"
+
+namespace glowq {
+
+namespace {
+
+__device__ __forceinline__ float block_sum(float v, float* red, int nwaves) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  __syncthreads();  // red may still be read from a previous call
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nwaves; ++i) t += red[i];
+  return t;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red, int nwaves) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nwaves; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+}  // namespace
+
+// x[m] = fp16(x[m] + delta[m]) (when delta != nullptr), h[m] = fp16(x[m] * rsqrt(mean(x[m]^2) + eps) * w), one
+// workgroup per token row, statistics in fp32.
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(half_t* __restrict__ x, const half_t* __restrict__ delta,
+                                                            const half_t* __restrict__ w, half_t* __restrict__ h,
+                                                            int H, float eps) {
+  __shared__ float red[16];
+  half_t* xr = x + (size_t)blockIdx.x * H;
+  const half_t* dr = delta ? delta + (size_t)blockIdx.x * H : nullptr;
+  half_t* hr = h + (size_t)blockIdx.x * H;
+  const int nw = blockDim.x >> 6;
+  float ss = 0.f;
+  for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {  // H % 8 == 0
+    h8 v = *reinterpret_cast<const h8*>(xr + i);
+    if (dr) {
+      const h8 d = *reinterpret_cast<const h8*>(dr + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (half_t)((float)v[j] + (float)d[j]);
+      *reinterpret_cast<h8*>(xr + i) = v;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss = __builtin_fmaf((float)v[j], (float)v[j], ss);
+  }
+  const float inv = rsqrtf(block_sum(ss, red, nw) / (float)H + eps);
+  for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+    const h8 v = *reinterpret_cast<const h8*>(xr + i);  // own writes of the first pass
+    const h8 ww = *reinterpret_cast<const h8*>(w + i);
+    h8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = (half_t)((float)(half_t)((float)v[j] * inv) * (float)ww[j]);
+    *reinterpret_cast<h8*>(hr + i) = o;
+  }
+}
+
+// out = silu(gate) * up, elementwise, fp32 math.
+__global__ __launch_bounds__(256) void silu_mul_kernel(const half_t* __restrict__ gate, const half_t* __restrict__ up,
+                                                        half_t* __restrict__ out, long n8) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (long)gridDim.x * blockDim.x) {
+    const h8 g = reinterpret_cast<const h8*>(gate)[i];
+    const h8 u = reinterpret_cast<const h8*>(up)[i];
+    h8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float gf = (float)g[j];
+      o[j] = (half_t)((float)(half_t)(gf / (1.f + __expf(-gf))) * (float)u[j]);
+    }
+    reinterpret_cast<h8*>(out)[i] = o;
+  }
+}
+
+// One query token against the cache, one workgroup per query head.
+//   q [heads, d], k_new / v_new [kv_heads, d]: this token's projections (k, q not yet rotated)
+//   cos / sin [max_len, d] fp32 tables (second half repeats the first), *pos the token's position
+//   cache_k / cache_v [kv_heads, max_len, d] fp16: positions < pos are read; position pos is WRITTEN by the first
+//   head of each KV group and taken from registers by all, so no workgroup reads what another one writes.
+//   out [heads, d] fp16.
+// Scores in LDS (max_len floats), softmax over [0, pos], then P.V with lanes across the head dimension.
+__global__ __launch_bounds__(256) void rope_attend_kernel(const half_t* __restrict__ q, const half_t* __restrict__ k_new,
+                                                           const half_t* __restrict__ v_new, const float* __restrict__ cos_t,
+                                                           const float* __restrict__ sin_t, const long* __restrict__ pos_p,
+                                                           half_t* __restrict__ cache_k, half_t* __restrict__ cache_v,
+                                                           half_t* __restrict__ out, int heads, int kv_heads, int d,
+                                                           int max_len, float scale) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* qs = reinterpret_cast<float*>(smem_raw);            // [d] rotated query
+  float* kn = qs + d;                                        // [d] rotated key of this token
+  float* vn = kn + d;                                        // [d] value of this token
+  float* red = vn + d;                                       // [16]
+  float* acc_part = red + 16;                                // [waves][d]
+  float* sc = acc_part + (blockDim.x >> 6) * d;              // [max_len] scores / probabilities
+  const int head = blockIdx.x;
+  const int rep = heads / kv_heads;
+  const int kvh = head / rep;
+  const int pos = (int)*pos_p;
+  const int half_d = d >> 1;
+  const int nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+
+  // rotary embedding of q and k_new: out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i + d/2] cos + x[i] sin
+  for (int i = threadIdx.x; i < half_d; i += blockDim.x) {
+    // the tables are rounded to fp16 first, as a half-precision model's rotary embedding does
+    const float c = (float)(half_t)cos_t[(size_t)pos * d + i], s = (float)(half_t)sin_t[(size_t)pos * d + i];
+    const float q0 = (float)q[(size_t)head * d + i], q1 = (float)q[(size_t)head * d + i + half_d];
+    qs[i] = (float)(half_t)(q0 * c - q1 * s);
+    qs[i + half_d] = (float)(half_t)(q1 * c + q0 * s);
+    const float k0 = (float)k_new[(size_t)kvh * d + i], k1 = (float)k_new[(size_t)kvh * d + i + half_d];
+    const half_t r0 = (half_t)(k0 * c - k1 * s), r1 = (half_t)(k1 * c + k0 * s);
+    kn[i] = (float)r0;
+    kn[i + half_d] = (float)r1;
+    const half_t v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
+    vn[i] = (float)v0;
+    vn[i + half_d] = (float)v1;
+    if (head == kvh * rep) {
+      half_t* ck = cache_k + ((size_t)kvh * max_len + pos) * d;
+      half_t* cv = cache_v + ((size_t)kvh * max_len + pos) * d;
+      ck[i] = r0; ck[i + half_d] = r1;
+      cv[i] = v0; cv[i + half_d] = v1;
+    }
+  }
+  __syncthreads();
+
+  // scores: one position per thread, the key row read as 16-byte pieces
+  const half_t* kbase = cache_k + (size_t)kvh * max_len * d;
+  float mx = -INFINITY;
+  for (int p = threadIdx.x; p <= pos; p += blockDim.x) {
+    float dot = 0.f;
+    if (p == pos) {
+      for (int i = 0; i < d; ++i) dot = __builtin_fmaf(qs[i], kn[i], dot);
+    } else {
+      const h8* kr = reinterpret_cast<const h8*>(kbase + (size_t)p * d);
+      for (int i = 0; i < d / 8; ++i) {
+        const h8 kv = kr[i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qs[8 * i + j], (float)kv[j], dot);
+      }
+    }
+    dot *= scale;
+    sc[p] = dot;
+    mx = fmaxf(mx, dot);
+  }
+  mx = block_max(mx, red, nw);
+  float sum = 0.f;
+  for (int p = threadIdx.x; p <= pos; p += blockDim.x) {
+    const float e = __expf(sc[p] - mx);
+    sc[p] = e;
+    sum += e;
+  }
+  sum = block_sum(sum, red, nw);  // its barriers also publish sc[]
+  const float inv = 1.f / sum;
+
+  // P.V: lane l holds dimensions 2l, 2l+1; the waves take positions round robin, 4 rows in flight each
+  const half_t* vbase = cache_v + (size_t)kvh * max_len * d;
+  float a0 = 0.f, a1 = 0.f;
+  if (2 * lane < d) {
+    int p = wave;
+    for (; p + 3 * nw < pos; p += 4 * nw) {
+      h2 v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const h2*>(vbase + (size_t)(p + j * nw) * d + 2 * lane);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float pr = sc[p + j * nw];
+        a0 = __builtin_fmaf(pr, (float)v[j][0], a0);
+        a1 = __builtin_fmaf(pr, (float)v[j][1], a1);
+      }
+    }
+    for (; p < pos; p += nw) {
+      const h2 v = *reinterpret_cast<const h2*>(vbase + (size_t)p * d + 2 * lane);
+      const float pr = sc[p];
+      a0 = __builtin_fmaf(pr, (float)v[0], a0);
+      a1 = __builtin_fmaf(pr, (float)v[1], a1);
+    }
+    if (wave == 0) {  // this token's own value
+      const float pr = sc[pos];
+      a0 = __builtin_fmaf(pr, vn[2 * lane], a0);
+      a1 = __builtin_fmaf(pr, vn[2 * lane + 1], a1);
+    }
+    acc_part[wave * d + 2 * lane] = a0;
+    acc_part[wave * d + 2 * lane + 1] = a1;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float t = 0.f;
+    for (int w = 0; w < nw; ++w) t += acc_part[w * d + i];
+    out[(size_t)head * d + i] = (half_t)(t * inv);
+  }
+}
+
+// Index of the first maximum of an fp16 vector, one workgroup; then token <- index, position += 1.
+__global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __restrict__ logits, int n, long* __restrict__ next_tok,
+                                                               long* __restrict__ tok, long* __restrict__ pos) {
+  __shared__ float bv[16];
+  __shared__ int bi[16];
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = (float)logits[i];
+    if (v > best) {  // ascending i per thread: the first maximum wins
+      best = v;
+      idx = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) {
+    const float ov = __shfl_xor(best, o);
+    const int oi = __shfl_xor(idx, o);
+    if (ov > best || (ov == best && oi < idx)) {
+      best = ov;
+      idx = oi;
+    }
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    bv[wave] = best;
+    bi[wave] = idx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+      if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+        best = bv[w];
+        idx = bi[w];
+      }
+    *next_tok = idx;
+    if (tok) *tok = idx;
+    if (pos) *pos += 1;
+  }
+}
+
+// ---- launchers ------------------------------------------------------------------------------
+hipError_t launch_add_rmsnorm(half_t* x, const half_t* delta, const half_t* w, half_t* h, int M, int H, float eps,
+                              hipStream_t stream) {
+  int threads = ((H / 8 + 63) / 64) * 64;
+  if (threads > 1024) threads = 1024;
+  if (threads < 64) threads = 64;
+  hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(M), dim3(threads), 0, stream, x, delta, w, h, H, eps);
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const half_t* gate, const half_t* up, half_t* out, long n, int num_cus, hipStream_t stream) {
+  const long n8 = n / 8;
+  long blocks = (n8 + 255) / 256;
+  if (blocks > (long)num_cus * 8) blocks = (long)num_cus * 8;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, gate, up, out, n8);
+  return hipGetLastError();
+}
+
+size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 4 * d + max_len) * sizeof(float); }
+
+hipError_t launch_rope_attend(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
+                              const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
+                              int heads, int kv_heads, int d, int max_len, float scale, hipStream_t stream) {
+  const size_t lds = rope_attend_lds(d, max_len);
+  static size_t configured = 48 * 1024;
+  if (lds > configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rope_attend_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    configured = lds;
+  }
+  hipLaunchKernelGGL(rope_attend_kernel, dim3(heads), dim3(256), lds, stream, q, k_new, v_new, cos_t, sin_t, pos,
+                     cache_k, cache_v, out, heads, kv_heads, d, max_len, scale);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax_advance(const half_t* logits, int n, long* next_tok, long* tok, long* pos, hipStream_t stream) {
+  hipLaunchKernelGGL(argmax_advance_kernel, dim3(1), dim3(1024), 0, stream, logits, n, next_tok, tok, pos);
+  return hipGetLastError();
+}
+
+}  // namespace glowq
+
+using namespace glowq;
+
+extern "C" {
+
+int glowq_add_rmsnorm(void* x, const void* delta, const void* weight, void* h, int M, int H, float eps, void* stream) {
+  if (!x || !weight || !h) return fail(GLOWQ_EINVAL, "add_rmsnorm: x, weight and h must be device pointers");
+  if (M <= 0 || H <= 0 || (H & 7)) return fail(GLOWQ_EINVAL, "add_rmsnorm: M > 0 and H a positive multiple of 8 (got M=%d, H=%d)", M, H);
+  hipError_t e = launch_add_rmsnorm(static_cast<half_t*>(x), static_cast<const half_t*>(delta), static_cast<const half_t*>(weight),
+                                    static_cast<half_t*>(h), M, H, eps, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "add_rmsnorm launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_silu_mul(const void* gate, const void* up, void* out, long n, void* stream) {
+  if (!gate || !up || !out) return fail(GLOWQ_EINVAL, "silu_mul: gate, up and out must be device pointers");
+  if (n <= 0 || (n & 7)) return fail(GLOWQ_EINVAL, "silu_mul: n must be a positive multiple of 8 (got %ld)", n);
+  hipError_t e = launch_silu_mul(static_cast<const half_t*>(gate), static_cast<const half_t*>(up), static_cast<half_t*>(out), n,
+                                 num_cus(), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "silu_mul launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
+                      const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,
+                      int max_len, float scale, void* stream) {
+  if (!q || !k_new || !v_new || !cos_table || !sin_table || !pos || !cache_k || !cache_v || !out)
+    return fail(GLOWQ_EINVAL, "rope_attend: all pointers must be device pointers");
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || head_dim <= 0 || (head_dim & 7) || head_dim > 128 || max_len <= 0)
+    return fail(GLOWQ_EINVAL, "rope_attend: heads %% kv_heads == 0, head_dim a multiple of 8 up to 128 (got %d, %d, %d)", heads,
+                kv_heads, head_dim);
+  if (rope_attend_lds(head_dim, max_len) > 160 * 1024)
+    return fail(GLOWQ_EUNSUPPORTED, "rope_attend: max_len %d does not fit the score buffer in LDS", max_len);
+  hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),
+                                    cos_table, sin_table, reinterpret_cast<const long*>(pos), static_cast<half_t*>(cache_k),
+                                    static_cast<half_t*>(cache_v), static_cast<half_t*>(out), heads, kv_heads, head_dim, max_len, scale,
+                                    static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "rope_attend launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_argmax_advance(const void* logits, int n, int64_t* next_token, int64_t* token, int64_t* pos, void* stream) {
+  if (!logits || !next_token || n <= 0) return fail(GLOWQ_EINVAL, "argmax_advance: logits and next_token must be device pointers, n > 0");
+  hipError_t e = launch_argmax_advance(static_cast<const half_t*>(logits), n, reinterpret_cast<long*>(next_token),
+                                       reinterpret_cast<long*>(token), reinterpret_cast<long*>(pos), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "argmax_advance launch failed: %s", hipGetErrorString(e));
+}
+
+}  // extern "C"

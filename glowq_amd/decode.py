@@ -10,7 +10,10 @@ src/step2_rsvd.py:487-527 for the low-rank factors.
 
     python -m glowq_amd.decode --layers 32 --prompt 512 --new 256        # Llama-3.1-8B shape, batch 1
 
-Only the linears are this library's kernels; norms, RoPE, attention and the lm_head are plain torch ops.
+Two ways to run a token: the module path (`Decoder.forward_tokens`: the patched linears inside plain torch norms, RoPE
+and attention; used for prefill and as the yardstick) and `FusedStep` (single-token decode as a fixed chain of this
+library's launches: add+RMSNorm, group linears, RoPE+cache append+attention, SwiGLU gating, greedy pick; only the
+lm_head matmul and the embedding lookup stay torch ops).
 """
 from __future__ import annotations
 
@@ -25,7 +28,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .correction import patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
+from .correction import AddSVDCorrection, patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
+from .kernels import load_w4a16_extension
 from .linear import CudaW4A16Linear, convert_to_cuda_w4a16
 
 
@@ -207,10 +211,89 @@ def load_glowq_artifacts(shared_path: str, bmap_path: str, device="cuda"):
     return shared, bmap
 
 
+class FusedStep:
+    """One decode token as a fixed chain of launches on static buffers (13 per layer), ready for HIP-graph capture.
+    Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
+    the one-call projection + group entry point, o_proj and down_proj as solo groups."""
+
+    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok):
+        cfg = model.cfg
+        self.model, self.cfg = model, cfg
+        self.ext = load_w4a16_extension()
+        dev = model.lm_head.weight.device
+        self.caches, self.cos, self.sin = caches, cos, sin
+        self.tok, self.pos, self.next_tok = tok, pos, next_tok
+        f16 = dict(dtype=torch.float16, device=dev)
+        qd, kd = cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim
+        self.x = torch.zeros(1, cfg.hidden, **f16)
+        self.h = torch.zeros(1, cfg.hidden, **f16)
+        self.qkv = torch.zeros(1, qd + 2 * kd, **f16)
+        self.attn = torch.zeros(1, qd, **f16)
+        self.o = torch.zeros(1, cfg.hidden, **f16)
+        self.gu = torch.zeros(1, 2 * cfg.intermediate, **f16)
+        self.act = torch.zeros(1, cfg.intermediate, **f16)
+        self.dn = torch.zeros(1, cfg.hidden, **f16)
+        self.logits = torch.zeros(1, cfg.vocab, **f16)
+        self.scale = cfg.head_dim ** -0.5
+        self.plan = []
+        for layer in model.model.layers:
+            at, mlp = layer.self_attn, layer.mlp
+            self.plan.append({
+                "ln1": layer.input_layernorm, "ln2": layer.post_attention_layernorm,
+                "qkv": self._group([at.q_proj, at.k_proj, at.v_proj],
+                                   [self.qkv[:, :qd], self.qkv[:, qd:qd + kd], self.qkv[:, qd + kd:]], f16),
+                "o": self._group([at.o_proj], [self.o], f16),
+                "gu": self._group([mlp.gate_proj, mlp.up_proj],
+                                  [self.gu[:, :cfg.intermediate], self.gu[:, cfg.intermediate:]], f16),
+                "down": self._group([mlp.down_proj], [self.dn], f16),
+            })
+        self.q_view, self.k_view, self.v_view = self.qkv[0, :qd], self.qkv[0, qd:qd + kd], self.qkv[0, qd + kd:]
+
+    @staticmethod
+    def _group(mods, outs, f16):
+        members, R, alpha, gs = [], None, 1.0, None
+        for mod in mods:
+            inner = mod.inner if isinstance(mod, AddSVDCorrection) else mod
+            if not isinstance(inner, CudaW4A16Linear):
+                raise TypeError("FusedStep needs every projection converted to CudaW4A16Linear")
+            L = None
+            if isinstance(mod, AddSVDCorrection) and mod.alpha_svd != 0.0:
+                L, alpha = mod.A_q, float(mod.alpha_svd)
+                R = mod.B_q if R is None else R
+            gs = inner.group_size
+            members.append({"qweight": inner.qweight_i32, "scales": inner.scales_f16, "qzeros": inner.qzeros_i32, "L": L,
+                            "bias": inner.bias})
+        r = torch.zeros(1, R.size(0), **f16) if R is not None else None
+        return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs}
+
+    def _linear(self, x, grp):
+        self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"], R=grp["R"])
+
+    @torch.no_grad()
+    def run(self):
+        ext, cfg = self.ext, self.cfg
+        torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=self.x)
+        delta = None
+        for lay, (ck, cv) in zip(self.plan, self.caches):
+            ext.add_rmsnorm(self.x, delta, lay["ln1"].weight, self.h, lay["ln1"].eps)
+            self._linear(self.h, lay["qkv"])
+            ext.rope_attend(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.attn, self.scale)
+            self._linear(self.attn, lay["o"])
+            ext.add_rmsnorm(self.x, self.o, lay["ln2"].weight, self.h, lay["ln2"].eps)
+            self._linear(self.h, lay["gu"])
+            ext.silu_mul(self.gu[:, :cfg.intermediate], self.gu[:, cfg.intermediate:], self.act)
+            self._linear(self.act, lay["down"])
+            delta = self.dn
+        norm = self.model.model.norm
+        ext.add_rmsnorm(self.x, delta, norm.weight, self.h, norm.eps)
+        torch.mm(self.h, self.model.lm_head.weight.t(), out=self.logits)
+        ext.argmax_advance(self.logits, self.next_tok, self.tok, self.pos)
+
+
 class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
-    def __init__(self, model: Decoder, use_graph: bool = True):
+    def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False):
         self.model = model
         cfg = model.cfg
         dev = model.lm_head.weight.device
@@ -224,11 +307,15 @@ class GreedyDecoder:
         self.next_tok = torch.zeros(1, dtype=torch.long, device=dev)
         self.use_graph = use_graph
         self.graph = None
+        self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok) if fused else None
 
     @torch.no_grad()
     def _step(self):
         """One token: logits of `tok` at `pos`, greedy pick, then advance `tok` and `pos` on the device (so a
         replayed graph needs no host-side update between tokens)."""
+        if self.fused is not None:
+            self.fused.run()
+            return
         logits = self.model.forward_tokens(self.tok, self.pos, self.caches, self.cos, self.sin)
         self.next_tok.copy_(logits.argmax(-1))
         self.tok.copy_(self.next_tok)
@@ -296,6 +383,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new", type=int, default=256)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
     ap.add_argument("--vocab", type=int, default=128256)
     args = ap.parse_args()
@@ -307,7 +395,7 @@ def main():
     model, _, _ = build_decoder(cfg, with_correction=not args.no_correction)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=not args.no_graph)
+    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path)
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=g)
     dec.generate(prompt, 4)  # warm-up (also captures the graph)
@@ -315,7 +403,7 @@ def main():
     print(json.dumps({
         "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
                     f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + ("" if args.no_correction else f" + GlowQ r={cfg.rank}"),
-        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph,
+        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph, "fused_step": not args.module_path,
         "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((args.new - 1) / decode_s, 1),
         "ms_per_token": round(decode_s * 1e3 / (args.new - 1), 3), "build_s": round(build_s, 1)}))
 

@@ -51,6 +51,10 @@ _SIGNATURES = {
     "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
     "glowq_set_tuning": (_I, [ctypes.c_char_p, _I]),
+    "glowq_add_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
+    "glowq_silu_mul": (_I, [_P, _P, _P, ctypes.c_long, _P]),
+    "glowq_rope_attend": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_argmax_advance": (_I, [_P, _I, _P, _P, _P, _P]),
 }
 
 
@@ -239,6 +243,66 @@ class W4A16Extension:
         if rc:
             self._raise(rc, "w4a16_group_forward")
         return result
+
+    # ------------------------------------------------------------------ single-token decode step around the linears
+    @staticmethod
+    def _f16(t, what):
+        _check(t.is_cuda and t.dtype == torch.float16 and t.is_contiguous(), f"{what} must be a contiguous CUDA fp16 tensor")
+
+    def add_rmsnorm(self, x, delta, weight, h, eps: float) -> None:
+        """x += delta (delta may be None), h = rmsnorm(x) * weight; x and h are [M, H] fp16, x is updated in place."""
+        self._f16(x, "x"), self._f16(weight, "weight"), self._f16(h, "h")
+        _check(x.dim() == 2 and h.shape == x.shape and weight.numel() == x.size(1), "add_rmsnorm: x, h [M, H] and weight [H]")
+        if delta is not None:
+            self._f16(delta, "delta")
+            _check(delta.shape == x.shape, "add_rmsnorm: delta must have the shape of x")
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_add_rmsnorm(x.data_ptr(), delta.data_ptr() if delta is not None else None, weight.data_ptr(),
+                                            h.data_ptr(), x.size(0), x.size(1), float(eps), self._stream(x.device))
+        if rc:
+            self._raise(rc, "add_rmsnorm")
+
+    def silu_mul(self, gate, up, out) -> None:
+        for t, n in ((gate, "gate"), (up, "up"), (out, "out")):
+            _check(t.is_cuda and t.dtype == torch.float16 and t.stride(-1) == 1, f"silu_mul: {n} must be CUDA fp16")
+        _check(gate.numel() == up.numel() == out.numel(), "silu_mul: sizes differ")
+        _check(gate.is_contiguous() and up.is_contiguous() and out.is_contiguous(), "silu_mul: tensors must be contiguous")
+        with torch.cuda.device(out.device):
+            rc = self.lib.glowq_silu_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), self._stream(out.device))
+        if rc:
+            self._raise(rc, "silu_mul")
+
+    def rope_attend(self, q, k_new, v_new, cos_table, sin_table, pos, cache_k, cache_v, out, scale: float) -> None:
+        """q [heads, d], k_new / v_new [kv_heads, d] of one token, tables [max_len, d] fp32, pos int64[1] on the device,
+        caches [kv_heads, max_len, d]: rotary embedding, cache append at pos, attention over 0..pos into out [heads, d]."""
+        for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new"), (cache_k, "cache_k"), (cache_v, "cache_v"), (out, "out")):
+            self._f16(t, n)
+        _check(cos_table.is_cuda and cos_table.dtype == torch.float32 and cos_table.is_contiguous()
+               and sin_table.dtype == torch.float32 and sin_table.is_contiguous() and sin_table.shape == cos_table.shape,
+               "rope_attend: tables must be contiguous CUDA fp32 [max_len, d]")
+        _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "rope_attend: pos must be one int64 on the device")
+        kv_heads, max_len, d = cache_k.shape
+        heads = q.numel() // d
+        _check(cache_v.shape == cache_k.shape and k_new.numel() == kv_heads * d and v_new.numel() == kv_heads * d
+               and out.numel() == heads * d and tuple(cos_table.shape) == (max_len, d), "rope_attend: shape mismatch")
+        with torch.cuda.device(q.device):
+            rc = self.lib.glowq_rope_attend(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), cos_table.data_ptr(),
+                                            sin_table.data_ptr(), pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(),
+                                            out.data_ptr(), heads, kv_heads, d, max_len, float(scale), self._stream(q.device))
+        if rc:
+            self._raise(rc, "rope_attend")
+
+    def argmax_advance(self, logits, next_token, token=None, pos=None) -> None:
+        """next_token[0] = first argmax of logits; then token[0] = next_token[0] and pos[0] += 1 when given."""
+        self._f16(logits, "logits")
+        for t in (next_token, token, pos):
+            _check(t is None or (t.is_cuda and t.dtype == torch.int64 and t.numel() == 1), "argmax_advance: int64[1] on the device")
+        with torch.cuda.device(logits.device):
+            rc = self.lib.glowq_argmax_advance(logits.data_ptr(), logits.numel(), next_token.data_ptr(),
+                                               token.data_ptr() if token is not None else None,
+                                               pos.data_ptr() if pos is not None else None, self._stream(logits.device))
+        if rc:
+            self._raise(rc, "argmax_advance")
 
     def route(self, M: int, K: int, N: int, group_size: int = 128) -> str:
         names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv"}

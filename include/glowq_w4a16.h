@@ -136,6 +136,32 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  */
 int glowq_set_tuning(const char* key, int value);
 
+/*
+ * ---- single-token decode step around the linears --------------------------------------------------------
+ * The reference runs these through Hugging Face's LlamaDecoderLayer (transformers, not vendored; its generate()
+ * loop is what `measure_generation_metrics` times, src/step3_eval_dataset.py:705-798, and the manual KV-cache loop
+ * of test/step3_1_layerwise.py:181-210).  Here they are four launches per layer that a HIP graph can replay.
+ * All tensors fp16 unless typed otherwise; positions and tokens are int64 on the device.
+ */
+
+/* x[m] += delta[m] (skipped when delta is NULL), h[m] = rmsnorm(x[m]) * weight; x [M, H] is updated in place. */
+int glowq_add_rmsnorm(void* x, const void* delta, const void* weight, void* h, int M, int H, float eps, void* stream);
+
+/* out = silu(gate) * up over n elements (n % 8 == 0). */
+int glowq_silu_mul(const void* gate, const void* up, void* out, long n, void* stream);
+
+/*
+ * Rotary embedding of q [heads, d] and k_new [kv_heads, d] at position *pos (cos/sin tables [max_len, d] fp32),
+ * append of k / v_new to the caches [kv_heads, max_len, d] at *pos, attention of the one query token over positions
+ * 0..*pos, out [heads, d].  d <= 128, max_len limited by the LDS score buffer (about 40k positions).
+ */
+int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
+                      const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,
+                      int max_len, float scale, void* stream);
+
+/* *next_token = index of the first maximum of logits[0..n); then *token = *next_token and *pos += 1 (each if non-NULL). */
+int glowq_argmax_advance(const void* logits, int n, int64_t* next_token, int64_t* token, int64_t* pos, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -124,3 +124,93 @@ def test_selective_decoder_and_artifact_round_trip(fp16_out, tmp_path):
     shared2, bmap2 = decode.load_glowq_artifacts(str(tmp_path / "low_rank_shared.pt"), str(tmp_path / "b_ref_map.json"))
     assert bmap2 == bmap and set(shared2) == set(shared)
     assert all(torch.equal(shared2[k].cpu(), shared[k].cpu()) for k in shared)
+
+
+def test_glue_kernels_match_torch(ext, fp16_out):
+    g = torch.Generator(device="cuda").manual_seed(11)
+    M, H = 3, 512
+    x = torch.randn(M, H, device="cuda", generator=g).half()
+    d = torch.randn(M, H, device="cuda", generator=g).half()
+    w = (1 + 0.1 * torch.randn(H, device="cuda", generator=g)).half()
+    h = torch.empty_like(x)
+    want_x = (x + d)
+    want_h = torch.nn.functional.rms_norm(want_x.float(), (H,), w.float(), 1e-5)
+    x2 = x.clone()
+    ext.add_rmsnorm(x2, d, w, h, 1e-5)
+    assert torch.equal(x2, want_x)
+    assert (h.float() - want_h).abs().max() <= 4e-3 * want_h.abs().max()
+    ext.add_rmsnorm(x2, None, w, h, 1e-5)          # no residual: x untouched
+    assert torch.equal(x2, want_x)
+
+    gate, up = torch.randn(1, 1024, device="cuda", generator=g).half() * 3, torch.randn(1, 1024, device="cuda", generator=g).half()
+    out = torch.empty_like(gate)
+    ext.silu_mul(gate, up, out)
+    want = torch.nn.functional.silu(gate.float()) * up.float()
+    assert (out.float() - want).abs().max() <= 4e-3 * want.abs().max()
+
+    logits = torch.randn(1, 5000, device="cuda", generator=g).half()
+    logits[0, 1234] = 9.0
+    logits[0, 4321] = 9.0                           # a tie: the first index wins
+    nxt, tok, pos = (torch.zeros(1, dtype=torch.long, device="cuda") for _ in range(3))
+    pos.fill_(41)
+    ext.argmax_advance(logits, nxt, tok, pos)
+    assert (int(nxt), int(tok), int(pos)) == (1234, 1234, 42)
+
+
+@pytest.mark.parametrize("pos", [0, 1, 37, 300])
+def test_rope_attend_matches_torch(ext, fp16_out, pos):
+    heads, kvh, d, max_len = 8, 2, 64, 320
+    g = torch.Generator(device="cuda").manual_seed(pos)
+    q = torch.randn(heads, d, device="cuda", generator=g).half()
+    k = torch.randn(kvh, d, device="cuda", generator=g).half()
+    v = torch.randn(kvh, d, device="cuda", generator=g).half()
+    ck = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    cv = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    model = decode.Decoder(decode.DecoderConfig(hidden=heads * d, layers=0, heads=heads, kv_heads=kvh, head_dim=d, intermediate=64,
+                                                vocab=8, max_len=max_len))
+    cos, sin = model.rope_tables("cuda")
+    p = torch.tensor([pos], device="cuda")
+    # torch yardstick in fp32 on the fp16-rounded tables
+    c, s = cos[pos].half().float(), sin[pos].half().float()
+    rot = lambda t: torch.cat((-t[..., d // 2:], t[..., :d // 2]), dim=-1)
+    qr = (q.float() * c + rot(q.float()) * s).half().float()
+    kr = (k.float() * c + rot(k.float()) * s).half()
+    K = torch.cat((ck[:, :pos].float(), kr.float()[:, None]), dim=1).repeat_interleave(heads // kvh, dim=0)
+    V = torch.cat((cv[:, :pos].float(), v.float()[:, None]), dim=1).repeat_interleave(heads // kvh, dim=0)
+    att = torch.softmax(torch.einsum("hd,htd->ht", qr, K) * d ** -0.5, dim=-1)
+    want = torch.einsum("ht,htd->hd", att, V)
+    ck2, cv2 = ck.clone(), cv.clone()
+    out = torch.empty(heads, d, dtype=torch.float16, device="cuda")
+    ext.rope_attend(q.reshape(-1), k.reshape(-1), v.reshape(-1), cos, sin, p, ck2, cv2, out, d ** -0.5)
+    torch.cuda.synchronize()
+    assert (out.float() - want).abs().max() <= 2e-3 + 2e-3 * want.abs().max()
+    assert torch.equal(ck2[:, pos], kr) and torch.equal(cv2[:, pos], v)          # appended at pos
+    keep = torch.ones(max_len, dtype=torch.bool, device="cuda")
+    keep[pos] = False
+    assert torch.equal(ck2[:, keep], ck[:, keep]) and torch.equal(cv2[:, keep], cv[:, keep])   # nothing else touched
+
+
+def test_fused_step_matches_module_path(fp16_out):
+    cfg = decode.DecoderConfig(**TINY)
+    model, _, _ = decode.build_decoder(cfg, seed=8)
+    prompt = torch.randint(0, cfg.vocab, (11,), generator=torch.Generator().manual_seed(4))
+    ref = decode.GreedyDecoder(model, use_graph=False)
+    fus = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    first = ref.prefill(prompt)
+    fus.prefill(prompt)
+    tok = first.clone()
+    for step in range(6):                                   # teacher forcing: both see the yardstick's tokens
+        pos = torch.tensor([prompt.numel() + step], device="cuda")
+        want = model.forward_tokens(tok, pos, ref.caches, ref.cos, ref.sin).float()
+        fus.tok.copy_(tok), fus.pos.copy_(pos)
+        fus.fused.run()
+        got = fus.fused.logits.float()
+        assert (got - want).abs().max() <= 1e-2 + 1e-2 * want.abs().max(), step
+        assert int(fus.pos) == int(pos) + 1 and int(fus.tok) == int(got.argmax())
+        tok = want.argmax(-1)
+    # the captured fused step replays to the same tokens as the eager fused step
+    eager, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)
+    graphed = decode.GreedyDecoder(model, use_graph=True, fused=True)
+    for _ in range(3):
+        got, _, _ = graphed.generate(prompt, 10)
+        assert torch.equal(got, eager)
