@@ -87,33 +87,59 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const half_t* __restrict_
   }
 }
 
-// One query token against the cache, one workgroup per query head.
+// Sum over the kLanes (8 or 16) consecutive lanes that share a cache row; every lane of the group gets the total.
+template <int kLanes>
+__device__ __forceinline__ float row_group_sum(float v) {
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true);  // row_half_mirror
+  v += __builtin_bit_cast(float, t);
+  if constexpr (kLanes == 16) {
+    t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true);  // row_mirror
+    v += __builtin_bit_cast(float, t);
+  }
+  return v;
+}
+
+// One query token against the cache, one workgroup (16 waves) per query head; kD = head dimension (64 or 128).
 //   q [heads, d], k_new / v_new [kv_heads, d]: this token's projections (k, q not yet rotated)
 //   cos / sin [max_len, d] fp32 tables (second half repeats the first), *pos the token's position
 //   cache_k / cache_v [kv_heads, max_len, d] fp16: positions < pos are read; position pos is WRITTEN by the first
-//   head of each KV group and taken from registers by all, so no workgroup reads what another one writes.
+//   head of each KV group and taken from LDS by all, so no workgroup reads what another one writes.
 //   out [heads, d] fp16.
-// Scores in LDS (max_len floats), softmax over [0, pos], then P.V with lanes across the head dimension.
-__global__ __launch_bounds__(256) void rope_attend_kernel(const half_t* __restrict__ q, const half_t* __restrict__ k_new,
-                                                           const half_t* __restrict__ v_new, const float* __restrict__ cos_t,
-                                                           const float* __restrict__ sin_t, const long* __restrict__ pos_p,
-                                                           half_t* __restrict__ cache_k, half_t* __restrict__ cache_v,
-                                                           half_t* __restrict__ out, int heads, int kv_heads, int d,
-                                                           int max_len, float scale) {
+// d/8 consecutive lanes share a cache row (16 bytes each: a wave load covers 4 or 8 whole rows, several loads in
+// flight), scores go to LDS (max_len floats), softmax over [0, pos], then P.V with the same lane mapping.
+template <int kD>
+__global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restrict__ q, const half_t* __restrict__ k_new,
+                                                            const half_t* __restrict__ v_new, const float* __restrict__ cos_t,
+                                                            const float* __restrict__ sin_t, const long* __restrict__ pos_p,
+                                                            half_t* __restrict__ cache_k, half_t* __restrict__ cache_v,
+                                                            half_t* __restrict__ out, int heads, int kv_heads, int max_len,
+                                                            float scale) {
+  constexpr int d = kD;
+  constexpr int kLanes = d / 8;           // lanes per cache row
+  constexpr int kRowsPerWave = 64 / kLanes;
+  constexpr int kUnroll = 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* qs = reinterpret_cast<float*>(smem_raw);            // [d] rotated query
   float* kn = qs + d;                                        // [d] rotated key of this token
   float* vn = kn + d;                                        // [d] value of this token
   float* red = vn + d;                                       // [16]
   float* acc_part = red + 16;                                // [waves][d]
-  float* sc = acc_part + (blockDim.x >> 6) * d;              // [max_len] scores / probabilities
+  float* sc = acc_part + 16 * d;                             // [max_len] scores / probabilities
   const int head = blockIdx.x;
   const int rep = heads / kv_heads;
   const int kvh = head / rep;
   const int pos = (int)*pos_p;
-  const int half_d = d >> 1;
+  constexpr int half_d = d >> 1;
   const int nw = blockDim.x >> 6;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  const int sub = lane % kLanes, rg = lane / kLanes;
+  const int row0 = wave * kRowsPerWave + rg;      // first cache row of this lane group
+  const int row_step = nw * kRowsPerWave;
 
   // rotary embedding of q and k_new: out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i + d/2] cos + x[i] sin
   for (int i = threadIdx.x; i < half_d; i += blockDim.x) {
@@ -138,25 +164,34 @@ __global__ __launch_bounds__(256) void rope_attend_kernel(const half_t* __restri
   }
   __syncthreads();
 
-  // scores: one position per thread, the key row read as 16-byte pieces
-  const half_t* kbase = cache_k + (size_t)kvh * max_len * d;
-  float mx = -INFINITY;
-  for (int p = threadIdx.x; p <= pos; p += blockDim.x) {
-    float dot = 0.f;
-    if (p == pos) {
-      for (int i = 0; i < d; ++i) dot = __builtin_fmaf(qs[i], kn[i], dot);
-    } else {
-      const h8* kr = reinterpret_cast<const h8*>(kbase + (size_t)p * d);
-      for (int i = 0; i < d / 8; ++i) {
-        const h8 kv = kr[i];
+  float qv[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qs[8 * i + j], (float)kv[j], dot);
-      }
+  for (int j = 0; j < 8; ++j) qv[j] = qs[8 * sub + j];
+
+  // scores of the cached positions [0, pos)
+  const half_t* kbase = cache_k + (size_t)kvh * max_len * d + 8 * sub;
+  for (int p0 = row0; p0 < pos; p0 += kUnroll * row_step) {
+    h8 kv[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) kv[u] = *reinterpret_cast<const h8*>(kbase + (size_t)min(p0 + u * row_step, pos - 1) * d);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      float dot = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qv[j], (float)kv[u][j], dot);
+      dot = row_group_sum<kLanes>(dot);
+      const int p = p0 + u * row_step;
+      if (sub == 0 && p < pos) sc[p] = dot * scale;
     }
-    dot *= scale;
-    sc[p] = dot;
-    mx = fmaxf(mx, dot);
   }
+  if (threadIdx.x == 0) {  // this token against itself
+    float dot = 0.f;
+    for (int i = 0; i < d; ++i) dot = __builtin_fmaf(qs[i], kn[i], dot);
+    sc[pos] = dot * scale;
+  }
+  __syncthreads();
+  float mx = -INFINITY;
+  for (int p = threadIdx.x; p <= pos; p += blockDim.x) mx = fmaxf(mx, sc[p]);
   mx = block_max(mx, red, nw);
   float sum = 0.f;
   for (int p = threadIdx.x; p <= pos; p += blockDim.x) {
@@ -167,35 +202,37 @@ __global__ __launch_bounds__(256) void rope_attend_kernel(const half_t* __restri
   sum = block_sum(sum, red, nw);  // its barriers also publish sc[]
   const float inv = 1.f / sum;
 
-  // P.V: lane l holds dimensions 2l, 2l+1; the waves take positions round robin, 4 rows in flight each
-  const half_t* vbase = cache_v + (size_t)kvh * max_len * d;
-  float a0 = 0.f, a1 = 0.f;
-  if (2 * lane < d) {
-    int p = wave;
-    for (; p + 3 * nw < pos; p += 4 * nw) {
-      h2 v[4];
+  // P.V over the cached positions, 8 dimensions per lane
+  const half_t* vbase = cache_v + (size_t)kvh * max_len * d + 8 * sub;
+  float acc[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const h2*>(vbase + (size_t)(p + j * nw) * d + 2 * lane);
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  for (int p0 = row0; p0 < pos; p0 += kUnroll * row_step) {
+    h8 vv[kUnroll];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float pr = sc[p + j * nw];
-        a0 = __builtin_fmaf(pr, (float)v[j][0], a0);
-        a1 = __builtin_fmaf(pr, (float)v[j][1], a1);
-      }
+    for (int u = 0; u < kUnroll; ++u) vv[u] = *reinterpret_cast<const h8*>(vbase + (size_t)min(p0 + u * row_step, pos - 1) * d);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int p = p0 + u * row_step;
+      const float pr = p < pos ? sc[p] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, (float)vv[u][j], acc[j]);
     }
-    for (; p < pos; p += nw) {
-      const h2 v = *reinterpret_cast<const h2*>(vbase + (size_t)p * d + 2 * lane);
-      const float pr = sc[p];
-      a0 = __builtin_fmaf(pr, (float)v[0], a0);
-      a1 = __builtin_fmaf(pr, (float)v[1], a1);
-    }
-    if (wave == 0) {  // this token's own value
-      const float pr = sc[pos];
-      a0 = __builtin_fmaf(pr, vn[2 * lane], a0);
-      a1 = __builtin_fmaf(pr, vn[2 * lane + 1], a1);
-    }
-    acc_part[wave * d + 2 * lane] = a0;
-    acc_part[wave * d + 2 * lane + 1] = a1;
+  }
+  if (wave == 0 && rg == 0) {  // this token's own value
+    const float pr = sc[pos];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, vn[8 * sub + j], acc[j]);
+  }
+  // the lane groups of a wave, then the waves
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+#pragma unroll
+    for (int o = kLanes; o < 64; o <<= 1) acc[j] += __shfl_xor(acc[j], o);
+  }
+  if (rg == 0) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc_part[wave * d + 8 * sub + j] = acc[j];
   }
   __syncthreads();
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
@@ -212,9 +249,19 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
   __shared__ int bi[16];
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+  const int n8 = (reinterpret_cast<uintptr_t>(logits) & 15) == 0 ? n / 8 : 0;  // 16-byte pieces, then the tail
+  for (int i = threadIdx.x; i < n8; i += blockDim.x) {
+    const h8 v = reinterpret_cast<const h8*>(logits)[i];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if ((float)v[j] > best) {  // ascending index per thread: the first maximum wins
+        best = (float)v[j];
+        idx = 8 * i + j;
+      }
+  }
+  for (int i = 8 * n8 + threadIdx.x; i < n; i += blockDim.x) {
     const float v = (float)logits[i];
-    if (v > best) {  // ascending i per thread: the first maximum wins
+    if (v > best || (v == best && i < idx)) {
       best = v;
       idx = i;
     }
@@ -265,22 +312,33 @@ hipError_t launch_silu_mul(const half_t* gate, const half_t* up, half_t* out, lo
   return hipGetLastError();
 }
 
-size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 4 * d + max_len) * sizeof(float); }
+size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 16 * d + max_len) * sizeof(float); }
 
-hipError_t launch_rope_attend(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
-                              const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
-                              int heads, int kv_heads, int d, int max_len, float scale, hipStream_t stream) {
-  const size_t lds = rope_attend_lds(d, max_len);
+template <int kD>
+static hipError_t launch_rope_attend_t(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
+                                       const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
+                                       int heads, int kv_heads, int max_len, float scale, hipStream_t stream) {
+  const size_t lds = rope_attend_lds(kD, max_len);
   static size_t configured = 48 * 1024;
   if (lds > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rope_attend_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rope_attend_kernel<kD>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     configured = lds;
   }
-  hipLaunchKernelGGL(rope_attend_kernel, dim3(heads), dim3(256), lds, stream, q, k_new, v_new, cos_t, sin_t, pos,
-                     cache_k, cache_v, out, heads, kv_heads, d, max_len, scale);
+  hipLaunchKernelGGL(rope_attend_kernel<kD>, dim3(heads), dim3(1024), lds, stream, q, k_new, v_new, cos_t, sin_t, pos,
+                     cache_k, cache_v, out, heads, kv_heads, max_len, scale);
   return hipGetLastError();
+}
+
+hipError_t launch_rope_attend(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
+                              const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
+                              int heads, int kv_heads, int d, int max_len, float scale, hipStream_t stream) {
+  if (d == 128)
+    return launch_rope_attend_t<128>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, heads, kv_heads, max_len, scale, stream);
+  if (d == 64)
+    return launch_rope_attend_t<64>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, heads, kv_heads, max_len, scale, stream);
+  return hipErrorInvalidValue;
 }
 
 hipError_t launch_argmax_advance(const half_t* logits, int n, long* next_tok, long* tok, long* pos, hipStream_t stream) {
@@ -315,9 +373,9 @@ int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const
                       int max_len, float scale, void* stream) {
   if (!q || !k_new || !v_new || !cos_table || !sin_table || !pos || !cache_k || !cache_v || !out)
     return fail(GLOWQ_EINVAL, "rope_attend: all pointers must be device pointers");
-  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || head_dim <= 0 || (head_dim & 7) || head_dim > 128 || max_len <= 0)
-    return fail(GLOWQ_EINVAL, "rope_attend: heads %% kv_heads == 0, head_dim a multiple of 8 up to 128 (got %d, %d, %d)", heads,
-                kv_heads, head_dim);
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || max_len <= 0)
+    return fail(GLOWQ_EINVAL, "rope_attend: heads must be a positive multiple of kv_heads (got %d, %d)", heads, kv_heads);
+  if (head_dim != 64 && head_dim != 128) return fail(GLOWQ_EUNSUPPORTED, "rope_attend: head_dim must be 64 or 128 (got %d)", head_dim);
   if (rope_attend_lds(head_dim, max_len) > 160 * 1024)
     return fail(GLOWQ_EUNSUPPORTED, "rope_attend: max_len %d does not fit the score buffer in LDS", max_len);
   hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),

@@ -153,7 +153,7 @@ int glowq_silu_mul(const void* gate, const void* up, void* out, long n, void* st
 /*
  * Rotary embedding of q [heads, d] and k_new [kv_heads, d] at position *pos (cos/sin tables [max_len, d] fp32),
  * append of k / v_new to the caches [kv_heads, max_len, d] at *pos, attention of the one query token over positions
- * 0..*pos, out [heads, d].  d <= 128, max_len limited by the LDS score buffer (about 40k positions).
+ * 0..*pos, out [heads, d].  d = 64 or 128, max_len limited by the LDS score buffer (about 38k positions).
  */
 int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
                       const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,
