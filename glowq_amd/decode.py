@@ -216,8 +216,9 @@ class FusedStep:
     Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
     the one-call projection + group entry point, o_proj and down_proj as solo groups."""
 
-    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok):
+    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True):
         cfg = model.cfg
+        self.share = share  # False: every module projects x on R by itself and launches alone (the no-sharing comparator)
         self.model, self.cfg = model, cfg
         self.ext = load_w4a16_extension()
         dev = model.lm_head.weight.device
@@ -267,7 +268,14 @@ class FusedStep:
         return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs}
 
     def _linear(self, x, grp):
-        self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"], R=grp["R"])
+        if self.share:
+            self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"], R=grp["R"])
+            return
+        # layer-wise correction without sharing (test/step3_1_layerwise.py:133-153): one projection and one launch per module
+        for mem, out in zip(grp["members"], grp["outs"]):
+            corrected = mem["L"] is not None
+            self.ext.group_forward(x, grp["r"] if corrected else None, [mem], grp["gs"], grp["alpha"], outs=[out],
+                                   R=grp["R"] if corrected else None)
 
     @torch.no_grad()
     def run(self):
@@ -293,7 +301,7 @@ class FusedStep:
 class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
-    def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False):
+    def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True):
         self.model = model
         cfg = model.cfg
         dev = model.lm_head.weight.device
@@ -307,7 +315,7 @@ class GreedyDecoder:
         self.next_tok = torch.zeros(1, dtype=torch.long, device=dev)
         self.use_graph = use_graph
         self.graph = None
-        self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok) if fused else None
+        self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok, share) if fused else None
 
     @torch.no_grad()
     def _step(self):
@@ -383,6 +391,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new", type=int, default=256)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-sharing", action="store_true", help="fused step with one projection and one launch per module")
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
     ap.add_argument("--vocab", type=int, default=128256)
@@ -395,7 +404,7 @@ def main():
     model, _, _ = build_decoder(cfg, with_correction=not args.no_correction)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path)
+    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path, share=not args.no_sharing)
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=g)
     dec.generate(prompt, 4)  # warm-up (also captures the graph)
@@ -403,7 +412,7 @@ def main():
     print(json.dumps({
         "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
                     f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + ("" if args.no_correction else f" + GlowQ r={cfg.rank}"),
-        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph, "fused_step": not args.module_path,
+        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph, "fused_step": not args.module_path, "group_sharing": not args.no_sharing,
         "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((args.new - 1) / decode_s, 1),
         "ms_per_token": round(decode_s * 1e3 / (args.new - 1), 3), "build_s": round(build_s, 1)}))
 

@@ -208,9 +208,45 @@ def test_fused_step_matches_module_path(fp16_out):
         assert (got - want).abs().max() <= 1e-2 + 1e-2 * want.abs().max(), step
         assert int(fus.pos) == int(pos) + 1 and int(fus.tok) == int(got.argmax())
         tok = want.argmax(-1)
+    # without sharing (one projection and one launch per module) the step computes the same tokens
+    alone, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True, share=False).generate(prompt, 10)
+    assert torch.equal(alone, decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)[0])
     # the captured fused step replays to the same tokens as the eager fused step
     eager, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)
     graphed = decode.GreedyDecoder(model, use_graph=True, fused=True)
     for _ in range(3):
         got, _, _ = graphed.generate(prompt, 10)
         assert torch.equal(got, eager)
+
+
+def test_perplexity_windows_and_effective_weight_network(fp16_out, tmp_path):
+    from glowq_amd import evaluate
+    cfg = decode.DecoderConfig(**TINY)
+    model, _, _ = decode.build_decoder(cfg, seed=9)
+    ids = torch.randint(0, cfg.vocab, (131,), generator=torch.Generator().manual_seed(5))
+    np.save(tmp_path / "ids.npy", ids.numpy().astype(np.int32))
+    assert torch.equal(evaluate.load_local_tokens(str(tmp_path / "ids.npy"), cfg.vocab), ids)
+    (tmp_path / "raw.bin").write_bytes(bytes([1, 2, 250]))
+    assert evaluate.load_local_tokens(str(tmp_path / "raw.bin"), cfg.vocab).tolist() == [1, 2, 250]
+    with pytest.raises(ValueError):
+        evaluate.load_local_tokens(str(tmp_path / "raw.bin"), 200)
+    ppl, secs = evaluate.evaluate_token_ids(model, ids, seq_len=40)
+    # the same windows by hand on the effective-weight network: 40+40+40+11 tokens -> 39+39+39+10 predictions
+    saved = _swap_in_reference(model)
+    tot, cnt = 0.0, 0
+    for b in range(0, 131, 40):
+        w = ids[b:b + 40]
+        lg = torch.from_numpy(_logits(model, w))
+        lp = torch.log_softmax(lg[:-1].double(), dim=-1)
+        tot += float(-lp[torch.arange(w.numel() - 1), w[1:]].sum())
+        cnt += w.numel() - 1
+    _restore(saved)
+    assert cnt == 127
+    want = float(np.exp(tot / cnt))
+    assert abs(ppl - want) <= 5e-3 * want and secs > 0
+    # a window of one token is skipped; uniform logits give PPL = vocab whatever the windows are
+    model.lm_head.weight.zero_()
+    ppl0, _ = evaluate.evaluate_token_ids(model, ids[:41], seq_len=40)
+    assert abs(ppl0 - cfg.vocab) <= 1e-3 * cfg.vocab
+    with pytest.raises(ValueError):
+        evaluate.evaluate_token_ids(model, ids, seq_len=cfg.max_len + 1)
