@@ -71,6 +71,102 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(half_t* __restrict__ 
   }
 }
 
+// Single-token forms that also produce the shared right-factor projection of their output, so the group launch that
+// follows needs no projection launch of its own.  One workgroup per row j of R: every workgroup recomputes the (cheap)
+// elementwise result, dots it with R[j] and writes r[j]; the elementwise outputs are written in 8-element chunks dealt
+// round robin over the workgroups.  x_out must not alias x_in (other workgroups still read it).
+__global__ __launch_bounds__(256) void add_rmsnorm_proj_kernel(const half_t* __restrict__ x_in, const half_t* __restrict__ delta,
+                                                               const half_t* __restrict__ w, half_t* __restrict__ x_out,
+                                                               half_t* __restrict__ h, const half_t* __restrict__ R,
+                                                               half_t* __restrict__ r, int H, int rank, float eps) {
+  __shared__ float red[16];
+  const int j = blockIdx.x;
+  const int nw = blockDim.x >> 6;
+  const int chunks = H >> 3;
+  constexpr int kMax = 4;  // chunks per thread: H <= 8 * 256 * 4
+  h8 xv[kMax], wv[kMax], rv[kMax];
+  // every load goes out before the first reduction: one memory round trip for the whole kernel
+#pragma unroll
+  for (int c = 0; c < kMax; ++c) {
+    const int i = min((int)(threadIdx.x + c * blockDim.x), chunks - 1);
+    xv[c] = reinterpret_cast<const h8*>(x_in)[i];
+    wv[c] = reinterpret_cast<const h8*>(w)[i];
+    rv[c] = reinterpret_cast<const h8*>(R + (size_t)j * H)[i];
+  }
+  if (delta) {
+    h8 dv[kMax];
+#pragma unroll
+    for (int c = 0; c < kMax; ++c) dv[c] = reinterpret_cast<const h8*>(delta)[min((int)(threadIdx.x + c * blockDim.x), chunks - 1)];
+#pragma unroll
+    for (int c = 0; c < kMax; ++c)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[c][e] = (half_t)((float)xv[c][e] + (float)dv[c][e]);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kMax; ++c) {
+    const bool live = threadIdx.x + c * blockDim.x < chunks;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = __builtin_fmaf(live ? (float)xv[c][e] : 0.f, (float)xv[c][e], ss);
+  }
+  const float inv = rsqrtf(block_sum(ss, red, nw) / (float)H + eps);
+  float dot = 0.f;
+#pragma unroll
+  for (int c = 0; c < kMax; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    if (i < chunks) {
+      h8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        o[e] = (half_t)((float)(half_t)((float)xv[c][e] * inv) * (float)wv[c][e]);
+        dot = __builtin_fmaf((float)o[e], (float)rv[c][e], dot);
+      }
+      if (i % rank == j) {
+        reinterpret_cast<h8*>(x_out)[i] = xv[c];
+        reinterpret_cast<h8*>(h)[i] = o;
+      }
+    }
+  }
+  dot = block_sum(dot, red, nw);
+  if (threadIdx.x == 0) r[j] = (half_t)dot;
+}
+
+// 1024 threads, at most kMax chunks of 8 per thread, all loads first.
+__global__ __launch_bounds__(1024) void silu_mul_proj_kernel(const half_t* __restrict__ gate, const half_t* __restrict__ up,
+                                                             half_t* __restrict__ out, const half_t* __restrict__ R,
+                                                             half_t* __restrict__ r, int n, int rank) {
+  __shared__ float red[16];
+  const int j = blockIdx.x;
+  const int nw = blockDim.x >> 6;
+  const int chunks = n >> 3;
+  constexpr int kMax = 4;  // n <= 8 * 1024 * 4
+  h8 gv[kMax], uv[kMax], rv[kMax];
+#pragma unroll
+  for (int c = 0; c < kMax; ++c) {
+    const int i = min((int)(threadIdx.x + c * blockDim.x), chunks - 1);
+    gv[c] = reinterpret_cast<const h8*>(gate)[i];
+    uv[c] = reinterpret_cast<const h8*>(up)[i];
+    rv[c] = reinterpret_cast<const h8*>(R + (size_t)j * n)[i];
+  }
+  float dot = 0.f;
+#pragma unroll
+  for (int c = 0; c < kMax; ++c) {
+    const int i = threadIdx.x + c * blockDim.x;
+    if (i < chunks) {
+      h8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float gf = (float)gv[c][e];
+        o[e] = (half_t)((float)(half_t)(gf / (1.f + __expf(-gf))) * (float)uv[c][e]);
+        dot = __builtin_fmaf((float)o[e], (float)rv[c][e], dot);
+      }
+      if (i % rank == j) reinterpret_cast<h8*>(out)[i] = o;
+    }
+  }
+  dot = block_sum(dot, red, nw);
+  if (threadIdx.x == 0) r[j] = (half_t)dot;
+}
+
 // out = silu(gate) * up, elementwise, fp32 math.
 __global__ __launch_bounds__(256) void silu_mul_kernel(const half_t* __restrict__ gate, const half_t* __restrict__ up,
                                                         half_t* __restrict__ out, long n8) {
@@ -312,6 +408,18 @@ hipError_t launch_silu_mul(const half_t* gate, const half_t* up, half_t* out, lo
   return hipGetLastError();
 }
 
+hipError_t launch_add_rmsnorm_proj(const half_t* x_in, const half_t* delta, const half_t* w, half_t* x_out, half_t* h,
+                                   const half_t* R, half_t* r, int H, int rank, float eps, hipStream_t stream) {
+  hipLaunchKernelGGL(add_rmsnorm_proj_kernel, dim3(rank), dim3(256), 0, stream, x_in, delta, w, x_out, h, R, r, H, rank, eps);
+  return hipGetLastError();
+}
+
+hipError_t launch_silu_mul_proj(const half_t* gate, const half_t* up, half_t* out, const half_t* R, half_t* r, int n, int rank,
+                                hipStream_t stream) {
+  hipLaunchKernelGGL(silu_mul_proj_kernel, dim3(rank), dim3(1024), 0, stream, gate, up, out, R, r, n, rank);
+  return hipGetLastError();
+}
+
 size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 16 * d + max_len) * sizeof(float); }
 
 template <int kD>
@@ -366,6 +474,28 @@ int glowq_silu_mul(const void* gate, const void* up, void* out, long n, void* st
   hipError_t e = launch_silu_mul(static_cast<const half_t*>(gate), static_cast<const half_t*>(up), static_cast<half_t*>(out), n,
                                  num_cus(), static_cast<hipStream_t>(stream));
   return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "silu_mul launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_add_rmsnorm_proj(const void* x_in, const void* delta, const void* weight, void* x_out, void* h, const void* R,
+                           void* r, int H, int rank, float eps, void* stream) {
+  if (!x_in || !weight || !x_out || !h || !R || !r) return fail(GLOWQ_EINVAL, "add_rmsnorm_proj: pointers must be device pointers");
+  if (x_in == x_out) return fail(GLOWQ_EINVAL, "add_rmsnorm_proj: x_out must not alias x_in");
+  if (H <= 0 || (H & 7) || H > 8192 || rank <= 0)
+    return fail(GLOWQ_EINVAL, "add_rmsnorm_proj: H a multiple of 8 up to 8192 and rank > 0 (got H=%d, rank=%d)", H, rank);
+  hipError_t e = launch_add_rmsnorm_proj(static_cast<const half_t*>(x_in), static_cast<const half_t*>(delta),
+                                         static_cast<const half_t*>(weight), static_cast<half_t*>(x_out), static_cast<half_t*>(h),
+                                         static_cast<const half_t*>(R), static_cast<half_t*>(r), H, rank, eps,
+                                         static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "add_rmsnorm_proj launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_silu_mul_proj(const void* gate, const void* up, void* out, const void* R, void* r, int n, int rank, void* stream) {
+  if (!gate || !up || !out || !R || !r) return fail(GLOWQ_EINVAL, "silu_mul_proj: pointers must be device pointers");
+  if (n <= 0 || (n & 7) || n > 32768 || rank <= 0)
+    return fail(GLOWQ_EINVAL, "silu_mul_proj: n a multiple of 8 up to 32768, rank > 0 (got %d, %d)", n, rank);
+  hipError_t e = launch_silu_mul_proj(static_cast<const half_t*>(gate), static_cast<const half_t*>(up), static_cast<half_t*>(out),
+                                      static_cast<const half_t*>(R), static_cast<half_t*>(r), n, rank, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "silu_mul_proj launch failed: %s", hipGetErrorString(e));
 }
 
 int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,

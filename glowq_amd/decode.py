@@ -212,7 +212,7 @@ def load_glowq_artifacts(shared_path: str, bmap_path: str, device="cuda"):
 
 
 class FusedStep:
-    """One decode token as a fixed chain of launches on static buffers (13 per layer), ready for HIP-graph capture.
+    """One decode token as a fixed chain of launches on static buffers (10 per layer), ready for HIP-graph capture.
     Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
     the one-call projection + group entry point, o_proj and down_proj as solo groups."""
 
@@ -227,6 +227,7 @@ class FusedStep:
         f16 = dict(dtype=torch.float16, device=dev)
         qd, kd = cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim
         self.x = torch.zeros(1, cfg.hidden, **f16)
+        self.x_alt = torch.zeros(1, cfg.hidden, **f16)   # the residual stream alternates between the two
         self.h = torch.zeros(1, cfg.hidden, **f16)
         self.qkv = torch.zeros(1, qd + 2 * kd, **f16)
         self.attn = torch.zeros(1, qd, **f16)
@@ -267,9 +268,20 @@ class FusedStep:
         r = torch.zeros(1, R.size(0), **f16) if R is not None else None
         return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs}
 
-    def _linear(self, x, grp):
+    def _norm(self, x, delta, ln, grp):
+        """Residual add + RMSNorm into self.h; with a shared group behind it the projection r = h R^T comes out of the same
+        launch.  Returns (residual stream after the add, whether r is already computed)."""
+        if self.share and grp["R"] is not None:
+            nxt = self.x_alt if x is self.x else self.x
+            self.ext.add_rmsnorm_proj(x, delta, ln.weight, nxt, self.h, grp["R"], grp["r"], ln.eps)
+            return nxt, True
+        self.ext.add_rmsnorm(x, delta, ln.weight, self.h, ln.eps)
+        return x, False
+
+    def _linear(self, x, grp, r_ready=False):
         if self.share:
-            self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"], R=grp["R"])
+            self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"],
+                                   R=None if r_ready else grp["R"])
             return
         # layer-wise correction without sharing (test/step3_1_layerwise.py:133-153): one projection and one launch per module
         for mem, out in zip(grp["members"], grp["outs"]):
@@ -280,20 +292,26 @@ class FusedStep:
     @torch.no_grad()
     def run(self):
         ext, cfg = self.ext, self.cfg
-        torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=self.x)
+        x = self.x
+        torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=x)
         delta = None
         for lay, (ck, cv) in zip(self.plan, self.caches):
-            ext.add_rmsnorm(self.x, delta, lay["ln1"].weight, self.h, lay["ln1"].eps)
-            self._linear(self.h, lay["qkv"])
+            x, ready = self._norm(x, delta, lay["ln1"], lay["qkv"])
+            self._linear(self.h, lay["qkv"], ready)
             ext.rope_attend(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.attn, self.scale)
             self._linear(self.attn, lay["o"])
-            ext.add_rmsnorm(self.x, self.o, lay["ln2"].weight, self.h, lay["ln2"].eps)
-            self._linear(self.h, lay["gu"])
-            ext.silu_mul(self.gu[:, :cfg.intermediate], self.gu[:, cfg.intermediate:], self.act)
-            self._linear(self.act, lay["down"])
+            x, ready = self._norm(x, self.o, lay["ln2"], lay["gu"])
+            self._linear(self.h, lay["gu"], ready)
+            gate, up, down = self.gu[:, :cfg.intermediate], self.gu[:, cfg.intermediate:], lay["down"]
+            if self.share and down["R"] is not None:
+                ext.silu_mul_proj(gate, up, self.act, down["R"], down["r"])
+                self._linear(self.act, down, True)
+            else:
+                ext.silu_mul(gate, up, self.act)
+                self._linear(self.act, down)
             delta = self.dn
         norm = self.model.model.norm
-        ext.add_rmsnorm(self.x, delta, norm.weight, self.h, norm.eps)
+        ext.add_rmsnorm(x, delta, norm.weight, self.h, norm.eps)
         torch.mm(self.h, self.model.lm_head.weight.t(), out=self.logits)
         ext.argmax_advance(self.logits, self.next_tok, self.tok, self.pos)
 

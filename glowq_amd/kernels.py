@@ -53,6 +53,8 @@ _SIGNATURES = {
     "glowq_set_tuning": (_I, [ctypes.c_char_p, _I]),
     "glowq_add_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
     "glowq_silu_mul": (_I, [_P, _P, _P, ctypes.c_long, _P]),
+    "glowq_add_rmsnorm_proj": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
+    "glowq_silu_mul_proj": (_I, [_P, _P, _P, _P, _P, _I, _I, _P]),
     "glowq_rope_attend": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_argmax_advance": (_I, [_P, _I, _P, _P, _P, _P]),
 }
@@ -271,6 +273,36 @@ class W4A16Extension:
             rc = self.lib.glowq_silu_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), self._stream(out.device))
         if rc:
             self._raise(rc, "silu_mul")
+
+    def add_rmsnorm_proj(self, x_in, delta, weight, x_out, h, R, r, eps: float) -> None:
+        """One token: x_out = x_in + delta, h = rmsnorm(x_out) * weight, r = h R^T (R [rank, H], r [1, rank])."""
+        for t, n in ((x_in, "x_in"), (weight, "weight"), (x_out, "x_out"), (h, "h"), (R, "R"), (r, "r")):
+            self._f16(t, n)
+        H = x_in.numel()
+        _check(x_out.numel() == H and h.numel() == H and weight.numel() == H and R.dim() == 2 and R.size(1) == H
+               and r.numel() == R.size(0), "add_rmsnorm_proj: shape mismatch")
+        if delta is not None:
+            self._f16(delta, "delta")
+            _check(delta.numel() == H, "add_rmsnorm_proj: delta must have the size of x")
+        with torch.cuda.device(x_in.device):
+            rc = self.lib.glowq_add_rmsnorm_proj(x_in.data_ptr(), delta.data_ptr() if delta is not None else None, weight.data_ptr(),
+                                                 x_out.data_ptr(), h.data_ptr(), R.data_ptr(), r.data_ptr(), H, R.size(0),
+                                                 float(eps), self._stream(x_in.device))
+        if rc:
+            self._raise(rc, "add_rmsnorm_proj")
+
+    def silu_mul_proj(self, gate, up, out, R, r) -> None:
+        """One token: out = silu(gate) * up, r = out R^T."""
+        for t, n in ((gate, "gate"), (up, "up"), (out, "out"), (R, "R"), (r, "r")):
+            self._f16(t, n)
+        n = gate.numel()
+        _check(up.numel() == n and out.numel() == n and R.dim() == 2 and R.size(1) == n and r.numel() == R.size(0),
+               "silu_mul_proj: shape mismatch")
+        with torch.cuda.device(out.device):
+            rc = self.lib.glowq_silu_mul_proj(gate.data_ptr(), up.data_ptr(), out.data_ptr(), R.data_ptr(), r.data_ptr(), n,
+                                              R.size(0), self._stream(out.device))
+        if rc:
+            self._raise(rc, "silu_mul_proj")
 
     def rope_attend(self, q, k_new, v_new, cos_table, sin_table, pos, cache_k, cache_v, out, scale: float) -> None:
         """q [heads, d], k_new / v_new [kv_heads, d] of one token, tables [max_len, d] fp32, pos int64[1] on the device,

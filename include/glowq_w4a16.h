@@ -151,6 +151,14 @@ int glowq_add_rmsnorm(void* x, const void* delta, const void* weight, void* h, i
 int glowq_silu_mul(const void* gate, const void* up, void* out, long n, void* stream);
 
 /*
+ * The two above for one token, each also writing r = (its output) R^T ([rank] fp16, R [rank, H] resp. [rank, n]) for the
+ * group launch that consumes the output: one launch instead of two.  x_out must not alias x_in.
+ */
+int glowq_add_rmsnorm_proj(const void* x_in, const void* delta, const void* weight, void* x_out, void* h, const void* R,
+                           void* r, int H, int rank, float eps, void* stream);
+int glowq_silu_mul_proj(const void* gate, const void* up, void* out, const void* R, void* r, int n, int rank, void* stream);
+
+/*
  * Rotary embedding of q [heads, d] and k_new [kv_heads, d] at position *pos (cos/sin tables [max_len, d] fp32),
  * append of k / v_new to the caches [kv_heads, max_len, d] at *pos, attention of the one query token over positions
  * 0..*pos, out [heads, d].  d = 64 or 128, max_len limited by the LDS score buffer (about 38k positions).

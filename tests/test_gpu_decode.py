@@ -250,3 +250,32 @@ def test_perplexity_windows_and_effective_weight_network(fp16_out, tmp_path):
     assert abs(ppl0 - cfg.vocab) <= 1e-3 * cfg.vocab
     with pytest.raises(ValueError):
         evaluate.evaluate_token_ids(model, ids, seq_len=cfg.max_len + 1)
+
+
+def test_glue_with_projection_matches_separate_launches(ext, fp16_out):
+    g = torch.Generator(device="cuda").manual_seed(21)
+    H, rank = 1024, 64
+    x = torch.randn(1, H, device="cuda", generator=g).half()
+    d = torch.randn(1, H, device="cuda", generator=g).half()
+    w = (1 + 0.1 * torch.randn(H, device="cuda", generator=g)).half()
+    R = (torch.randn(rank, H, device="cuda", generator=g) * H ** -0.5).half()
+    x_ref, h_ref = x.clone(), torch.empty_like(x)
+    ext.add_rmsnorm(x_ref, d, w, h_ref, 1e-5)
+    r_ref = ext.shared_proj(h_ref, R)
+    x_out, h, r = torch.empty_like(x), torch.empty_like(x), torch.empty(1, rank, dtype=torch.float16, device="cuda")
+    ext.add_rmsnorm_proj(x, d, w, x_out, h, R, r, 1e-5)
+    assert torch.equal(x_out, x_ref) and torch.equal(h, h_ref)
+    assert (r.float() - r_ref.float()).abs().max() <= 2e-3 * r_ref.float().abs().max() + 1e-3
+    with pytest.raises(RuntimeError):
+        ext.add_rmsnorm_proj(x, d, w, x, h, R, r, 1e-5)           # in place is refused: other workgroups still read x
+
+    n = 2048
+    gate, up = torch.randn(1, n, device="cuda", generator=g).half() * 2, torch.randn(1, n, device="cuda", generator=g).half()
+    R2 = (torch.randn(rank, n, device="cuda", generator=g) * n ** -0.5).half()
+    act_ref = torch.empty_like(gate)
+    ext.silu_mul(gate, up, act_ref)
+    r2_ref = ext.shared_proj(act_ref, R2)
+    act, r2 = torch.empty_like(gate), torch.empty(1, rank, dtype=torch.float16, device="cuda")
+    ext.silu_mul_proj(gate, up, act, R2, r2)
+    assert torch.equal(act, act_ref)
+    assert (r2.float() - r2_ref.float()).abs().max() <= 2e-3 * r2_ref.float().abs().max() + 1e-3
