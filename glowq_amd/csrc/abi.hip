@@ -24,6 +24,7 @@ hipError_t launch_unpack(const int32_t*, uint8_t*, int, int, int, int, hipStream
 hipError_t launch_shared_proj_small(const half_t*, const half_t*, half_t*, int, int, int, hipStream_t);
 // skinny.hip / gemm.hip
 bool skinny_supported(const GroupDev& g);
+bool skinny_group_form(const GroupDev& g);
 hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream);
 bool gemm_supported(const GroupDev& g);
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream);
@@ -68,7 +69,9 @@ constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
 
 // Route limits, settable at run time (glowq_set_tuning) and initialised from the environment:
 //   wave_dot_max_m  rows up to which the wave-dot GEMV is preferred over the skinny MFMA kernel (GLOWQ_WAVEDOT_M)
-//   quad_max_m      rows up to which the 4x4x4 matrix-core GEMV is used; 0 switches it off (GLOWQ_QUAD_M)
+//   quad_max_m      rows up to which the 4x4x4 matrix-core GEMV is used; 0 switches it off (GLOWQ_QUAD_M).  Above it
+//                   the skinny MFMA kernel takes over; where only that kernel's first form applies (K % 256 != 0 or
+//                   small groups) the 4x4x4 GEMV still serves up to 16 rows
 //   quad_min_m      rows from which it is used (GLOWQ_QUAD_MIN_M; a single row is faster on the wave-dot kernel)
 int env_or(const char* name, int fallback) {
   const char* v = getenv(name);
@@ -76,7 +79,7 @@ int env_or(const char* name, int fallback) {
 }
 int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 std::atomic<int> g_wave_dot_max_m{clampi(env_or("GLOWQ_WAVEDOT_M", kWaveDotMaxM), 0, kWaveDotMaxM)};
-std::atomic<int> g_quad_max_m{clampi(env_or("GLOWQ_QUAD_M", 16), 0, 16)};
+std::atomic<int> g_quad_max_m{clampi(env_or("GLOWQ_QUAD_M", 4), 0, 16)};
 std::atomic<int> g_quad_min_m{clampi(env_or("GLOWQ_QUAD_MIN_M", 2), 1, 16)};
 int wave_dot_pref_m() { return g_wave_dot_max_m.load(std::memory_order_relaxed); }
 bool quad_wanted(int M) {
@@ -142,7 +145,9 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
-  if (quad_wanted(g.M) && force != kRouteSkinny && quad_capacity(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr) > 0) {
+  const bool quad_rows = quad_wanted(g.M) ||
+                         (g.M > 1 && g.M <= 16 && g_quad_max_m.load(std::memory_order_relaxed) > 0 && !(skinny_supported(g) && skinny_group_form(g)));
+  if (quad_rows && force != kRouteSkinny && quad_capacity(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr) > 0) {
     bool ok = true;
     for (int i = 0; i < g.n_members; ++i)  // 16-byte L rows; 32-bit byte offsets inside every buffer of a member
       ok = ok && (g.mem[i].L == nullptr || aligned16(g.mem[i].L)) && (long)g.mem[i].N * g.mem[i].ldw * 4 < (1L << 31);

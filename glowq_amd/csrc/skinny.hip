@@ -240,7 +240,226 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
   }
 }
 
+// Second form of the kernel for K % 256 == 0 and group sizes of 128 and up.  A wave walks 256-deep super-blocks;
+// lane (column c, half h) owns the 64 contiguous bytes of row c that hold codes [256 sb + 128 h, +128): exactly one
+// quantisation group, so one scale and one zero-point per lane, column tile and super-block, and the four 16-byte loads
+// of a lane hit the same 128-byte line back to back (the first form touches every line in four separate blocks and
+// fetches scale and zero-point with every one of them).  The activations follow the same k assignment, but reach the
+// A operand through a wave-private LDS tile: the wave loads the 128-byte row segments of half a super-block in memory
+// order (8 lanes per segment, every line requested once per instruction) and reads the fragments back in MFMA lane
+// order.  Loading the fragments straight from memory (one 16-byte request per lane and line) cost 22 us of the 45 us
+// of a 28672 x 4096 layer at 32 rows: every request pulls a whole line out of L2.
+template <int kMT, int kNT>
+__global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves = blockDim.x >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+
+  SkinnyMember mem = g.mem[0];
+  int blk_base = 0;
+#define GLOWQ_PICK(i)                                          \
+  if (g.n_members > i && (int)blockIdx.x >= g.blk_end[i - 1]) { \
+    mem = g.mem[i];                                            \
+    blk_base = g.blk_end[i - 1];                               \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
+  const int n0 = ((int)blockIdx.x - blk_base) * (32 * kNT);
+
+  int ncol[kNT];
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) ncol[tn] = min(n0 + tn * 32 + ln, mem.N - 1);
+  int mrow[kMT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm) mrow[tm] = min(tm * 32 + ln, g.M - 1);
+
+  f16v acc[kMT][kNT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
+
+  // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
+  const bool corrected = mem.L != nullptr && g.r != nullptr;
+  if (corrected) {
+    const int lblocks = g.rank >> 6;
+    for (int jb = wave; jb < lblocks; jb += waves) {
+      const int kb = jb * 64;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        h8 af[kMT];
+#pragma unroll
+        for (int tm = 0; tm < kMT; ++tm)
+          af[tm] = *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kb + 32 * lh + 8 * t);
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) {
+          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kb + 32 * lh + 8 * t);
+#pragma unroll
+          for (int tm = 0; tm < kMT; ++tm) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf, acc[tm][tn], 0, 0, 0);
+        }
+      }
+    }
+    if (g.alpha != 1.0f) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= g.alpha;
+    }
+  }
+
+  // ---- phase 2: super-blocks of 256 columns, contiguous range per wave ---------------------------------------
+  struct BRegs {
+    u32x4 b[kNT * 4];  // a super-block in load order: row 8 q + lane / 8 of the column tile, piece lane % 8
+    uint32_t s[kNT], z[kNT];
+  };
+  struct ARegs {
+    u32x4 a[kMT * 8];  // half a super-block in load order: segment 8 q + lane / 8, piece lane % 8
+  };
+  constexpr int kSegStride = 144;                      // 128 bytes of a row segment + 16: conflict-free fragment reads
+  constexpr int kATile = kMT * 64 * kSegStride;        // bytes per wave
+  constexpr int kBTile = kNT * 32 * kSegStride;
+  unsigned char* atile = smem + (size_t)wave * (kATile + kBTile);
+  unsigned char* btile = atile + kATile;
+  const int sblocks = g.K >> 8;
+  const int per = (sblocks + waves - 1) / waves;
+  const int first = wave * per;
+  const int mine = max(0, min(per, sblocks - first));
+  uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point word of the super-block being computed
+  auto issue_b = [&](int i, BRegs& rb) {
+    const int sb = min(first + i, sblocks - 1);  // past-the-end prefetches re-read the last one
+    const int grp = (sb * 256 + lh * 128) >> g.gs_shift;
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = min(n0 + tn * 32 + q * 8 + (lane >> 3), mem.N - 1);
+        rb.b[tn * 4 + q] = *reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw + sb * 32 + (lane & 7) * 4);
+      }
+      rb.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
+      rb.z[tn] = (uint32_t)mem.qzeros[(size_t)ncol[tn] * mem.ldz + (grp >> 3)];
+    }
+  };
+  auto stage_b = [&](const BRegs& rb) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous super-block are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<u32x4*>(btile + (tn * 32 + q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = rb.b[tn * 4 + q];
+      cur_s[tn] = rb.s[tn];
+      cur_z[tn] = rb.z[tn];
+    }
+  };
+  auto issue_a = [&](int i, int jj, ARegs& ra) {  // jj: first or second half of every lane's 128 columns
+    const int kbase = min(first + i, sblocks - 1) * 256 + jj * 64 + (lane & 7) * 8;
+#pragma unroll
+    for (int q = 0; q < kMT * 8; ++q) {
+      const int seg = q * 8 + (lane >> 3);             // (token row, half of the super-block)
+      const int row = min(seg >> 1, g.M - 1);
+      // loads whose four token rows all lie past M are skipped: their accumulator rows are never stored
+      if (q * 4 < g.M) ra.a[q] = *reinterpret_cast<const u32x4*>(g.x + (size_t)row * g.K + kbase + (seg & 1) * 128);
+      else ra.a[q] = u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto stage_a = [&](const ARegs& ra) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous half are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < kMT * 8; ++q)
+      *reinterpret_cast<u32x4*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = ra.a[q];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto compute = [&](int i, int j) {
+    const int grp = ((first + i) * 256 + lh * 128) >> g.gs_shift;
+    h8 bf[kNT][4];
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      const half_t z = (half_t)(float)nibble(cur_z[tn], grp & 7);
+      const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
+      const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh};
+      const h2 s2 = bitcast_u32<h2>(cur_s[tn] | (cur_s[tn] << 16));
+      const u32x4 bw = *reinterpret_cast<const u32x4*>(btile + (tn * 32 + ln) * kSegStride + lh * 64 + j * 16);
+      bf[tn][0] = dequant_word_sk(bw.x, zb_lo, zb_hi, s2);
+      bf[tn][1] = dequant_word_sk(bw.y, zb_lo, zb_hi, s2);
+      bf[tn][2] = dequant_word_sk(bw.z, zb_lo, zb_hi, s2);
+      bf[tn][3] = dequant_word_sk(bw.w, zb_lo, zb_hi, s2);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm) {
+        const h8 af = nibble_order(*reinterpret_cast<const u32x4*>(atile + (((tm * 32 + ln) * 2 + lh) * kSegStride) + (4 * (j & 1) + t) * 16));
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf[tn][t], acc[tm][tn], 0, 0, 0);
+      }
+    }
+  };
+
+  // Weights one super-block ahead, activations half a super-block ahead, both in registers in load order and moved to
+  // the LDS tiles when their turn begins.  The weight loads go out behind the activation loads of the first half:
+  // waiting for those activations then leaves the weights in flight.
+#define GLOWQ_PIN_LOADS() asm volatile("" ::: "memory")
+  BRegs B;
+  ARegs A;
+  issue_b(0, B);
+  issue_a(0, 0, A);
+  GLOWQ_PIN_LOADS();
+  for (int i = 0; i < mine; ++i) {
+    stage_b(B); stage_a(A);
+    issue_a(i, 1, A); issue_b(i + 1, B); GLOWQ_PIN_LOADS();
+    compute(i, 0); compute(i, 1);
+    stage_a(A);
+    issue_a(i + 1, 0, A); GLOWQ_PIN_LOADS();
+    compute(i, 2); compute(i, 3);
+  }
+#undef GLOWQ_PIN_LOADS
+  __syncthreads();  // the reduction buffer below overlays the staging tiles
+
+  // ---- the waves' partial tiles meet in LDS: [wave][tm][tn][16 regs][64 lanes] floats --------------------------
+  float* red = reinterpret_cast<float*>(smem);
+  constexpr int kTile = kMT * kNT * 16 * 64;
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) red[(size_t)wave * kTile + ((tm * kNT + tn) * 16 + i) * 64 + lane] = acc[tm][tn][i];
+  __syncthreads();
+  const int slots = kMT * kNT * 16 * 64;
+  for (int sidx = threadIdx.x; sidx < slots; sidx += blockDim.x) {
+    float v = 0.f;
+    for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + sidx];
+    const int l = sidx & 63;
+    const int i = (sidx >> 6) & 15;
+    const int tt = sidx >> 10;
+    const int tm = tt / kNT, tn = tt - tm * kNT;
+    const int n = n0 + tn * 32 + (l & 31);
+    const int m = tm * 32 + 8 * (i >> 2) + 4 * (l >> 5) + (i & 3);
+    if (m < g.M && n < mem.N) {
+      const float b = mem.bias ? (float)mem.bias[n] : 0.f;
+      mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
+    }
+  }
+}
+
 // ---- host side ------------------------------------------------------------------------------------------
+// The second form needs whole 256-column super-blocks and one quantisation group per 128-column half.
+bool skinny_group_form(const GroupDev& g) {
+  static const int env_form = getenv("GLOWQ_SKINNY_FORM") ? atoi(getenv("GLOWQ_SKINNY_FORM")) : -1;
+  return (g.K & 255) == 0 && g.group_size >= 128 && env_form != 0;
+}
+
 bool skinny_supported(const GroupDev& g) {
   if (g.M < 1 || g.M > 64) return false;
   if ((g.K & 63) != 0 || (g.group_size & 31) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
@@ -255,10 +474,11 @@ bool skinny_supported(const GroupDev& g) {
   return true;
 }
 
-template <int kMT, int kNT>
+template <int kMT, int kNT, bool kGroupForm>
 static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) {
-  auto kern = skinny_mfma_kernel<kMT, kNT>;
-  const size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
+  auto kern = kGroupForm ? skinny_group_kernel<kMT, kNT> : skinny_mfma_kernel<kMT, kNT>;
+  size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
+  if (kGroupForm && lds < (size_t)waves * (kMT * 64 + kNT * 32) * 144) lds = (size_t)waves * (kMT * 64 + kNT * 32) * 144;
   static size_t configured = 48 * 1024;
   if (lds > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -275,7 +495,6 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) 
 }
 
 hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
-  (void)num_cus;
   SkinnyArgs a;
   a.x = g.x;
   a.r = g.r;
@@ -302,10 +521,35 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
   }
   static const int env_waves = getenv("GLOWQ_SKINNY_WAVES") ? atoi(getenv("GLOWQ_SKINNY_WAVES")) : 0;
   int waves = (env_waves >= 1 && env_waves <= 8) ? env_waves : 8;
+  if (skinny_group_form(g)) {
+    // two column tiles per wave halve the activation traffic, one gives twice the workgroups: the wide tile only
+    // where there are columns to fill the chip with it
+    long cols = 0;
+    for (int i = 0; i < g.n_members; ++i) cols += g.mem[i].N;
+    const bool wide = cols >= 64L * num_cus;
+    if (env_waves < 1) waves = wide ? 4 : (g.M <= 32 ? 8 : 6);  // staging tiles: 18 / 13.5 / 22.5 KB of LDS per wave
+    if (waves > (g.K >> 8)) waves = g.K >> 8;
+    if (g.M <= 32) return wide ? launch_skinny_t<1, 2, true>(a, waves, stream) : launch_skinny_t<1, 1, true>(a, waves, stream);
+    if (!wide) {
+      if (waves > 6) waves = 6;
+      return launch_skinny_t<2, 1, true>(a, waves, stream);  // 2 x 2 tiles do not fit the register file with the staging
+    }
+    // many columns and more than 32 rows: two passes of 32 rows over the wide tile beat one pass over the narrow one
+    for (int m0 = 0; m0 < g.M; m0 += 32) {
+      SkinnyArgs c = a;
+      c.M = g.M - m0 < 32 ? g.M - m0 : 32;
+      c.x = a.x + (size_t)m0 * g.K;
+      c.r = a.r ? a.r + (size_t)m0 * g.rank : nullptr;
+      for (int i = 0; i < g.n_members; ++i) c.mem[i].y = a.mem[i].y + (size_t)m0 * a.mem[i].ldy;
+      hipError_t e = launch_skinny_t<1, 2, true>(c, waves, stream);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   const int kblocks = g.K >> 6;
   if (waves > kblocks) waves = kblocks;
-  if (g.M <= 32) return launch_skinny_t<1, 2>(a, waves, stream);
-  return launch_skinny_t<2, 2>(a, waves, stream);
+  if (g.M <= 32) return launch_skinny_t<1, 2, false>(a, waves, stream);
+  return launch_skinny_t<2, 2, false>(a, waves, stream);
 }
 
 }  // namespace glowq
