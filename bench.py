@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[1]): the decode linears of a Llama-3.1-8B-shaped model at batch 1 --
+Workload (the headline configuration of the benchmark): the decode linears of a Llama-3.1-8B-shaped model at batch 1 --
 per layer the QKV group (N = 4096+1024+1024, K = 4096), o_proj (4096x4096), the gate|up group
 (N = 2 x 14336, K = 4096) and down_proj (K = 14336, N = 4096); int4 codes, asymmetric per-group scale and
 zero-point (g = 128), fp16 activations ~ N(0,1), shared rank-128 correction on every group.  One STEP is
@@ -252,7 +252,7 @@ def main():
         "dtype": "int4 weights x fp16 activations, fp32 accumulate",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE configs[1]: Llama-3.1-8B decode linears (qkv 6144x4096, o 4096x4096, gate|up 28672x4096, "
+            "workload": "Llama-3.1-8B decode linears (qkv 6144x4096, o 4096x4096, gate|up 28672x4096, "
                         "down 4096x14336), int4 g=128 asym, shared rank-128 correction, batch tokens 1, 32 layers of distinct weights",
             "tokens": M_TOKENS, "rank": RANK, "group_size": GROUP_SIZE, "layers": LAYERS,
             "launches_per_step": 2 * len(GROUPS) * LAYERS, "execution": "HIP graph replay",
