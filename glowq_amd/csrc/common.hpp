@@ -49,6 +49,21 @@ int fail(int code, const char* fmt, ...);
 // Compute units of the current device (cached).
 int num_cus();
 
+// Raises a kernel's dynamic LDS limit to `bytes` on the current device when that is above the 48 KB default and above
+// what this call site asked for before.  `raised` is the call site's own table (one slot per device).
+struct LdsLimit {
+  size_t raised[64] = {};
+};
+inline hipError_t ensure_dynamic_lds(const void* kernel, size_t bytes, LdsLimit& site) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  if (bytes <= site.raised[dev]) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) site.raised[dev] = bytes;
+  return e;
+}
+
 __device__ __forceinline__ uint32_t nibble(uint32_t word, int idx) { return (word >> (4 * idx)) & 0xFu; }
 
 template <typename T>

@@ -427,13 +427,8 @@ static hipError_t launch_rope_attend_t(const half_t* q, const half_t* k_new, con
                                        const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
                                        int heads, int kv_heads, int max_len, float scale, hipStream_t stream) {
   const size_t lds = rope_attend_lds(kD, max_len);
-  static size_t configured = 48 * 1024;
-  if (lds > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rope_attend_kernel<kD>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = lds;
-  }
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(rope_attend_kernel<kD>), lds, lds_limit); e != hipSuccess) return e;
   hipLaunchKernelGGL(rope_attend_kernel<kD>, dim3(heads), dim3(1024), lds, stream, q, k_new, v_new, cos_t, sin_t, pos,
                      cache_k, cache_v, out, heads, kv_heads, max_len, scale);
   return hipGetLastError();

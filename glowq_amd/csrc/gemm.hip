@@ -319,12 +319,8 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
   auto kern = gemm_mfma_kernel<kMT, kNT, kQuant>;
   const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t);
-  static bool configured = false;
-  if (!configured && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   const int m_blocks = (gg.m[0].M + BM - 1) / BM;
   int total = 0;
   for (int i = 0; i < gg.n; ++i) {
@@ -535,12 +531,8 @@ hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, 
   if (rank > 64 && wide) {
     constexpr int NT = 4;
     const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
-    static bool configured = false;
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return e;
-      configured = true;
-    }
+    static LdsLimit lds_limit;
+    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), lds, lds_limit); e != hipSuccess) return e;
     hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 127) / 128), dim3(256), lds, stream, x, R, r, M, K, rank);
   } else {
     constexpr int NT = 2;

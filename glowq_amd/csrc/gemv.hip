@@ -348,12 +348,8 @@ static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int m
                                     hipStream_t stream) {
   auto kern = gemv_wave_dot_kernel<kM, kRows, kLW, kWide>;
   const int threads = waves * kWave;
-  static size_t configured = 48 * 1024;  // largest dynamic LDS size this instantiation was raised to
-  if (lds > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = lds;
-  }
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   // resident workgroups per CU for this block size and LDS footprint; the last answer is remembered
   static int last_threads = 0, last_occ = 0;
   static size_t last_lds = 0;

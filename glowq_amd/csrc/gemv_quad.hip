@@ -417,12 +417,8 @@ static hipError_t launch_quad_t(const GroupDev& g, int kit, int num_cus, size_t 
   if (slices_env >= 1 && slices_env <= waves && waves % slices_env == 0 && slices_env <= kit) slices = slices_env;
   const int blocks_per_wg = waves / slices;
   const size_t lds = lds_base + (slices > 1 ? (size_t)2 * waves * kTok4 * 4 * sizeof(float) : 0);
-  static size_t configured = 48 * 1024;
-  if (lds > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = lds;
-  }
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   const int threads = waves * kWave;
   const int resident = num_cus * wg_per_cu;
   int wgs_needed = 0;

@@ -479,12 +479,8 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) 
   auto kern = kGroupForm ? skinny_group_kernel<kMT, kNT> : skinny_mfma_kernel<kMT, kNT>;
   size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
   if (kGroupForm && lds < (size_t)waves * (kMT * 64 + kNT * 32) * 144) lds = (size_t)waves * (kMT * 64 + kNT * 32) * 144;
-  static size_t configured = 48 * 1024;
-  if (lds > configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = lds;
-  }
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   int total = 0;
   for (int i = 0; i < a.n_members; ++i) {
     total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
