@@ -72,7 +72,12 @@ __device__ __forceinline__ h8 dequant_word(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2
 }
 
 // kQuant: B is the int4 weight (with the optional correction phase in front); otherwise B is plain fp16.
-template <int kMT, int kNT, bool kQuant>
+// kSuper (quantised B, K % 256 == 0, group sizes of 128 and up): the K loop walks 256-column super-blocks in which lane
+// (column c, half h) owns the 64 contiguous bytes of codes [256 sb + 128 h, +128) of its weight row -- one quantisation
+// group, one scale and zero-point per super-block -- and the weights reach the B operand through a wave-private LDS tile
+// that is filled in memory order (8 lanes per 128-byte row segment).  Fragment loads straight from memory, one 16-byte
+// request per lane and cache line, make every request pull a whole line out of L2.
+template <int kMT, int kNT, bool kQuant, bool kSuper = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
 void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   // member of this workgroup, picked with scalar selects from fixed kernel-argument offsets
@@ -197,7 +202,110 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   // ---- phase 2: the main K loop ---------------------------------------------------------------------
   const int steps = a.K / kBK;
   const int gs_shift = __builtin_ctz(a.group_size);  // group sizes on this route are powers of two
-  if constexpr (kQuant) {
+  if constexpr (kQuant && kSuper) {
+    // Sub-step ks = 4 sb + j covers columns {256 sb + 128 h + 32 j + [0, 32) : h = 0, 1}; the activation stage keeps
+    // its [BM][64] shape with octets 0-3 = half 0 and octets 4-7 = half 1, so the fragment reads do not change.
+    constexpr int kSeg = 144;  // bytes per row segment in the weight tile: 128 + 16, conflict-free fragment reads
+    unsigned char* btile = smem + (size_t)2 * BM * kARow * sizeof(half_t) + (size_t)wave * (32 * kNT) * kSeg;
+    auto load_a_sub = [&](ARegs& dst, int ks) {
+      const int kc = min(ks, steps - 1);
+      const int kbase = (kc >> 2) * 256 + (kc & 3) * 32;
+#pragma unroll
+      for (int i = 0; i < kMT; ++i) {
+        const int q = tid + 256 * i;
+        const int row = min(m0 + (q >> 3), a.M - 1);
+        const int oct = q & 7;
+        dst.v[i] = *reinterpret_cast<const u32x4*>(a.x + (size_t)row * a.K + kbase + (oct >> 2) * 128 + (oct & 3) * 8);
+      }
+    };
+    struct BLoad {
+      u32x4 w[kNT * 4];  // a super-block of the wave's 32 kNT weight rows in load order: row 8 q + lane / 8, piece lane % 8
+      uint32_t s[kNT], z[kNT];
+    };
+    uint32_t cur_s[kNT], cur_z[kNT];
+    auto issue_b = [&](int sb, BLoad& bl) {
+      const int sbc = min(sb, (steps >> 2) - 1);
+      const int grp = (sbc * 256 + lh * 128) >> gs_shift;
+#pragma unroll
+      for (int q = 0; q < kNT * 4; ++q) {
+        const int n = min(bn * BN + wave * (32 * kNT) + q * 8 + (lane >> 3), a.N - 1);
+        bl.w[q] = *reinterpret_cast<const u32x4*>(a.qweight + (size_t)n * a.ldw + sbc * 32 + (lane & 7) * 4);
+      }
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        bl.s[tn] = reinterpret_cast<const unsigned short*>(a.scales)[(size_t)ncol[tn] * a.lds + grp];
+        bl.z[tn] = (uint32_t)a.qzeros[(size_t)ncol[tn] * a.ldz + (grp >> 3)];
+      }
+    };
+    auto stage_b = [&](const BLoad& bl) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous super-block are done
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int q = 0; q < kNT * 4; ++q)
+        *reinterpret_cast<u32x4*>(btile + (q * 8 + (lane >> 3)) * kSeg + (lane & 7) * 16) = bl.w[q];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        cur_s[tn] = bl.s[tn];
+        cur_z[tn] = bl.z[tn];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    BLoad bl;
+    // j is a compile-time constant at every call site (the loop below is unrolled by four)
+    auto step = [&](int ks, int j, ARegs& a_fill, const ARegs& a_store) {
+      const int sb = ks >> 2;
+      if (j == 0) stage_b(bl);
+      const int grp = (sb * 256 + lh * 128) >> gs_shift;
+      u32x4 raw[kNT];
+      h2 zb_lo[kNT], zb_hi[kNT], s2[kNT];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        const half_t z = (half_t)(float)nibble(cur_z[tn], grp & 7);
+        const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
+        zb_lo[tn] = h2{zl, zl};
+        zb_hi[tn] = h2{zh, zh};
+        s2[tn] = bitcast_u32<h2>(cur_s[tn] | (cur_s[tn] << 16));
+        raw[tn] = *reinterpret_cast<const u32x4*>(btile + (tn * 32 + ln) * kSeg + lh * 64 + j * 16);
+      }
+      load_a_sub(a_fill, ks + 2);
+      if (j == 0) issue_b(sb + 1, bl);  // behind the activation loads: waiting for those leaves the weights in flight
+      // one code word per MFMA step is dequantised right before its MFMAs: 8 fragment registers live instead of 32
+      constexpr int kChunk = kMT < 4 ? kMT : 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        h8 bf[kNT];
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn) bf[tn] = dequant_word(raw[tn][t], zb_lo[tn], zb_hi[tn], s2[tn]);
+#pragma unroll
+        for (int c = 0; c < kMT; c += kChunk) {
+          h8 af[kChunk];
+#pragma unroll
+          for (int i = 0; i < kChunk; ++i) af[i] = read_a(stage, c + i, t);
+#pragma unroll
+          for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+            for (int i = 0; i < kChunk; ++i)
+              acc[c + i][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[tn], acc[c + i][tn], 0, 0, 0);
+        }
+      }
+      store_a_from(a_store, stage ^ 1, true);
+      __syncthreads();
+      stage ^= 1;
+    };
+    load_a_sub(areg, 0);
+    issue_b(0, bl);
+    load_a_sub(areg1, 1);
+    store_a_from(areg, stage, true);
+    __syncthreads();
+    for (int ks = 0; ks < steps; ks += 4) {  // steps is a multiple of 4 here
+      step(ks, 0, areg, areg1);
+      step(ks + 1, 1, areg1, areg);
+      step(ks + 2, 2, areg, areg1);
+      step(ks + 3, 3, areg1, areg);
+    }
+  } else if constexpr (kQuant) {
     // quantised B: per step and column tile one 16-byte load of codes, one scale, one zero-point word.
     // Two register sets alternate (no copies), and the prefetch of the next step is unconditional (the
     // last step re-reads its own block): a uniform number of loads per step keeps the wait counts exact,
@@ -314,11 +422,11 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-template <int kMT, int kNT, bool kQuant>
+template <int kMT, int kNT, bool kQuant, bool kSuper = false>
 static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
-  auto kern = gemm_mfma_kernel<kMT, kNT, kQuant>;
-  const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t);
+  auto kern = gemm_mfma_kernel<kMT, kNT, kQuant, kSuper>;
+  const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t) + (kSuper ? (size_t)4 * (32 * kNT) * 144 : 0);
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   const int m_blocks = (gg.m[0].M + BM - 1) / BM;
@@ -341,8 +449,11 @@ static hipError_t launch_gemm_group(GemmGroup& gg, hipStream_t stream) {
   static const int mt_max = getenv("GLOWQ_GEMM_MT") ? atoi(getenv("GLOWQ_GEMM_MT")) : 4;
   int mt = M > 128 ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
   if (mt > mt_max) mt = mt_max;
-#define GLOWQ_GEMM_CASE(MT, NT) \
-  if (mt == MT && nt == NT) return launch_gemm_t<MT, NT, true>(gg, stream);
+  static const int env_super = getenv("GLOWQ_GEMM_SUPER") ? atoi(getenv("GLOWQ_GEMM_SUPER")) : 1;
+  const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128;
+#define GLOWQ_GEMM_CASE(MT, NT)                                                            \
+  if (mt == MT && nt == NT)                                                                \
+    return super ? launch_gemm_t<MT, NT, true, true>(gg, stream) : launch_gemm_t<MT, NT, true>(gg, stream);
   GLOWQ_GEMM_CASE(8, 2) GLOWQ_GEMM_CASE(4, 2) GLOWQ_GEMM_CASE(2, 2) GLOWQ_GEMM_CASE(1, 2)
   GLOWQ_GEMM_CASE(8, 1) GLOWQ_GEMM_CASE(4, 1) GLOWQ_GEMM_CASE(2, 1) GLOWQ_GEMM_CASE(1, 1)
 #undef GLOWQ_GEMM_CASE
@@ -523,7 +634,6 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
 
 hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int num_cus,
                                    hipStream_t stream) {
-  (void)num_cus;
   if ((K % kBK) != 0 || K < kBK) return hipErrorInvalidValue;
   const int m_blocks = (M + 31) / 32;
   const size_t lds_x = (size_t)2 * 32 * kPRow * sizeof(half_t);
@@ -534,6 +644,11 @@ hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, 
     static LdsLimit lds_limit;
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), lds, lds_limit); e != hipSuccess) return e;
     hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 127) / 128), dim3(256), lds, stream, x, R, r, M, K, rank);
+  } else if (m_blocks * ((rank + 63) / 64) < num_cus && rank > 32) {
+    // too few workgroups with 64 columns each: 32 columns per workgroup double them (R is small, re-reading it is free)
+    constexpr int NT = 1;
+    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
+    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 31) / 32), dim3(256), lds, stream, x, R, r, M, K, rank);
   } else {
     constexpr int NT = 2;
     const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
