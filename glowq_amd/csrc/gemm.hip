@@ -439,16 +439,37 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   return hipGetLastError();
 }
 
-static hipError_t launch_gemm_group(GemmGroup& gg, hipStream_t stream) {
-  // row tiles per workgroup: the largest that M fills (capped: 4 keeps two workgroups per CU resident);
-  // column tiles: 2 per wave unless every member is narrow
+static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stream) {
+  // Tile choice: the largest tile (most reuse of both operands) whose workgroup count still fills the chip; when
+  // none does, the one with the most workgroups.  Row tiles are capped by M (and at 4: 8 spills), column tiles at
+  // 2 per wave unless every member is narrow.
   int n_max = 0;
   for (int i = 0; i < gg.n; ++i) n_max = gg.m[i].N > n_max ? gg.m[i].N : n_max;
-  const int nt = n_max > 128 ? 2 : 1;
+  const int nt_cap = n_max > 128 ? 2 : 1;
   const int M = gg.m[0].M;
   static const int mt_max = getenv("GLOWQ_GEMM_MT") ? atoi(getenv("GLOWQ_GEMM_MT")) : 4;
-  int mt = M > 128 ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
-  if (mt > mt_max) mt = mt_max;
+  int mt_cap = M > 128 ? 8 : (M > 64 ? 4 : (M > 32 ? 2 : 1));
+  if (mt_cap > mt_max) mt_cap = mt_max;
+  static const int order[6][2] = {{4, 2}, {2, 2}, {4, 1}, {2, 1}, {1, 2}, {1, 1}};
+  int mt = 1, nt = 1;
+  long best = -1;
+  for (int c = 0; c < 6; ++c) {
+    const int cmt = order[c][0], cnt = order[c][1];
+    if (cmt > mt_cap || cnt > nt_cap) continue;
+    long wgs = 0;
+    for (int i = 0; i < gg.n; ++i) wgs += (long)((M + 32 * cmt - 1) / (32 * cmt)) * ((gg.m[i].N + 128 * cnt - 1) / (128 * cnt));
+    if (wgs >= num_cus) {
+      mt = cmt;
+      nt = cnt;
+      break;
+    }
+    if (wgs > best) {
+      best = wgs;
+      mt = cmt;
+      nt = cnt;
+    }
+  }
+  if (mt_cap == 8 && mt == 4 && mt_max >= 8) mt = 8;
   static const int env_super = getenv("GLOWQ_GEMM_SUPER") ? atoi(getenv("GLOWQ_GEMM_SUPER")) : 1;
   const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128;
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
@@ -476,7 +497,6 @@ bool gemm_supported(const GroupDev& g) {
 }
 
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
-  (void)num_cus;
   GemmGroup gg;
   gg.n = g.n_members;
   for (int i = 0; i < g.n_members; ++i) {
@@ -502,7 +522,7 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
     a.ldy = m.ldy;
     a.alpha = g.alpha;
   }
-  return launch_gemm_group(gg, stream);
+  return launch_gemm_group(gg, num_cus, stream);
 }
 
 // ---- shared projection for many rows: r[M, rank] = fp16(x[M, K] . R[rank, K]^T) ---------------------------
