@@ -71,7 +71,8 @@ class Attention(nn.Module):
 
     def forward(self, x, cos, sin, cache_k, cache_v, pos_idx, mask):
         """x [T, hidden]; cos/sin [T, head_dim]; caches [kv_heads, max_len, head_dim]; pos_idx [T] (device,
-        positions of the T tokens); mask [T, max_len] additive."""
+        positions of the T tokens); mask [T, max_len] additive, or None when the T tokens are positions 0..T-1 of an
+        empty cache (prefill): attention then runs causally over the new keys alone."""
         cfg = self.cfg
         T = x.size(0)
         q = self.q_proj(x).view(T, cfg.heads, cfg.head_dim).transpose(0, 1)      # [H, T, d]
@@ -80,8 +81,11 @@ class Attention(nn.Module):
         q, k = _rope(q, cos, sin), _rope(k, cos, sin)
         cache_k.index_copy_(1, pos_idx, k.to(cache_k.dtype))
         cache_v.index_copy_(1, pos_idx, v.to(cache_v.dtype))
-        out = F.scaled_dot_product_attention(q.to(cache_k.dtype).unsqueeze(0), cache_k.unsqueeze(0), cache_v.unsqueeze(0),
-                                             attn_mask=mask.unsqueeze(0).unsqueeze(0), enable_gqa=True)
+        if mask is None:
+            out = F.scaled_dot_product_attention(q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0), is_causal=True, enable_gqa=True)
+        else:
+            out = F.scaled_dot_product_attention(q.to(cache_k.dtype).unsqueeze(0), cache_k.unsqueeze(0), cache_v.unsqueeze(0),
+                                                 attn_mask=mask.unsqueeze(0).unsqueeze(0), enable_gqa=True)
         out = out.squeeze(0).transpose(0, 1).reshape(T, cfg.heads * cfg.head_dim)
         return self.o_proj(out)
 
@@ -140,13 +144,16 @@ class Decoder(nn.Module):
         ang = torch.cat((ang, ang), dim=-1)
         return ang.cos(), ang.sin()
 
-    def forward_tokens(self, tokens, pos_idx, caches, cos_t, sin_t):
-        """tokens [T] (device), pos_idx [T] (device): logits [T, vocab] after writing the KV cache at pos_idx."""
+    def forward_tokens(self, tokens, pos_idx, caches, cos_t, sin_t, from_empty_cache: bool = False):
+        """tokens [T] (device), pos_idx [T] (device): logits [T, vocab] after writing the KV cache at pos_idx.
+        `from_empty_cache`: pos_idx is 0..T-1 and nothing older is cached, so attention needs no mask over the cache."""
         cfg = self.cfg
         x = self.model.embed_tokens(tokens)
         cos, sin = cos_t.index_select(0, pos_idx).to(x.dtype), sin_t.index_select(0, pos_idx).to(x.dtype)
-        col = torch.arange(cfg.max_len, device=tokens.device)
-        mask = torch.where(col[None, :] <= pos_idx[:, None], 0.0, float("-inf")).to(torch.float16)
+        mask = None
+        if not from_empty_cache:
+            col = torch.arange(cfg.max_len, device=tokens.device)
+            mask = torch.where(col[None, :] <= pos_idx[:, None], 0.0, float("-inf")).to(torch.float16)
         for layer, (ck, cv) in zip(self.model.layers, caches):
             x = layer(x, cos, sin, ck, cv, pos_idx, mask)
         return self.lm_head(self.model.norm(x))
@@ -351,7 +358,7 @@ class GreedyDecoder:
     def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
         T = prompt.numel()
         pos = torch.arange(T, device=self.dev)
-        logits = self.model.forward_tokens(prompt.to(self.dev), pos, self.caches, self.cos, self.sin)
+        logits = self.model.forward_tokens(prompt.to(self.dev), pos, self.caches, self.cos, self.sin, from_empty_cache=True)
         return logits[-1].argmax().reshape(1)
 
     @torch.no_grad()

@@ -56,7 +56,7 @@ def evaluate_token_ids(model: Decoder, input_ids: torch.Tensor, seq_len: int = 2
             continue
         window = input_ids[begin:end].to(dev)
         pos = torch.arange(end - begin, device=dev)
-        logits = model.forward_tokens(window, pos, dec.caches, dec.cos, dec.sin)
+        logits = model.forward_tokens(window, pos, dec.caches, dec.cos, dec.sin, from_empty_cache=True)
         loss = F.cross_entropy(logits[:-1].float(), window[1:])
         n = end - begin - 1
         total_loss += float(loss) * n

@@ -91,6 +91,18 @@ def test_tiny_decoder_logits_match_effective_weight_network(fp16_out, T):
     assert np.abs(without - want).max() > 10 * max(err, 1e-3)
 
 
+def test_prefill_without_mask_matches_masked_path(fp16_out):
+    model, _, _ = decode.build_decoder(decode.DecoderConfig(**TINY), seed=12)
+    tokens = torch.randint(0, TINY["vocab"], (23,), generator=torch.Generator().manual_seed(3)).cuda()
+    pos = torch.arange(23, device="cuda")
+    a, b = decode.GreedyDecoder(model, use_graph=False), decode.GreedyDecoder(model, use_graph=False)
+    masked = model.forward_tokens(tokens, pos, a.caches, a.cos, a.sin).float()
+    causal = model.forward_tokens(tokens, pos, b.caches, b.cos, b.sin, from_empty_cache=True).float()
+    assert (masked - causal).abs().max() <= 2e-3 + 2e-3 * masked.abs().max()
+    for (ka, va), (kb, vb) in zip(a.caches, b.caches):          # both leave the same cache behind
+        assert (ka.float() - kb.float()).abs().max() <= 2e-3 and (va.float() - vb.float()).abs().max() <= 2e-3
+
+
 def test_graph_replay_matches_eager_decode(fp16_out):
     model, _, _ = decode.build_decoder(decode.DecoderConfig(**TINY), seed=6)
     prompt = torch.randint(0, TINY["vocab"], (9,), generator=torch.Generator().manual_seed(1))
