@@ -2,6 +2,8 @@
 // decode: residual add + RMSNorm, rotary embedding + KV-cache append + attention of one query token over the
 // cache, SwiGLU gating, greedy pick.  Plain HBM/L2-latency-bound kernels; they exist so that a decode step is
 // a short chain of launches that a HIP graph can replay, not to be clever.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace glowq {
@@ -213,8 +215,8 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
                                                             const half_t* __restrict__ v_new, const float* __restrict__ cos_t,
                                                             const float* __restrict__ sin_t, const long* __restrict__ pos_p,
                                                             half_t* __restrict__ cache_k, half_t* __restrict__ cache_v,
-                                                            half_t* __restrict__ out, int heads, int kv_heads, int max_len,
-                                                            float scale) {
+                                                            half_t* __restrict__ out, float* __restrict__ part, int heads,
+                                                            int kv_heads, int max_len, float scale) {
   constexpr int d = kD;
   constexpr int kLanes = d / 8;           // lanes per cache row
   constexpr int kRowsPerWave = 64 / kLanes;
@@ -230,6 +232,12 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
   const int rep = heads / kv_heads;
   const int kvh = head / rep;
   const int pos = (int)*pos_p;
+  // context split: workgroup (head, s) of gridDim.y takes the cached positions [pb, pe); the last split also takes the
+  // token itself.  With a split the unnormalised partial {max, sum, acc[d]} goes to `part`, else the result to `out`.
+  const int splits = gridDim.y, split = blockIdx.y;
+  const int chunk = (pos + splits - 1) / splits;
+  const int pb = min(split * chunk, pos), pe = min(pb + chunk, pos);
+  const bool own = split == splits - 1;
   constexpr int half_d = d >> 1;
   const int nw = blockDim.x >> 6;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
@@ -251,7 +259,7 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
     const half_t v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
     vn[i] = (float)v0;
     vn[i + half_d] = (float)v1;
-    if (head == kvh * rep) {
+    if (head == kvh * rep && split == 0) {
       half_t* ck = cache_k + ((size_t)kvh * max_len + pos) * d;
       half_t* cv = cache_v + ((size_t)kvh * max_len + pos) * d;
       ck[i] = r0; ck[i + half_d] = r1;
@@ -264,12 +272,12 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
 #pragma unroll
   for (int j = 0; j < 8; ++j) qv[j] = qs[8 * sub + j];
 
-  // scores of the cached positions [0, pos)
+  // scores of the cached positions [pb, pe)
   const half_t* kbase = cache_k + (size_t)kvh * max_len * d + 8 * sub;
-  for (int p0 = row0; p0 < pos; p0 += kUnroll * row_step) {
+  for (int p0 = pb + row0; p0 < pe; p0 += kUnroll * row_step) {
     h8 kv[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) kv[u] = *reinterpret_cast<const h8*>(kbase + (size_t)min(p0 + u * row_step, pos - 1) * d);
+    for (int u = 0; u < kUnroll; ++u) kv[u] = *reinterpret_cast<const h8*>(kbase + (size_t)min(p0 + u * row_step, pe - 1) * d);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       float dot = 0.f;
@@ -277,24 +285,28 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
       for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qv[j], (float)kv[u][j], dot);
       dot = row_group_sum<kLanes>(dot);
       const int p = p0 + u * row_step;
-      if (sub == 0 && p < pos) sc[p] = dot * scale;
+      if (sub == 0 && p < pe) sc[p] = dot * scale;
     }
   }
-  if (threadIdx.x == 0) {  // this token against itself
+  if (threadIdx.x == 0 && own) {  // this token against itself
     float dot = 0.f;
     for (int i = 0; i < d; ++i) dot = __builtin_fmaf(qs[i], kn[i], dot);
     sc[pos] = dot * scale;
   }
   __syncthreads();
+  // positions of this workgroup: pb..pe-1, and pos itself for the last split (index pe when pe == pos)
+  const int plast = own ? pos : pe - 1;
   float mx = -INFINITY;
-  for (int p = threadIdx.x; p <= pos; p += blockDim.x) mx = fmaxf(mx, sc[p]);
+  for (int p = pb + threadIdx.x; p <= plast; p += blockDim.x)
+    if (p < pe || p == pos) mx = fmaxf(mx, sc[p]);
   mx = block_max(mx, red, nw);
   float sum = 0.f;
-  for (int p = threadIdx.x; p <= pos; p += blockDim.x) {
-    const float e = __expf(sc[p] - mx);
-    sc[p] = e;
-    sum += e;
-  }
+  for (int p = pb + threadIdx.x; p <= plast; p += blockDim.x)
+    if (p < pe || p == pos) {
+      const float e = __expf(sc[p] - mx);
+      sc[p] = e;
+      sum += e;
+    }
   sum = block_sum(sum, red, nw);  // its barriers also publish sc[]
   const float inv = 1.f / sum;
 
@@ -303,19 +315,19 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int p0 = row0; p0 < pos; p0 += kUnroll * row_step) {
+  for (int p0 = pb + row0; p0 < pe; p0 += kUnroll * row_step) {
     h8 vv[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) vv[u] = *reinterpret_cast<const h8*>(vbase + (size_t)min(p0 + u * row_step, pos - 1) * d);
+    for (int u = 0; u < kUnroll; ++u) vv[u] = *reinterpret_cast<const h8*>(vbase + (size_t)min(p0 + u * row_step, pe - 1) * d);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int p = p0 + u * row_step;
-      const float pr = p < pos ? sc[p] : 0.f;
+      const float pr = p < pe ? sc[p] : 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, (float)vv[u][j], acc[j]);
     }
   }
-  if (wave == 0 && rg == 0) {  // this token's own value
+  if (wave == 0 && rg == 0 && own) {  // this token's own value
     const float pr = sc[pos];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, vn[8 * sub + j], acc[j]);
@@ -331,10 +343,59 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
     for (int j = 0; j < 8; ++j) acc_part[wave * d + 8 * sub + j] = acc[j];
   }
   __syncthreads();
+  float* mine = part ? part + ((size_t)head * splits + split) * (d + 2) : nullptr;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float t = 0.f;
     for (int w = 0; w < nw; ++w) t += acc_part[w * d + i];
-    out[(size_t)head * d + i] = (half_t)(t * inv);
+    if (part) mine[2 + i] = t;
+    else out[(size_t)head * d + i] = (half_t)(t * inv);
+  }
+  if (part && threadIdx.x == 0) {
+    mine[0] = mx;   // -inf for an empty split: its weight in the combination is exp(-inf) = 0
+    mine[1] = sum;
+  }
+}
+
+// Combines the split partials of rope_attend_kernel into out [heads * d] fp16 and, with R, also computes the shared
+// projection r[j] = out . R[j] of the group that consumes it: one workgroup per row of R recomputes the combination
+// (the partials are a few tens of KB) and writes 8-element chunks of `out` dealt round robin, as the other fused
+// glue kernels do.  Without R a few workgroups just write their chunks.
+__global__ __launch_bounds__(256) void attend_combine_proj_kernel(const float* __restrict__ part, half_t* __restrict__ out,
+                                                                  const half_t* __restrict__ R, half_t* __restrict__ r,
+                                                                  int heads, int d, int splits) {
+  __shared__ float red[16];
+  const int j = blockIdx.x, nwg = gridDim.x;
+  const int n = heads * d, chunks = n >> 3;
+  const int nw = blockDim.x >> 6;
+  float dot = 0.f;
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    const int head = (c << 3) / d, i0 = (c << 3) - head * d;
+    const float* ph = part + (size_t)head * splits * (d + 2);
+    float mx = -INFINITY;
+    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ph[s * (d + 2)]);
+    float den = 0.f, acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float w = __expf(ph[s * (d + 2)] - mx);
+      den = __builtin_fmaf(w, ph[s * (d + 2) + 1], den);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, ph[s * (d + 2) + 2 + i0 + e], acc[e]);
+    }
+    const float inv = 1.f / den;
+    h8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (half_t)(acc[e] * inv);
+    if (R) {
+      const h8 rr = reinterpret_cast<const h8*>(R + (size_t)j * n)[c];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot = __builtin_fmaf((float)o[e], (float)rr[e], dot);
+    }
+    if (c % nwg == j) reinterpret_cast<h8*>(out)[c] = o;
+  }
+  if (R) {
+    dot = block_sum(dot, red, nw);
+    if (threadIdx.x == 0) r[j] = (half_t)dot;
   }
 }
 
@@ -425,23 +486,35 @@ size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 16 * d
 template <int kD>
 static hipError_t launch_rope_attend_t(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
                                        const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
-                                       int heads, int kv_heads, int max_len, float scale, hipStream_t stream) {
+                                       float* part, int splits, int heads, int kv_heads, int max_len, float scale,
+                                       hipStream_t stream) {
   const size_t lds = rope_attend_lds(kD, max_len);
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(rope_attend_kernel<kD>), lds, lds_limit); e != hipSuccess) return e;
-  hipLaunchKernelGGL(rope_attend_kernel<kD>, dim3(heads), dim3(1024), lds, stream, q, k_new, v_new, cos_t, sin_t, pos,
-                     cache_k, cache_v, out, heads, kv_heads, max_len, scale);
+  static const int env_threads = getenv("GLOWQ_ATTEND_THREADS") ? atoi(getenv("GLOWQ_ATTEND_THREADS")) : 0;
+  const int threads = (env_threads >= 64 && env_threads <= 1024 && env_threads % 64 == 0) ? env_threads : 1024;
+  hipLaunchKernelGGL(rope_attend_kernel<kD>, dim3(heads, splits), dim3(threads), lds, stream, q, k_new, v_new,
+                     cos_t, sin_t, pos, cache_k, cache_v, out, part, heads, kv_heads, max_len, scale);
   return hipGetLastError();
 }
 
 hipError_t launch_rope_attend(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
-                              const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out,
-                              int heads, int kv_heads, int d, int max_len, float scale, hipStream_t stream) {
+                              const float* sin_t, const long* pos, half_t* cache_k, half_t* cache_v, half_t* out, float* part,
+                              int splits, int heads, int kv_heads, int d, int max_len, float scale, hipStream_t stream) {
   if (d == 128)
-    return launch_rope_attend_t<128>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, heads, kv_heads, max_len, scale, stream);
+    return launch_rope_attend_t<128>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, part, splits, heads, kv_heads,
+                                     max_len, scale, stream);
   if (d == 64)
-    return launch_rope_attend_t<64>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, heads, kv_heads, max_len, scale, stream);
+    return launch_rope_attend_t<64>(q, k_new, v_new, cos_t, sin_t, pos, cache_k, cache_v, out, part, splits, heads, kv_heads,
+                                    max_len, scale, stream);
   return hipErrorInvalidValue;
+}
+
+hipError_t launch_attend_combine_proj(const float* part, half_t* out, const half_t* R, half_t* r, int heads, int d, int splits,
+                                      int rank, hipStream_t stream) {
+  const int wgs = R ? rank : 32;
+  hipLaunchKernelGGL(attend_combine_proj_kernel, dim3(wgs), dim3(256), 0, stream, part, out, R, r, heads, d, splits);
+  return hipGetLastError();
 }
 
 hipError_t launch_argmax_advance(const half_t* logits, int n, long* next_tok, long* tok, long* pos, hipStream_t stream) {
@@ -505,9 +578,39 @@ int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const
     return fail(GLOWQ_EUNSUPPORTED, "rope_attend: max_len %d does not fit the score buffer in LDS", max_len);
   hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),
                                     cos_table, sin_table, reinterpret_cast<const long*>(pos), static_cast<half_t*>(cache_k),
-                                    static_cast<half_t*>(cache_v), static_cast<half_t*>(out), heads, kv_heads, head_dim, max_len, scale,
-                                    static_cast<hipStream_t>(stream));
+                                    static_cast<half_t*>(cache_v), static_cast<half_t*>(out), nullptr, 1, heads, kv_heads, head_dim,
+                                    max_len, scale, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "rope_attend launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_rope_attend_split(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
+                            const int64_t* pos, void* cache_k, void* cache_v, float* partials, int splits, int heads,
+                            int kv_heads, int head_dim, int max_len, float scale, void* stream) {
+  if (!q || !k_new || !v_new || !cos_table || !sin_table || !pos || !cache_k || !cache_v || !partials)
+    return fail(GLOWQ_EINVAL, "rope_attend_split: all pointers must be device pointers");
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || max_len <= 0 || splits < 1 || splits > 64)
+    return fail(GLOWQ_EINVAL, "rope_attend_split: heads a positive multiple of kv_heads, 1..64 splits (got %d, %d, %d)", heads,
+                kv_heads, splits);
+  if (head_dim != 64 && head_dim != 128)
+    return fail(GLOWQ_EUNSUPPORTED, "rope_attend_split: head_dim must be 64 or 128 (got %d)", head_dim);
+  if (rope_attend_lds(head_dim, max_len) > 160 * 1024)
+    return fail(GLOWQ_EUNSUPPORTED, "rope_attend_split: max_len %d does not fit the score buffer in LDS", max_len);
+  hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),
+                                    cos_table, sin_table, reinterpret_cast<const long*>(pos), static_cast<half_t*>(cache_k),
+                                    static_cast<half_t*>(cache_v), nullptr, partials, splits, heads, kv_heads, head_dim, max_len,
+                                    scale, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "rope_attend_split launch failed: %s", hipGetErrorString(e));
+}
+
+int glowq_attend_combine_proj(const float* partials, void* out, const void* R, void* r, int heads, int head_dim, int splits,
+                              int rank, void* stream) {
+  if (!partials || !out) return fail(GLOWQ_EINVAL, "attend_combine_proj: partials and out must be device pointers");
+  if ((R == nullptr) != (r == nullptr)) return fail(GLOWQ_EINVAL, "attend_combine_proj: R and r go together");
+  if (heads <= 0 || head_dim <= 0 || (head_dim & 7) || splits < 1 || (R && rank <= 0))
+    return fail(GLOWQ_EINVAL, "attend_combine_proj: bad sizes (heads %d, head_dim %d, splits %d, rank %d)", heads, head_dim, splits, rank);
+  hipError_t e = launch_attend_combine_proj(partials, static_cast<half_t*>(out), static_cast<const half_t*>(R), static_cast<half_t*>(r),
+                                            heads, head_dim, splits, rank, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? GLOWQ_OK : fail(GLOWQ_ELAUNCH, "attend_combine_proj launch failed: %s", hipGetErrorString(e));
 }
 
 int glowq_argmax_advance(const void* logits, int n, int64_t* next_token, int64_t* token, int64_t* pos, void* stream) {

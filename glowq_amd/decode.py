@@ -223,7 +223,7 @@ class FusedStep:
     Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
     the one-call projection + group entry point, o_proj and down_proj as solo groups."""
 
-    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True):
+    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 1):
         cfg = model.cfg
         self.share = share  # False: every module projects x on R by itself and launches alone (the no-sharing comparator)
         self.model, self.cfg = model, cfg
@@ -243,6 +243,10 @@ class FusedStep:
         self.act = torch.zeros(1, cfg.intermediate, **f16)
         self.dn = torch.zeros(1, cfg.hidden, **f16)
         self.logits = torch.zeros(1, cfg.vocab, **f16)
+        # context split per head: measured slower than one workgroup per head up to ~800 cached tokens (2.45 vs 2.37 ms per
+        # token at 4 splits); meant for long contexts
+        self.splits = attention_splits
+        self.partials = torch.zeros(cfg.heads, attention_splits, cfg.head_dim + 2, dtype=torch.float32, device=dev)
         self.scale = cfg.head_dim ** -0.5
         self.plan = []
         for layer in model.model.layers:
@@ -305,8 +309,16 @@ class FusedStep:
         for lay, (ck, cv) in zip(self.plan, self.caches):
             x, ready = self._norm(x, delta, lay["ln1"], lay["qkv"])
             self._linear(self.h, lay["qkv"], ready)
-            ext.rope_attend(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.attn, self.scale)
-            self._linear(self.attn, lay["o"])
+            o = lay["o"]
+            if self.splits > 1:
+                # the context split over several workgroups per head; the merge also projects the result on o_proj's R
+                ext.rope_attend_split(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.partials, self.scale)
+                ready = self.share and o["R"] is not None
+                ext.attend_combine_proj(self.partials, self.attn, o["R"] if ready else None, o["r"] if ready else None)
+                self._linear(self.attn, o, ready)
+            else:
+                ext.rope_attend(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.attn, self.scale)
+                self._linear(self.attn, o)
             x, ready = self._norm(x, self.o, lay["ln2"], lay["gu"])
             self._linear(self.h, lay["gu"], ready)
             gate, up, down = self.gu[:, :cfg.intermediate], self.gu[:, cfg.intermediate:], lay["down"]

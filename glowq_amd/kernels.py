@@ -56,6 +56,8 @@ _SIGNATURES = {
     "glowq_add_rmsnorm_proj": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
     "glowq_silu_mul_proj": (_I, [_P, _P, _P, _P, _P, _I, _I, _P]),
     "glowq_rope_attend": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_rope_attend_split": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_attend_combine_proj": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "glowq_argmax_advance": (_I, [_P, _I, _P, _P, _P, _P]),
 }
 
@@ -323,6 +325,47 @@ class W4A16Extension:
                                             out.data_ptr(), heads, kv_heads, d, max_len, float(scale), self._stream(q.device))
         if rc:
             self._raise(rc, "rope_attend")
+
+    def rope_attend_split(self, q, k_new, v_new, cos_table, sin_table, pos, cache_k, cache_v, partials, scale: float) -> None:
+        """As rope_attend, with the context split over partials.size(1) workgroups per head; partials is a
+        [heads, splits, d + 2] fp32 buffer that receives {max, sum, unnormalised acc} of every split."""
+        for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new"), (cache_k, "cache_k"), (cache_v, "cache_v")):
+            self._f16(t, n)
+        kv_heads, max_len, d = cache_k.shape
+        heads = q.numel() // d
+        _check(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and partials.dim() == 3
+               and partials.size(0) == heads and partials.size(2) == d + 2, "rope_attend_split: partials must be fp32 [heads, splits, d + 2]")
+        _check(cos_table.dtype == torch.float32 and cos_table.is_contiguous() and sin_table.dtype == torch.float32
+               and sin_table.is_contiguous() and tuple(cos_table.shape) == (max_len, d) and sin_table.shape == cos_table.shape,
+               "rope_attend_split: tables must be contiguous CUDA fp32 [max_len, d]")
+        _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "rope_attend_split: pos must be one int64 on the device")
+        _check(cache_v.shape == cache_k.shape and k_new.numel() == kv_heads * d and v_new.numel() == kv_heads * d,
+               "rope_attend_split: shape mismatch")
+        with torch.cuda.device(q.device):
+            rc = self.lib.glowq_rope_attend_split(q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), cos_table.data_ptr(),
+                                                  sin_table.data_ptr(), pos.data_ptr(), cache_k.data_ptr(), cache_v.data_ptr(),
+                                                  partials.data_ptr(), partials.size(1), heads, kv_heads, d, max_len, float(scale),
+                                                  self._stream(q.device))
+        if rc:
+            self._raise(rc, "rope_attend_split")
+
+    def attend_combine_proj(self, partials, out, R=None, r=None) -> None:
+        """out [heads * d] fp16 from the split partials; with R [rank, heads * d] also r = out R^T ([rank] fp16)."""
+        self._f16(out, "out")
+        heads, splits, d2 = partials.shape
+        d = d2 - 2
+        _check(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and out.numel() == heads * d,
+               "attend_combine_proj: partials fp32 [heads, splits, d + 2], out [heads * d]")
+        _check((R is None) == (r is None), "attend_combine_proj: R and r go together")
+        if R is not None:
+            self._f16(R, "R"), self._f16(r, "r")
+            _check(R.dim() == 2 and R.size(1) == heads * d and r.numel() == R.size(0), "attend_combine_proj: R [rank, heads * d], r [rank]")
+        with torch.cuda.device(out.device):
+            rc = self.lib.glowq_attend_combine_proj(partials.data_ptr(), out.data_ptr(), R.data_ptr() if R is not None else None,
+                                                    r.data_ptr() if r is not None else None, heads, d, splits,
+                                                    R.size(0) if R is not None else 0, self._stream(out.device))
+        if rc:
+            self._raise(rc, "attend_combine_proj")
 
     def argmax_advance(self, logits, next_token, token=None, pos=None) -> None:
         """next_token[0] = first argmax of logits; then token[0] = next_token[0] and pos[0] += 1 when given."""

@@ -167,6 +167,18 @@ int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const
                       const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,
                       int max_len, float scale, void* stream);
 
+/*
+ * The same with the context split over `splits` workgroups per head: each writes its unnormalised partial
+ * {max, sum, acc[d]} to partials [heads, splits, d + 2] fp32 (caller's buffer).  glowq_attend_combine_proj merges them
+ * into out [heads * d] fp16 and, when R [rank, heads * d] is given, also writes r = out R^T ([rank] fp16) for the group
+ * that consumes the attention output -- the o_proj group then needs no projection launch.
+ */
+int glowq_rope_attend_split(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
+                            const int64_t* pos, void* cache_k, void* cache_v, float* partials, int splits, int heads,
+                            int kv_heads, int head_dim, int max_len, float scale, void* stream);
+int glowq_attend_combine_proj(const float* partials, void* out, const void* R, void* r, int heads, int head_dim, int splits,
+                              int rank, void* stream);
+
 /* *next_token = index of the first maximum of logits[0..n); then *token = *next_token and *pos += 1 (each if non-NULL). */
 int glowq_argmax_advance(const void* logits, int n, int64_t* next_token, int64_t* token, int64_t* pos, void* stream);
 

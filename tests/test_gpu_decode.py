@@ -202,6 +202,37 @@ def test_rope_attend_matches_torch(ext, fp16_out, pos):
     assert torch.equal(ck2[:, keep], ck[:, keep]) and torch.equal(cv2[:, keep], cv[:, keep])   # nothing else touched
 
 
+@pytest.mark.parametrize("pos,splits", [(0, 4), (1, 4), (3, 8), (37, 4), (300, 4), (300, 7)])
+def test_split_attention_and_merge_match_single_workgroup(ext, fp16_out, pos, splits):
+    heads, kvh, d, max_len, rank = 8, 2, 128, 320, 64
+    g = torch.Generator(device="cuda").manual_seed(100 + pos)
+    q = torch.randn(heads * d, device="cuda", generator=g).half()
+    k = torch.randn(kvh * d, device="cuda", generator=g).half()
+    v = torch.randn(kvh * d, device="cuda", generator=g).half()
+    ck = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    cv = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    R = (torch.randn(rank, heads * d, device="cuda", generator=g) * (heads * d) ** -0.5).half()
+    model = decode.Decoder(decode.DecoderConfig(hidden=heads * d, layers=0, heads=heads, kv_heads=kvh, head_dim=d, intermediate=64,
+                                                vocab=8, max_len=max_len))
+    cos, sin = model.rope_tables("cuda")
+    p = torch.tensor([pos], device="cuda")
+    ck1, cv1, want = ck.clone(), cv.clone(), torch.empty(heads * d, dtype=torch.float16, device="cuda")
+    ext.rope_attend(q, k, v, cos, sin, p, ck1, cv1, want, d ** -0.5)
+    ck2, cv2 = ck.clone(), cv.clone()
+    part = torch.full((heads, splits, d + 2), float("nan"), device="cuda")
+    got, r = torch.empty_like(want), torch.empty(rank, dtype=torch.float16, device="cuda")
+    ext.rope_attend_split(q, k, v, cos, sin, p, ck2, cv2, part, d ** -0.5)
+    ext.attend_combine_proj(part, got, R, r)
+    torch.cuda.synchronize()
+    assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+    assert (got.float() - want.float()).abs().max() <= 1e-3 + 2e-3 * want.float().abs().max()
+    r_ref = ext.shared_proj(got.reshape(1, -1), R).reshape(-1)
+    assert (r.float() - r_ref.float()).abs().max() <= 1e-3 + 2e-3 * r_ref.float().abs().max()
+    plain = torch.empty_like(want)
+    ext.attend_combine_proj(part, plain)                      # without R: only the merge
+    assert torch.equal(plain, got)
+
+
 def test_fused_step_matches_module_path(fp16_out):
     cfg = decode.DecoderConfig(**TINY)
     model, _, _ = decode.build_decoder(cfg, seed=8)
@@ -223,6 +254,17 @@ def test_fused_step_matches_module_path(fp16_out):
     # without sharing (one projection and one launch per module) the step computes the same tokens
     alone, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True, share=False).generate(prompt, 10)
     assert torch.equal(alone, decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)[0])
+    # the context split over 3 workgroups per head merges to the same logits within tolerance
+    spl = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    spl.fused = decode.FusedStep(model, spl.caches, spl.cos, spl.sin, spl.tok, spl.pos, spl.next_tok, attention_splits=3)
+    spl.prefill(prompt)
+    spl.tok.copy_(first), spl.pos.fill_(prompt.numel())
+    spl.fused.run()
+    one = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    one.prefill(prompt)
+    one.tok.copy_(first), one.pos.fill_(prompt.numel())
+    one.fused.run()
+    assert (spl.fused.logits.float() - one.fused.logits.float()).abs().max() <= 1e-2
     # the captured fused step replays to the same tokens as the eager fused step
     eager, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)
     graphed = decode.GreedyDecoder(model, use_graph=True, fused=True)
