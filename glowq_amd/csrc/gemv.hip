@@ -27,9 +27,8 @@ __host__ __device__ inline size_t wave_dot_r_offset(int M, int K) {
   return (off + 15) & ~(size_t)15;
 }
 
-// partial sums of the slice waves: [2 parities][row blocks per workgroup][slices][rows x tokens] floats;
-
-__host__ __device__ inline size_t wave_dot_part_offset(int M, int K, int rank) {
+// Total LDS bytes of a workgroup: the above plus M rows of r.
+__host__ __device__ inline size_t wave_dot_lds_total(int M, int K, int rank) {
   return (wave_dot_r_offset(M, K) + (size_t)M * rank * sizeof(half_t) + 15) & ~(size_t)15;
 }
 
@@ -324,7 +323,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const GroupDev g) {
 
 // ---- host launchers ---------------------------------------------------------------------
 size_t wave_dot_lds_bytes(int M, int K, int rank, bool has_r) {
-  return wave_dot_part_offset(M, K, has_r ? rank : 0);
+  return wave_dot_lds_total(M, K, has_r ? rank : 0);
 }
 
 static int env_int(const char* name, int fallback) {
