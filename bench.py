@@ -226,6 +226,33 @@ def main():
         by = algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK)
         per_group[name] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
 
+    # the same layers at more token rows per call (batched decode): reported next to the metric, not part of it;
+    # 8 layers of distinct weights (1 GB) per replay keep the last-level cache out of the picture
+    batched = {}
+    for rows in (4, 16, 64):
+        xb = {name: torch.randn(rows, K, device=dev, generator=g).half() for name, (K, _) in GROUPS.items()}
+        rb = torch.empty(rows, RANK, dtype=torch.float16, device=dev)
+        ob = {name: [torch.empty(rows, N, dtype=torch.float16, device=dev) for N in Ns] for name, (_, Ns) in GROUPS.items()}
+        gb = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            for name in GROUPS:  # outside the capture first: kernel attributes of the routes these shapes take
+                ext.group_forward(xb[name], rb, layers[0][name][0], GROUP_SIZE, 1.0, outs=ob[name], R=layers[0][name][1])
+            torch.cuda.synchronize()
+            with torch.cuda.graph(gb, stream=side):
+                for layer in layers[:8]:
+                    for name in GROUPS:
+                        ext.group_forward(xb[name], rb, layer[name][0], GROUP_SIZE, 1.0, outs=ob[name], R=layer[name][1])
+        torch.cuda.synchronize()
+        gb.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            gb.replay()
+        b.record()
+        torch.cuda.synchronize()
+        batched[str(rows)] = round(a.elapsed_time(b) * 1e3 / 5 / 8, 2)
+
     if args.calibrate_copy:
         # cold sources: 8 distinct 256 MiB buffers, each copied once (the kernel shows up in a profile as
         # torch's elementwise copy kernel with 134217728 elements)
@@ -262,6 +289,7 @@ def main():
         "decode_tok_per_s_linears_only": round(1e3 / ms_per_step, 1),
         "algorithmic_bytes_per_layer": bytes_layer,
         "per_group": per_group,
+        "batched_rows_us_per_layer": batched,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",
