@@ -221,42 +221,68 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
   constexpr int kLanes = d / 8;           // lanes per cache row
   constexpr int kRowsPerWave = 64 / kLanes;
   constexpr int kUnroll = 4;
+  constexpr int half_d = d >> 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* qs = reinterpret_cast<float*>(smem_raw);            // [d] rotated query
   float* kn = qs + d;                                        // [d] rotated key of this token
   float* vn = kn + d;                                        // [d] value of this token
-  float* red = vn + d;                                       // [16]
-  float* acc_part = red + 16;                                // [waves][d]
-  float* sc = acc_part + 16 * d;                             // [max_len] scores / probabilities
+  float* wave_m = vn + d;                                    // [16] running maximum of each wave
+  float* wave_l = wave_m + 16;                               // [16] sum of exponentials of each wave
+  float* acc_part = wave_l + 16;                             // [waves][d]
   const int head = blockIdx.x;
   const int rep = heads / kv_heads;
   const int kvh = head / rep;
-  const int pos = (int)*pos_p;
-  // context split: workgroup (head, s) of gridDim.y takes the cached positions [pb, pe); the last split also takes the
-  // token itself.  With a split the unnormalised partial {max, sum, acc[d]} goes to `part`, else the result to `out`.
+  // context split: the cached positions are dealt to the gridDim.y workgroups of a head row by row, workgroup s taking
+  // s, s + splits, ...; the last one also takes the token itself.  Which rows a lane reads first therefore does not
+  // depend on the position, and those loads go out before anything else is known.  With a split the unnormalised
+  // partial {max, sum, -, -, acc[d]} goes to `part`, else the result to `out`.
   const int splits = gridDim.y, split = blockIdx.y;
-  const int chunk = (pos + splits - 1) / splits;
-  const int pb = min(split * chunk, pos), pe = min(pb + chunk, pos);
   const bool own = split == splits - 1;
-  constexpr int half_d = d >> 1;
   const int nw = blockDim.x >> 6;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
   const int sub = lane % kLanes, rg = lane / kLanes;
-  const int row0 = wave * kRowsPerWave + rg;      // first cache row of this lane group
+  const int row0 = wave * kRowsPerWave + rg;      // first of this lane group's rows (counted within the workgroup)
   const int row_step = nw * kRowsPerWave;
+  auto position = [&](int t) { return split + splits * t; };
+
+  // One pass over the rows with a running maximum (no score buffer): every lane group keeps {m, l, acc[8 of its
+  // dimensions]} for its own rows.  The key and the value row of a position are loaded together, one batch of kUnroll
+  // rows ahead of the batch being worked on.
+  const half_t* kbase = cache_k + (size_t)kvh * max_len * d + 8 * sub;
+  const half_t* vbase = cache_v + (size_t)kvh * max_len * d + 8 * sub;
+  struct Batch {
+    h8 k[kUnroll], v[kUnroll];
+  };
+  auto fetch = [&](int t, Batch& bt) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const size_t off = (size_t)min(position(t + u * row_step), max_len - 1) * d;  // rows past the position go unused
+      bt.k[u] = *reinterpret_cast<const h8*>(kbase + off);
+      bt.v[u] = *reinterpret_cast<const h8*>(vbase + off);
+    }
+  };
+  Batch b0, b1;
+  fetch(row0, b0);
+  float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
+  half_t v0 = (half_t)0.f, v1 = (half_t)0.f;
+  if (threadIdx.x < half_d) {
+    const int i = threadIdx.x;
+    q0 = (float)q[(size_t)head * d + i], q1 = (float)q[(size_t)head * d + i + half_d];
+    k0 = (float)k_new[(size_t)kvh * d + i], k1 = (float)k_new[(size_t)kvh * d + i + half_d];
+    v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
+  }
+  const int pos = (int)*pos_p;
 
   // rotary embedding of q and k_new: out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i + d/2] cos + x[i] sin
-  for (int i = threadIdx.x; i < half_d; i += blockDim.x) {
+  if (threadIdx.x < half_d) {
+    const int i = threadIdx.x;
     // the tables are rounded to fp16 first, as a half-precision model's rotary embedding does
-    const float c = (float)(half_t)cos_t[(size_t)pos * d + i], s = (float)(half_t)sin_t[(size_t)pos * d + i];
-    const float q0 = (float)q[(size_t)head * d + i], q1 = (float)q[(size_t)head * d + i + half_d];
-    qs[i] = (float)(half_t)(q0 * c - q1 * s);
-    qs[i + half_d] = (float)(half_t)(q1 * c + q0 * s);
-    const float k0 = (float)k_new[(size_t)kvh * d + i], k1 = (float)k_new[(size_t)kvh * d + i + half_d];
-    const half_t r0 = (half_t)(k0 * c - k1 * s), r1 = (half_t)(k1 * c + k0 * s);
+    const float c = (float)(half_t)cos_t[(size_t)pos * d + i], sn = (float)(half_t)sin_t[(size_t)pos * d + i];
+    qs[i] = (float)(half_t)(q0 * c - q1 * sn);
+    qs[i + half_d] = (float)(half_t)(q1 * c + q0 * sn);
+    const half_t r0 = (half_t)(k0 * c - k1 * sn), r1 = (half_t)(k1 * c + k0 * sn);
     kn[i] = (float)r0;
     kn[i + half_d] = (float)r1;
-    const half_t v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
     vn[i] = (float)v0;
     vn[i + half_d] = (float)v1;
     if (head == kvh * rep && split == 0) {
@@ -272,86 +298,99 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
 #pragma unroll
   for (int j = 0; j < 8; ++j) qv[j] = qs[8 * sub + j];
 
-  // scores of the cached positions [pb, pe)
-  const half_t* kbase = cache_k + (size_t)kvh * max_len * d + 8 * sub;
-  for (int p0 = pb + row0; p0 < pe; p0 += kUnroll * row_step) {
-    h8 kv[kUnroll];
+  float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) kv[u] = *reinterpret_cast<const h8*>(kbase + (size_t)min(p0 + u * row_step, pe - 1) * d);
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  auto fold = [&](int t, const Batch& bt) {
+    float sv[kUnroll];
+    float bm = m;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       float dot = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qv[j], (float)kv[u][j], dot);
+      for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qv[j], (float)bt.k[u][j], dot);
       dot = row_group_sum<kLanes>(dot);
-      const int p = p0 + u * row_step;
-      if (sub == 0 && p < pe) sc[p] = dot * scale;
+      sv[u] = (position(t + u * row_step) < pos) ? dot * scale : -INFINITY;
+      bm = fmaxf(bm, sv[u]);
     }
-  }
-  if (threadIdx.x == 0 && own) {  // this token against itself
-    float dot = 0.f;
-    for (int i = 0; i < d; ++i) dot = __builtin_fmaf(qs[i], kn[i], dot);
-    sc[pos] = dot * scale;
-  }
-  __syncthreads();
-  // positions of this workgroup: pb..pe-1, and pos itself for the last split (index pe when pe == pos)
-  const int plast = own ? pos : pe - 1;
-  float mx = -INFINITY;
-  for (int p = pb + threadIdx.x; p <= plast; p += blockDim.x)
-    if (p < pe || p == pos) mx = fmaxf(mx, sc[p]);
-  mx = block_max(mx, red, nw);
-  float sum = 0.f;
-  for (int p = pb + threadIdx.x; p <= plast; p += blockDim.x)
-    if (p < pe || p == pos) {
-      const float e = __expf(sc[p] - mx);
-      sc[p] = e;
-      sum += e;
-    }
-  sum = block_sum(sum, red, nw);  // its barriers also publish sc[]
-  const float inv = 1.f / sum;
-
-  // P.V over the cached positions, 8 dimensions per lane
-  const half_t* vbase = cache_v + (size_t)kvh * max_len * d + 8 * sub;
-  float acc[8];
+    // the first row of a batch is always a real one, so bm is finite here
+    const float keep = __expf(m - bm);
+    l *= keep;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int p0 = pb + row0; p0 < pe; p0 += kUnroll * row_step) {
-    h8 vv[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u) vv[u] = *reinterpret_cast<const h8*>(vbase + (size_t)min(p0 + u * row_step, pe - 1) * d);
+    for (int j = 0; j < 8; ++j) acc[j] *= keep;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      const int p = p0 + u * row_step;
-      const float pr = p < pe ? sc[p] : 0.f;
+      const float e = __expf(sv[u] - bm);
+      l += e;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, (float)vv[u][j], acc[j]);
+      for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(e, (float)bt.v[u][j], acc[j]);
+    }
+    m = bm;
+  };
+  {
+    const int step = kUnroll * row_step;
+    int t = row0;
+    while (position(t) < pos) {
+      const int t1 = t + step;
+      if (position(t1) < pos) fetch(t1, b1);
+      fold(t, b0);
+      if (position(t1) >= pos) break;
+      const int t2 = t1 + step;
+      if (position(t2) < pos) fetch(t2, b0);
+      fold(t1, b1);
+      t = t2;
     }
   }
-  if (wave == 0 && rg == 0 && own) {  // this token's own value
-    const float pr = sc[pos];
+  if (wave == 0 && rg == 0 && own) {  // this token against itself
+    float dot = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(pr, vn[8 * sub + j], acc[j]);
+    for (int j = 0; j < 8; ++j) dot = __builtin_fmaf(qv[j], kn[8 * sub + j], dot);
+    const float sv = row_group_sum<kLanes>(dot) * scale;
+    const float bm = fmaxf(m, sv);
+    const float keep = __expf(m - bm), e = __expf(sv - bm);
+    l = l * keep + e;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(e, vn[8 * sub + j], acc[j] * keep);
+    m = bm;
   }
-  // the lane groups of a wave, then the waves
+  // the lane groups of a wave meet through lane exchanges, the waves through LDS
+  {
+    float mw = m;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+    for (int o = kLanes; o < 64; o <<= 1) mw = fmaxf(mw, __shfl_xor(mw, o));
+    const float keep = (m == -INFINITY) ? 0.f : __expf(m - mw);
+    l *= keep;
 #pragma unroll
-    for (int o = kLanes; o < 64; o <<= 1) acc[j] += __shfl_xor(acc[j], o);
-  }
-  if (rg == 0) {
+    for (int o = kLanes; o < 64; o <<= 1) l += __shfl_xor(l, o);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc_part[wave * d + 8 * sub + j] = acc[j];
+    for (int j = 0; j < 8; ++j) {
+      acc[j] *= keep;
+#pragma unroll
+      for (int o = kLanes; o < 64; o <<= 1) acc[j] += __shfl_xor(acc[j], o);
+    }
+    if (rg == 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc_part[wave * d + 8 * sub + j] = acc[j];
+      if (sub == 0) {
+        wave_m[wave] = mw;
+        wave_l[wave] = l;
+      }
+    }
   }
   __syncthreads();
-  float* mine = part ? part + ((size_t)head * splits + split) * (d + 2) : nullptr;
+  float* mine = part ? part + ((size_t)head * splits + split) * (d + 4) : nullptr;
+  float mx = -INFINITY;
+  for (int w = 0; w < nw; ++w) mx = fmaxf(mx, wave_m[w]);
+  float sum = 0.f;
+  for (int w = 0; w < nw; ++w) sum += (wave_m[w] == -INFINITY) ? 0.f : wave_l[w] * __expf(wave_m[w] - mx);
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float t = 0.f;
-    for (int w = 0; w < nw; ++w) t += acc_part[w * d + i];
-    if (part) mine[2 + i] = t;
-    else out[(size_t)head * d + i] = (half_t)(t * inv);
+    for (int w = 0; w < nw; ++w) t += (wave_m[w] == -INFINITY) ? 0.f : acc_part[w * d + i] * __expf(wave_m[w] - mx);
+    if (part) mine[4 + i] = t;
+    else out[(size_t)head * d + i] = (half_t)(t / sum);
   }
   if (part && threadIdx.x == 0) {
-    mine[0] = mx;   // -inf for an empty split: its weight in the combination is exp(-inf) = 0
+    mine[0] = mx;   // -inf for a split without rows: its weight in the combination is exp(-inf) = 0
     mine[1] = sum;
   }
 }
@@ -360,34 +399,62 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
 // projection r[j] = out . R[j] of the group that consumes it: one workgroup per row of R recomputes the combination
 // (the partials are a few tens of KB) and writes 8-element chunks of `out` dealt round robin, as the other fused
 // glue kernels do.  Without R a few workgroups just write their chunks.
-__global__ __launch_bounds__(256) void attend_combine_proj_kernel(const float* __restrict__ part, half_t* __restrict__ out,
-                                                                  const half_t* __restrict__ R, half_t* __restrict__ r,
-                                                                  int heads, int d, int splits) {
+constexpr int kCombineSplits = 8;  // splits whose partials are all fetched before any is used
+__global__ __launch_bounds__(1024) void attend_combine_proj_kernel(const float* __restrict__ part, half_t* __restrict__ out,
+                                                                   const half_t* __restrict__ R, half_t* __restrict__ r,
+                                                                   int heads, int d, int splits) {
   __shared__ float red[16];
   const int j = blockIdx.x, nwg = gridDim.x;
   const int n = heads * d, chunks = n >> 3;
   const int nw = blockDim.x >> 6;
+  const int stride = d + 4;
   float dot = 0.f;
   for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
     const int head = (c << 3) / d, i0 = (c << 3) - head * d;
-    const float* ph = part + (size_t)head * splits * (d + 2);
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ph[s * (d + 2)]);
-    float den = 0.f, acc[8];
+    const float* ph = part + (size_t)head * splits * stride;
+    h8 rr;
+    if (R) rr = reinterpret_cast<const h8*>(R + (size_t)j * n)[c];
+    float mx = -INFINITY, den = 0.f, acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float w = __expf(ph[s * (d + 2)] - mx);
-      den = __builtin_fmaf(w, ph[s * (d + 2) + 1], den);
+    if (splits <= kCombineSplits) {
+      float pm[kCombineSplits], pl[kCombineSplits];
+      f4 lo[kCombineSplits], hi[kCombineSplits];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, ph[s * (d + 2) + 2 + i0 + e], acc[e]);
+      for (int s = 0; s < kCombineSplits; ++s) {
+        const float* ps = ph + min(s, splits - 1) * stride;
+        pm[s] = s < splits ? ps[0] : -INFINITY;
+        pl[s] = ps[1];
+        lo[s] = *reinterpret_cast<const f4*>(ps + 4 + i0);
+        hi[s] = *reinterpret_cast<const f4*>(ps + 8 + i0);
+      }
+#pragma unroll
+      for (int s = 0; s < kCombineSplits; ++s) mx = fmaxf(mx, pm[s]);
+#pragma unroll
+      for (int s = 0; s < kCombineSplits; ++s) {
+        const float w = (pm[s] == -INFINITY) ? 0.f : __expf(pm[s] - mx);
+        den = __builtin_fmaf(w, pl[s], den);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[e] = __builtin_fmaf(w, lo[s][e], acc[e]);
+          acc[4 + e] = __builtin_fmaf(w, hi[s][e], acc[4 + e]);
+        }
+      }
+    } else {
+      for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ph[s * stride]);
+      for (int s = 0; s < splits; ++s) {
+        const float pm = ph[s * stride];
+        const float w = (pm == -INFINITY) ? 0.f : __expf(pm - mx);
+        den = __builtin_fmaf(w, ph[s * stride + 1], den);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, ph[s * stride + 4 + i0 + e], acc[e]);
+      }
     }
     const float inv = 1.f / den;
     h8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (half_t)(acc[e] * inv);
     if (R) {
-      const h8 rr = reinterpret_cast<const h8*>(R + (size_t)j * n)[c];
 #pragma unroll
       for (int e = 0; e < 8; ++e) dot = __builtin_fmaf((float)o[e], (float)rr[e], dot);
     }
@@ -481,7 +548,10 @@ hipError_t launch_silu_mul_proj(const half_t* gate, const half_t* up, half_t* ou
   return hipGetLastError();
 }
 
-size_t rope_attend_lds(int d, int max_len) { return (size_t)(3 * d + 16 + 16 * d + max_len) * sizeof(float); }
+size_t rope_attend_lds(int d, int max_len) {
+  (void)max_len;  // no per-position buffer: the context length is bounded by the cache alone
+  return (size_t)(3 * d + 32 + 16 * d) * sizeof(float);
+}
 
 template <int kD>
 static hipError_t launch_rope_attend_t(const half_t* q, const half_t* k_new, const half_t* v_new, const float* cos_t,
@@ -513,7 +583,10 @@ hipError_t launch_rope_attend(const half_t* q, const half_t* k_new, const half_t
 hipError_t launch_attend_combine_proj(const float* part, half_t* out, const half_t* R, half_t* r, int heads, int d, int splits,
                                       int rank, hipStream_t stream) {
   const int wgs = R ? rank : 32;
-  hipLaunchKernelGGL(attend_combine_proj_kernel, dim3(wgs), dim3(256), 0, stream, part, out, R, r, heads, d, splits);
+  const int chunks = heads * d / 8;
+  int threads = (chunks + 63) / 64 * 64;  // one 8-element chunk per thread where the workgroup size allows
+  threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+  hipLaunchKernelGGL(attend_combine_proj_kernel, dim3(wgs), dim3(threads), 0, stream, part, out, R, r, heads, d, splits);
   return hipGetLastError();
 }
 
@@ -574,8 +647,6 @@ int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || max_len <= 0)
     return fail(GLOWQ_EINVAL, "rope_attend: heads must be a positive multiple of kv_heads (got %d, %d)", heads, kv_heads);
   if (head_dim != 64 && head_dim != 128) return fail(GLOWQ_EUNSUPPORTED, "rope_attend: head_dim must be 64 or 128 (got %d)", head_dim);
-  if (rope_attend_lds(head_dim, max_len) > 160 * 1024)
-    return fail(GLOWQ_EUNSUPPORTED, "rope_attend: max_len %d does not fit the score buffer in LDS", max_len);
   hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),
                                     cos_table, sin_table, reinterpret_cast<const long*>(pos), static_cast<half_t*>(cache_k),
                                     static_cast<half_t*>(cache_v), static_cast<half_t*>(out), nullptr, 1, heads, kv_heads, head_dim,
@@ -593,8 +664,6 @@ int glowq_rope_attend_split(const void* q, const void* k_new, const void* v_new,
                 kv_heads, splits);
   if (head_dim != 64 && head_dim != 128)
     return fail(GLOWQ_EUNSUPPORTED, "rope_attend_split: head_dim must be 64 or 128 (got %d)", head_dim);
-  if (rope_attend_lds(head_dim, max_len) > 160 * 1024)
-    return fail(GLOWQ_EUNSUPPORTED, "rope_attend_split: max_len %d does not fit the score buffer in LDS", max_len);
   hipError_t e = launch_rope_attend(static_cast<const half_t*>(q), static_cast<const half_t*>(k_new), static_cast<const half_t*>(v_new),
                                     cos_table, sin_table, reinterpret_cast<const long*>(pos), static_cast<half_t*>(cache_k),
                                     static_cast<half_t*>(cache_v), nullptr, partials, splits, heads, kv_heads, head_dim, max_len,

@@ -222,7 +222,7 @@ class FusedStep:
     Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
     the one-call projection + group entry point, o_proj and down_proj as solo groups."""
 
-    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 1):
+    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 4):
         cfg = model.cfg
         self.share = share  # False: every module projects x on R by itself and launches alone (the no-sharing comparator)
         self.model, self.cfg = model, cfg
@@ -242,10 +242,11 @@ class FusedStep:
         self.act = torch.zeros(1, cfg.intermediate, **f16)
         self.dn = torch.zeros(1, cfg.hidden, **f16)
         self.logits = torch.zeros(1, cfg.vocab, **f16)
-        # context split per head: measured slower than one workgroup per head up to ~800 cached tokens (2.45 vs 2.37 ms per
-        # token at 4 splits); meant for long contexts
+        # cached positions dealt to several workgroups per head; the merge kernel also produces o_proj's projection, so the
+        # launch count is the same as with one workgroup per head (2.36 ms per token at 4 or 8 splits, 2.40 ms at 1, with
+        # 512..768 cached tokens)
         self.splits = attention_splits
-        self.partials = torch.zeros(cfg.heads, attention_splits, cfg.head_dim + 2, dtype=torch.float32, device=dev)
+        self.partials = torch.zeros(cfg.heads, attention_splits, cfg.head_dim + 4, dtype=torch.float32, device=dev)
         self.scale = cfg.head_dim ** -0.5
         self.plan = []
         for layer in model.model.layers:
@@ -337,7 +338,8 @@ class FusedStep:
 class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
-    def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True):
+    def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True,
+                 attention_splits: int = 4):
         self.model = model
         cfg = model.cfg
         dev = model.lm_head.weight.device
@@ -351,7 +353,8 @@ class GreedyDecoder:
         self.next_tok = torch.zeros(1, dtype=torch.long, device=dev)
         self.use_graph = use_graph
         self.graph = None
-        self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok, share) if fused else None
+        self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok, share,
+                               attention_splits) if fused else None
 
     @torch.no_grad()
     def _step(self):
@@ -431,6 +434,7 @@ def main():
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
     ap.add_argument("--vocab", type=int, default=128256)
+    ap.add_argument("--attention-splits", type=int, default=4, help="workgroups per head in the fused step's attention")
     args = ap.parse_args()
     import os
 
@@ -440,7 +444,8 @@ def main():
     model, _, _ = build_decoder(cfg, with_correction=not args.no_correction)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path, share=not args.no_sharing)
+    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path, share=not args.no_sharing,
+                        attention_splits=args.attention_splits)
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=g)
     dec.generate(prompt, 4)  # warm-up (also captures the graph)

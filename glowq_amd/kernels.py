@@ -328,13 +328,13 @@ class W4A16Extension:
 
     def rope_attend_split(self, q, k_new, v_new, cos_table, sin_table, pos, cache_k, cache_v, partials, scale: float) -> None:
         """As rope_attend, with the context split over partials.size(1) workgroups per head; partials is a
-        [heads, splits, d + 2] fp32 buffer that receives {max, sum, unnormalised acc} of every split."""
+        [heads, splits, d + 4] fp32 buffer that receives {max, sum, 2 unused, unnormalised acc} of every split."""
         for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new"), (cache_k, "cache_k"), (cache_v, "cache_v")):
             self._f16(t, n)
         kv_heads, max_len, d = cache_k.shape
         heads = q.numel() // d
         _check(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and partials.dim() == 3
-               and partials.size(0) == heads and partials.size(2) == d + 2, "rope_attend_split: partials must be fp32 [heads, splits, d + 2]")
+               and partials.size(0) == heads and partials.size(2) == d + 4, "rope_attend_split: partials must be fp32 [heads, splits, d + 4]")
         _check(cos_table.dtype == torch.float32 and cos_table.is_contiguous() and sin_table.dtype == torch.float32
                and sin_table.is_contiguous() and tuple(cos_table.shape) == (max_len, d) and sin_table.shape == cos_table.shape,
                "rope_attend_split: tables must be contiguous CUDA fp32 [max_len, d]")
@@ -353,9 +353,9 @@ class W4A16Extension:
         """out [heads * d] fp16 from the split partials; with R [rank, heads * d] also r = out R^T ([rank] fp16)."""
         self._f16(out, "out")
         heads, splits, d2 = partials.shape
-        d = d2 - 2
+        d = d2 - 4
         _check(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and out.numel() == heads * d,
-               "attend_combine_proj: partials fp32 [heads, splits, d + 2], out [heads * d]")
+               "attend_combine_proj: partials fp32 [heads, splits, d + 4], out [heads * d]")
         _check((R is None) == (r is None), "attend_combine_proj: R and r go together")
         if R is not None:
             self._f16(R, "R"), self._f16(r, "r")

@@ -161,15 +161,15 @@ int glowq_silu_mul_proj(const void* gate, const void* up, void* out, const void*
 /*
  * Rotary embedding of q [heads, d] and k_new [kv_heads, d] at position *pos (cos/sin tables [max_len, d] fp32),
  * append of k / v_new to the caches [kv_heads, max_len, d] at *pos, attention of the one query token over positions
- * 0..*pos, out [heads, d].  d = 64 or 128, max_len limited by the LDS score buffer (about 38k positions).
+ * 0..*pos, out [heads, d].  d = 64 or 128; one pass with a running maximum, so max_len is bounded by the caches alone.
  */
 int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
                       const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,
                       int max_len, float scale, void* stream);
 
 /*
- * The same with the context split over `splits` workgroups per head: each writes its unnormalised partial
- * {max, sum, acc[d]} to partials [heads, splits, d + 2] fp32 (caller's buffer).  glowq_attend_combine_proj merges them
+ * The same with the cached positions dealt row by row to `splits` workgroups per head: each writes its unnormalised
+ * partial {max, sum, 2 unused, acc[d]} to partials [heads, splits, d + 4] fp32 (caller's buffer).  glowq_attend_combine_proj merges them
  * into out [heads * d] fp16 and, when R [rank, heads * d] is given, also writes r = out R^T ([rank] fp16) for the group
  * that consumes the attention output -- the o_proj group then needs no projection launch.
  */

@@ -169,9 +169,10 @@ def test_glue_kernels_match_torch(ext, fp16_out):
     assert (int(nxt), int(tok), int(pos)) == (1234, 1234, 42)
 
 
-@pytest.mark.parametrize("pos", [0, 1, 37, 300])
-def test_rope_attend_matches_torch(ext, fp16_out, pos):
-    heads, kvh, d, max_len = 8, 2, 64, 320
+@pytest.mark.parametrize("d,max_len,pos", [(64, 320, 0), (64, 320, 1), (64, 320, 37), (64, 320, 300), (128, 2100, 257),
+                                           (128, 2100, 700), (128, 2100, 2047), (64, 1500, 1300)])
+def test_rope_attend_matches_torch(ext, fp16_out, d, max_len, pos):
+    heads, kvh = 8, 2
     g = torch.Generator(device="cuda").manual_seed(pos)
     q = torch.randn(heads, d, device="cuda", generator=g).half()
     k = torch.randn(kvh, d, device="cuda", generator=g).half()
@@ -219,7 +220,7 @@ def test_split_attention_and_merge_match_single_workgroup(ext, fp16_out, pos, sp
     ck1, cv1, want = ck.clone(), cv.clone(), torch.empty(heads * d, dtype=torch.float16, device="cuda")
     ext.rope_attend(q, k, v, cos, sin, p, ck1, cv1, want, d ** -0.5)
     ck2, cv2 = ck.clone(), cv.clone()
-    part = torch.full((heads, splits, d + 2), float("nan"), device="cuda")
+    part = torch.full((heads, splits, d + 4), float("nan"), device="cuda")
     got, r = torch.empty_like(want), torch.empty(rank, dtype=torch.float16, device="cuda")
     ext.rope_attend_split(q, k, v, cos, sin, p, ck2, cv2, part, d ** -0.5)
     ext.attend_combine_proj(part, got, R, r)
