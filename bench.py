@@ -39,6 +39,15 @@ GROUPS = {
     "gate_up": (4096, [14336, 14336]),
     "down_proj": (14336, [4096]),
 }
+# the prefill configuration of the same benchmark: Qwen2.5-7B-shaped layer at 2048 tokens (MFMA-bound)
+PREFILL_TOKENS = 2048
+PREFILL_GROUPS = {
+    "qkv": (3584, [3584, 512, 512]),
+    "o_proj": (3584, [3584]),
+    "gate_up": (3584, [18944, 18944]),
+    "down_proj": (18944, [3584]),
+}
+MFMA_FP16_PEAK_TFLOPS = 2516.6
 DOMINANT = "gate_up"
 DOMINANT_TRAFFIC_BYTES = 68708000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
 
@@ -51,12 +60,12 @@ def algorithmic_bytes(M, K, N, rank, gs=GROUP_SIZE):
     return b
 
 
-def make_layer(torch, dev, seed):
+def make_layer(torch, dev, seed, groups=None):
     """Random codes / zero-point nibbles (any bit pattern is a valid quantised weight), scales in the
     range a N(0, 0.02) weight produces, R ~ N(0, 1/K), L ~ N(0, 0.01^2)."""
     g = torch.Generator(device=dev).manual_seed(seed)
     layer = {}
-    for name, (K, Ns) in GROUPS.items():
+    for name, (K, Ns) in (groups or GROUPS).items():
         G = K // GROUP_SIZE
         members = []
         for N in Ns:
@@ -113,12 +122,52 @@ def cpu_baseline(torch, budget_s=18.0):
     }
 
 
+def prefill_leg(torch, ext, dev):
+    """Every group of a Qwen2.5-7B-shaped layer at 2048 tokens: projection launch + group launch as in decode,
+    algorithmic flops 2 M N K + 2 M r K + 2 M N r against the dense fp16 MFMA peak."""
+    g = torch.Generator(device=dev).manual_seed(11)
+    prefill = {"workload": f"Qwen2.5-7B-shaped layer, M={PREFILL_TOKENS}, int4 g=128 asym, shared rank-{RANK} correction",
+               "per_group": {}}
+    pl = make_layer(torch, dev, 7, PREFILL_GROUPS)
+    tot_us, tot_fl = 0.0, 0.0
+    for name, (K, Ns) in PREFILL_GROUPS.items():
+        members, R = pl[name]
+        xp = torch.randn(PREFILL_TOKENS, K, device=dev, generator=g).half()
+        rp = torch.empty(PREFILL_TOKENS, RANK, dtype=torch.float16, device=dev)
+        op = [torch.empty(PREFILL_TOKENS, N, dtype=torch.float16, device=dev) for N in Ns]
+        for _ in range(2):
+            ext.group_forward(xp, rp, members, GROUP_SIZE, 1.0, outs=op, R=R)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(5):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(4):
+                ext.group_forward(xp, rp, members, GROUP_SIZE, 1.0, outs=op, R=R)
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b) * 1e3 / 4)
+        us = sorted(ts)[len(ts) // 2]
+        N = sum(Ns)
+        fl = 2.0 * PREFILL_TOKENS * (N * K + RANK * K + N * RANK)
+        prefill["per_group"][name] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
+                                      "frac_mfma_peak": round(fl / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+        tot_us += us
+        tot_fl += fl
+        del xp, rp, op
+    prefill["us_per_layer"] = round(tot_us, 1)
+    prefill["TFLOPs"] = round(tot_fl / tot_us / 1e6, 1)
+    prefill["frac_mfma_peak"] = round(tot_fl / tot_us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)
+    return prefill
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--prefill-only", action="store_true", help="run only the prefill leg and print it (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of known size (256 MiB read + 256 MiB written each) so that "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiling run can be scaled")
@@ -136,6 +185,10 @@ def main():
     ext = load_w4a16_extension()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_leg(torch, ext, dev)}))
+        return
 
     layers = [make_layer(torch, dev, 100 + i) for i in range(LAYERS)]
     g = torch.Generator(device=dev).manual_seed(1)
@@ -253,6 +306,8 @@ def main():
         torch.cuda.synchronize()
         batched[str(rows)] = round(a.elapsed_time(b) * 1e3 / 5 / 8, 2)
 
+    prefill = prefill_leg(torch, ext, dev)
+
     if args.calibrate_copy:
         # cold sources: 8 distinct 256 MiB buffers, each copied once (the kernel shows up in a profile as
         # torch's elementwise copy kernel with 134217728 elements)
@@ -290,6 +345,7 @@ def main():
         "algorithmic_bytes_per_layer": bytes_layer,
         "per_group": per_group,
         "batched_rows_us_per_layer": batched,
+        "prefill": prefill,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",

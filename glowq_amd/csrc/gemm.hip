@@ -56,11 +56,16 @@ __device__ __forceinline__ h8 permute_for_nibble_order(const h8& v) {
 // 8 codes of one word -> fp16((code - zero) * scale), in nibble order (0,4,1,5,2,6,3,7).
 // zb_lo = -(1024 + zero), zb_hi = -(64 + zero), both exact in fp16.
 __device__ __forceinline__ h8 dequant_word(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2) {
+  // the two exponent patterns (1024.0 and 64.0 in both halves) live in vector registers: with the nibble mask as the one
+  // scalar operand the mask-and-merge is then a single v_and_or_b32 instead of an AND and an OR
+  uint32_t e1024, e64;
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(e1024));
+  asm("v_mov_b32 %0, 0x54005400" : "=v"(e64));
   const uint32_t hi = w >> 8;
-  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | 0x64006400u);
-  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | 0x54005400u);
-  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | 0x64006400u);
-  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | 0x54005400u);
+  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | e1024);
+  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | e64);
+  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | e1024);
+  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | e64);
   const h2 d0 = (q0 + zb_lo) * s2;
   const h2 d1 = (q1 + zb_hi) * s2;
   const h2 d2 = (q2 + zb_lo) * s2;
@@ -470,6 +475,10 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stre
     }
   }
   if (mt_cap == 8 && mt == 4 && mt_max >= 8) mt = 8;
+  static const int force_mt = getenv("GLOWQ_GEMM_FORCE_MT") ? atoi(getenv("GLOWQ_GEMM_FORCE_MT")) : 0;
+  static const int force_nt = getenv("GLOWQ_GEMM_FORCE_NT") ? atoi(getenv("GLOWQ_GEMM_FORCE_NT")) : 0;
+  if (force_mt > 0 && force_mt <= mt_cap) mt = force_mt;
+  if (force_nt > 0 && force_nt <= nt_cap) nt = force_nt;
   static const int env_super = getenv("GLOWQ_GEMM_SUPER") ? atoi(getenv("GLOWQ_GEMM_SUPER")) : 1;
   const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128;
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
