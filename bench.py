@@ -48,6 +48,15 @@ PREFILL_GROUPS = {
     "down_proj": (18944, [3584]),
 }
 MFMA_FP16_PEAK_TFLOPS = 2516.6
+# the selective configuration (GlowQ-S): Qwen3-14B-shaped layer, rank 256, correction on a seeded half of the groups
+SELECTIVE_RANK = 256
+SELECTIVE_LAYERS = 4
+SELECTIVE_GROUPS = {
+    "qkv": (5120, [5120, 1024, 1024]),
+    "o_proj": (5120, [5120]),
+    "gate_up": (5120, [17408, 17408]),
+    "down_proj": (17408, [5120]),
+}
 DOMINANT = "gate_up"
 DOMINANT_TRAFFIC_BYTES = 68708000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
 
@@ -60,7 +69,7 @@ def algorithmic_bytes(M, K, N, rank, gs=GROUP_SIZE):
     return b
 
 
-def make_layer(torch, dev, seed, groups=None):
+def make_layer(torch, dev, seed, groups=None, rank=RANK):
     """Random codes / zero-point nibbles (any bit pattern is a valid quantised weight), scales in the
     range a N(0, 0.02) weight produces, R ~ N(0, 1/K), L ~ N(0, 0.01^2)."""
     g = torch.Generator(device=dev).manual_seed(seed)
@@ -73,10 +82,10 @@ def make_layer(torch, dev, seed, groups=None):
                 "qweight": torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=g),
                 "scales": (torch.rand(N, G, device=dev, generator=g) * 0.004 + 0.006).half(),
                 "qzeros": torch.randint(-2**31, 2**31 - 1, (N, (G + 7) // 8), dtype=torch.int32, device=dev, generator=g),
-                "L": (torch.randn(N, RANK, device=dev, generator=g) * 0.01).half(),
+                "L": (torch.randn(N, rank, device=dev, generator=g) * 0.01).half(),
                 "bias": None,
             })
-        R = (torch.randn(RANK, K, device=dev, generator=g) * K ** -0.5).half()
+        R = (torch.randn(rank, K, device=dev, generator=g) * K ** -0.5).half()
         layer[name] = (members, R)
     return layer
 
@@ -161,6 +170,71 @@ def prefill_leg(torch, ext, dev):
     return prefill
 
 
+def selective_leg(torch, ext, dev):
+    """GlowQ-S on a Qwen3-14B-shaped layer (rank 256) across the switch from the GEMV kernels to the MFMA kernels:
+    per token-row count the time of every group with its correction (projection + group launch) and without (the bare
+    quantised group: what an unselected group costs), the kernel route taken, and the layer with a seeded random half
+    of its groups selected.  4 layers of distinct weights (660 MB) per replay."""
+    g = torch.Generator(device=dev).manual_seed(21)
+    layers = [make_layer(torch, dev, 300 + i, SELECTIVE_GROUPS, SELECTIVE_RANK) for i in range(SELECTIVE_LAYERS)]
+    names = list(SELECTIVE_GROUPS)
+    pick = torch.randperm(SELECTIVE_LAYERS * len(names), generator=torch.Generator().manual_seed(1234))
+    selected = set(int(i) for i in pick[: SELECTIVE_LAYERS * len(names) // 2])  # groups enumerated layer-major
+    side = torch.cuda.Stream()
+    out = {"workload": f"Qwen3-14B-shaped layer, int4 g=128 asym, rank {SELECTIVE_RANK}, {SELECTIVE_LAYERS} layers of "
+                       f"distinct weights, correction on a seeded half of the groups", "rows": {}}
+
+    def timed(run):
+        with torch.cuda.stream(side):
+            run()  # outside the capture first: kernel attributes
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=side):
+                run()
+        torch.cuda.synchronize()
+        gr.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            gr.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / 5
+
+    for rows in (1, 4, 16, 64):
+        xs = {n: torch.randn(rows, K, device=dev, generator=g).half() for n, (K, _) in SELECTIVE_GROUPS.items()}
+        rb = torch.empty(rows, SELECTIVE_RANK, dtype=torch.float16, device=dev)
+        ob = {n: [torch.empty(rows, N, dtype=torch.float16, device=dev) for N in Ns] for n, (_, Ns) in SELECTIVE_GROUPS.items()}
+        bare = [{n: [dict(m, L=None) for m in layer[n][0]] for n in names} for layer in layers]
+
+        def corrected(n, layer):
+            ext.group_forward(xs[n], rb, layer[n][0], GROUP_SIZE, 1.0, outs=ob[n], R=layer[n][1])
+
+        def plain(n, li):
+            ext.group_forward(xs[n], None, bare[li][n], GROUP_SIZE, 0.0, outs=ob[n])
+
+        entry = {"route": {n: ext.route(rows, K, sum(Ns), GROUP_SIZE) for n, (K, Ns) in SELECTIVE_GROUPS.items()},
+                 "corrected_us": {}, "plain_us": {}}
+        for n in names:
+            entry["corrected_us"][n] = round(timed(lambda: [corrected(n, layer) for layer in layers]) / SELECTIVE_LAYERS, 2)
+            entry["plain_us"][n] = round(timed(lambda: [plain(n, li) for li in range(SELECTIVE_LAYERS)]) / SELECTIVE_LAYERS, 2)
+
+        def half():
+            for li, layer in enumerate(layers):
+                for gi, n in enumerate(names):
+                    if li * len(names) + gi in selected:
+                        corrected(n, layer)
+                    else:
+                        plain(n, li)
+
+        entry["all_corrected_us_per_layer"] = round(sum(entry["corrected_us"].values()), 2)
+        entry["none_corrected_us_per_layer"] = round(sum(entry["plain_us"].values()), 2)
+        entry["half_selected_us_per_layer"] = round(timed(half) / SELECTIVE_LAYERS, 2)
+        out["rows"][str(rows)] = entry
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -168,6 +242,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill leg and print it (profiling runs)")
+    ap.add_argument("--selective-only", action="store_true", help="run only the GlowQ-S leg and print it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of known size (256 MiB read + 256 MiB written each) so that "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiling run can be scaled")
@@ -188,6 +263,10 @@ def main():
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_leg(torch, ext, dev)}))
+        return
+
+    if args.selective_only:
+        print(json.dumps({"selective": selective_leg(torch, ext, dev)}))
         return
 
     layers = [make_layer(torch, dev, 100 + i) for i in range(LAYERS)]
@@ -282,7 +361,7 @@ def main():
     # the same layers at more token rows per call (batched decode): reported next to the metric, not part of it;
     # 8 layers of distinct weights (1 GB) per replay keep the last-level cache out of the picture
     batched = {}
-    for rows in (4, 16, 64):
+    for rows in (2, 4, 8, 16, 64):
         xb = {name: torch.randn(rows, K, device=dev, generator=g).half() for name, (K, _) in GROUPS.items()}
         rb = torch.empty(rows, RANK, dtype=torch.float16, device=dev)
         ob = {name: [torch.empty(rows, N, dtype=torch.float16, device=dev) for N in Ns] for name, (_, Ns) in GROUPS.items()}
@@ -320,6 +399,10 @@ def main():
         torch.cuda.synchronize()
         del srcs, dst
 
+    del layers, graph, gdom
+    torch.cuda.empty_cache()
+    selective = selective_leg(torch, ext, dev)
+
     result = {
         "metric": "W4A16+GlowQ decode linears, microseconds per layer (Llama-3.1-8B shape, batch 1)",
         "value": round(us_per_layer, 3),
@@ -346,6 +429,7 @@ def main():
         "per_group": per_group,
         "batched_rows_us_per_layer": batched,
         "prefill": prefill,
+        "selective": selective,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",

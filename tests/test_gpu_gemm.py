@@ -44,7 +44,8 @@ def test_gemm_route_falls_back_on_odd_shapes(ext):
 
 
 @pytest.mark.parametrize("M,K,rank", [(1, 2048, 64), (3, 4096, 128), (8, 1024, 256), (300, 1024, 128), (2048, 512, 64),
-                                      (70, 3584, 256), (5, 200, 24)])
+                                      (70, 3584, 256), (5, 200, 24), (64, 17408, 256), (17, 4096, 128), (100, 14336, 40),
+                                      (33, 5184, 96), (512, 4160, 128)])
 def test_shared_proj(ext, M, K, rank):
     g = torch.Generator().manual_seed(M + K + rank)
     x = torch.randn(M, K, generator=g).half().numpy()
