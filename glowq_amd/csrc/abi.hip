@@ -28,7 +28,9 @@ bool skinny_group_form(const GroupDev& g);
 hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream);
 bool gemm_supported(const GroupDev& g);
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream);
-hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t);
+hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t, void* ws,
+                                   size_t ws_bytes);
+size_t proj_workspace_bytes(int M, int K, int rank, int num_cus);
 }  // namespace glowq
 
 using namespace glowq;
@@ -169,7 +171,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     // r = x R^T goes ahead as a launch of its own.  (Folding it into the group kernel was measured: the
     // R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch costs.)
     if (g.M > 16 && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
-      e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream);
+      e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream, g.ws, g.ws_bytes);
     else
       e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
     if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
@@ -277,7 +279,8 @@ int glowq_unpack_int4(const int32_t* packed, uint8_t* codes, int rows, int total
   return GLOWQ_OK;
 }
 
-int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int rank, void* stream) {
+static int shared_proj_impl(const void* x, const void* R, void* r, int M, int K, int rank, void* ws, size_t ws_bytes,
+                            void* stream) {
   if (!x || !R || !r) return fail(GLOWQ_EINVAL, "shared_proj: NULL pointer");
   if (M <= 0 || K <= 0 || rank <= 0) return fail(GLOWQ_EINVAL, "shared_proj: M, K and rank must be > 0");
   const half_t* xp = static_cast<const half_t*>(x);
@@ -285,7 +288,7 @@ int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int r
   half_t* rp = static_cast<half_t*>(r);
   hipError_t e;
   if (M > 16 && (K & 63) == 0 && aligned16(x) && aligned16(R)) {
-    e = launch_shared_proj_mfma(xp, Rp, rp, M, K, rank, num_cus(), static_cast<hipStream_t>(stream));
+    e = launch_shared_proj_mfma(xp, Rp, rp, M, K, rank, num_cus(), static_cast<hipStream_t>(stream), ws, ws_bytes);
   } else {
     if ((K & 7) == 0 && (!aligned16(x) || !aligned16(R)))
       return fail(GLOWQ_EUNSUPPORTED, "shared_proj: x and R must be 16-byte aligned");
@@ -294,6 +297,17 @@ int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int r
   if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
   return GLOWQ_OK;
 }
+
+int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int rank, void* stream) {
+  return shared_proj_impl(x, R, r, M, K, rank, nullptr, 0, stream);
+}
+
+int glowq_shared_proj_ws(const void* x, const void* R, void* r, int M, int K, int rank, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+  return shared_proj_impl(x, R, r, M, K, rank, workspace, workspace_bytes, stream);
+}
+
+size_t glowq_proj_workspace_bytes(int M, int K, int rank) { return proj_workspace_bytes(M, K, rank, num_cus()); }
 
 int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
                               int K, int group_size, int rank, float alpha, void* stream) {
@@ -327,8 +341,9 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
   return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
 }
 
-int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
-                                    int n_members, int M, int K, int group_size, int rank, float alpha, void* stream) {
+static int group_forward_fused_impl(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                    int n_members, int M, int K, int group_size, int rank, float alpha, void* ws,
+                                    size_t ws_bytes, void* stream) {
   int rc = check_common(x, M, K, group_size);
   if (rc) return rc;
   if (members == nullptr || n_members < 1 || n_members > GLOWQ_MAX_MEMBERS)
@@ -347,6 +362,8 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
   g.x = static_cast<const half_t*>(x);
   g.R = static_cast<const half_t*>(R);
   g.r_out = static_cast<half_t*>(r_out);
+  g.ws = ws;
+  g.ws_bytes = ws_bytes;
   g.rank = rank;
   g.alpha = alpha;
   g.n_members = n_members;
@@ -356,6 +373,18 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
   if (alpha == 0.0f)
     for (int i = 0; i < n_members; ++i) g.mem[i].L = nullptr;  // r is still produced: callers cache it
   return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
+}
+
+int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                    int n_members, int M, int K, int group_size, int rank, float alpha, void* stream) {
+  return group_forward_fused_impl(x, R, r_out, members, n_members, M, K, group_size, rank, alpha, nullptr, 0, stream);
+}
+
+int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                       int n_members, int M, int K, int group_size, int rank, float alpha,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  return group_forward_fused_impl(x, R, r_out, members, n_members, M, K, group_size, rank, alpha, workspace,
+                                  workspace_bytes, stream);
 }
 
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {

@@ -36,6 +36,8 @@ struct GroupDev {
   // set by the entry point that also produces r: the projection r_out = x R^T is launched ahead of the group
   const half_t* R;  // [rank, K] or nullptr
   half_t* r_out;
+  void* ws;         // caller's workspace for the many-row projection (or nullptr) and its size
+  size_t ws_bytes;
   MemberDev mem[GLOWQ_MAX_MEMBERS];
   int task_end[GLOWQ_MAX_MEMBERS];  // exclusive prefix of per-member task counts
   int wg_end[GLOWQ_MAX_MEMBERS];    // exclusive prefix of the workgroups assigned to each member

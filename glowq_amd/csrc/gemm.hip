@@ -543,9 +543,18 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
 constexpr int kPK = 256;           // k depth of one block (4 waves x 64)
 constexpr int kPRow = kPK + 8;     // padded LDS row in halves
 
+//
+// Split K (gridDim.z > 1): workgroup z of a tile takes a contiguous range of blocks and leaves its fp32 partial tile
+// in the caller's workspace, [tile][slice][kNT * 1024] floats in accumulator-register order; proj_reduce_kernel then
+// adds the partials in slice order and writes r.  (Finishing a tile in the workgroup that arrives last at a counter
+// was measured first: the device-scope traffic it needs inside one launch costs 20 us and more, a second launch 4.)
+struct ProjSplit {
+  float* partials;
+};
+
 template <int kNT>
 __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict__ x, const half_t* __restrict__ R,
-                                                        half_t* __restrict__ r, int M, int K, int rank) {
+                                                        half_t* __restrict__ r, int M, int K, int rank, ProjSplit sp) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* lds_x = reinterpret_cast<half_t*>(smem);  // [2][32][kPRow]; reused for the final reduction
   const int tid = threadIdx.x;
@@ -554,7 +563,11 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
   const int ln = lane & 31, lh = lane >> 5;
   const int m0 = blockIdx.x * 32;
   const int n0 = blockIdx.y * (32 * kNT);
-  const int blocks = (K + kPK - 1) / kPK;  // K is a multiple of 64; the last block may be partial
+  const int all_blocks = (K + kPK - 1) / kPK;  // K is a multiple of 64; the last block may be partial
+  const int slices = gridDim.z;
+  const int per_slice = (all_blocks + slices - 1) / slices;
+  const int blk_begin = min((int)blockIdx.z * per_slice, all_blocks);
+  const int blocks = min(blk_begin + per_slice, all_blocks);  // this workgroup walks blocks [blk_begin, blocks)
 
   int ncol[kNT];
 #pragma unroll
@@ -615,7 +628,7 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
   // stage.  Two blocks of loads are in flight at any time.
   auto block = [&](int blk, BRegs& br, XRegs& x_fill, const XRegs& x_store) {
     BRegs cur = br;
-    const int kn = min(blk + 2, blocks - 1) * kPK;
+    const int kn = min(blk + 2, all_blocks - 1) * kPK;
     load_b(kn, br);
     load_x(kn, x_fill);
     mma_block(stage, blk * kPK, cur);
@@ -625,13 +638,13 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
   };
   XRegs x0, x1;
   BRegs b0, b1;
-  load_x(0, x0);
-  load_b(0, b0);
-  load_x(min(1, blocks - 1) * kPK, x1);
-  load_b(min(1, blocks - 1) * kPK, b1);
+  load_x(min(blk_begin, all_blocks - 1) * kPK, x0);
+  load_b(min(blk_begin, all_blocks - 1) * kPK, b0);
+  load_x(min(blk_begin + 1, all_blocks - 1) * kPK, x1);
+  load_b(min(blk_begin + 1, all_blocks - 1) * kPK, b1);
   store_x(0, x0);
   __syncthreads();
-  for (int blk = 0; blk < blocks; blk += 2) {
+  for (int blk = blk_begin; blk < blocks; blk += 2) {
     block(blk, b0, x0, x1);
     if (blk + 1 >= blocks) break;
     block(blk + 1, b1, x1, x0);
@@ -655,35 +668,114 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
       float v = 0.f;
 #pragma unroll
       for (int w = 0; w < 4; ++w) v += red[((w * kNT + tn) * 16 + i) * 64 + lane];
-      const int m = m0 + 8 * (i >> 2) + 4 * lh + (i & 3);
-      if (m < M && n < rank) r[(size_t)m * rank + n] = (half_t)v;
+      if (slices == 1) {
+        const int m = m0 + 8 * (i >> 2) + 4 * lh + (i & 3);
+        if (m < M && n < rank) r[(size_t)m * rank + n] = (half_t)v;
+      } else {
+        const size_t tile = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+        sp.partials[(tile * slices + blockIdx.z) * (kNT * 1024) + (tn * 16 + i) * 64 + lane] = v;
+      }
     }
   }
 }
 
-hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int num_cus,
-                                   hipStream_t stream) {
-  if ((K % kBK) != 0 || K < kBK) return hipErrorInvalidValue;
+// r[m, n] = fp16(sum over the slices, in slice order, of the partial tiles of proj_mfma_kernel<kNT>).  One thread per
+// accumulator element of a tile; m_blocks = gridDim.x of the producing launch.
+__global__ __launch_bounds__(256) void proj_reduce_kernel(const float* __restrict__ partials, half_t* __restrict__ r, int M,
+                                                          int rank, int nt, int slices, int m_blocks) {
+  const int per_tile = nt * 1024;
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;  // element of the tile: (tn * 16 + i) * 64 + lane
+  const int tile = blockIdx.y;
+  if (e >= per_tile) return;
+  const int lane = e & 63, i = (e >> 6) & 15, tn = e >> 10;
+  const int m = (tile % m_blocks) * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+  const int n = (tile / m_blocks) * (32 * nt) + tn * 32 + (lane & 31);
+  const float* src = partials + (size_t)tile * slices * per_tile + e;
+  float v = 0.f;
+  int z = 0;
+  for (; z + 8 <= slices; z += 8) {
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = src[(size_t)(z + u) * per_tile];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v += t[u];
+  }
+  for (; z < slices; ++z) v += src[(size_t)z * per_tile];
+  if (m < M && n < rank) r[(size_t)m * rank + n] = (half_t)v;
+}
+
+// How a projection is cut: columns per workgroup (32 * nt) and K slices.  The tile width follows the workgroup count
+// (narrow tiles where 64 columns each would leave CUs idle; R is small, re-reading it is cheap).  K is split only with a
+// workspace, where the tiles alone fill less than half the chip and K is long enough for the second launch to pay
+// (from 4096 columns): then as many slices as bring the workgroup count to about two per CU, each at least two
+// blocks deep, as far as the workspace reaches.
+struct ProjPlan {
+  int nt, slices;
+};
+static ProjPlan plan_proj(int M, int K, int rank, int num_cus, size_t ws_bytes) {
+  const int m_blocks = (M + 31) / 32;
+  const int blocks = (K + kPK - 1) / kPK;
+  ProjPlan best;
+  best.slices = 1;
+  best.nt = (m_blocks * ((rank + 63) / 64) < num_cus && rank > 32) ? 1 : 2;
+  if (blocks < 16) return best;
+  long best_wgs = (long)m_blocks * ((rank + 32 * best.nt - 1) / (32 * best.nt));
+  // with a workspace: the tile width whose split brings the most workgroups (up to two per CU); the wider tile on a
+  // tie, since x is then read fewer times
+  for (int nt : {2, 1}) {
+    if (nt == 2 && rank <= 32) continue;
+    const long tiles = (long)m_blocks * ((rank + 32 * nt - 1) / (32 * nt));
+    if (tiles * 2 > num_cus || tiles > 65535) continue;
+    long want = (2L * num_cus + tiles - 1) / tiles;
+    const int min_depth = tiles >= 16 ? 4 : 2;  // blocks per slice: the partials of many tiles are traffic of their own
+    if (want > blocks / min_depth) want = blocks / min_depth;
+    const long fit = (long)(ws_bytes / sizeof(float) / ((size_t)tiles * nt * 1024));
+    if (want > fit) want = fit;
+    if (want < 2) continue;
+    long wgs = tiles * want;
+    if (wgs > 2L * num_cus) wgs = 2L * num_cus;
+    if (wgs > best_wgs) {
+      best_wgs = wgs;
+      best.nt = nt;
+      best.slices = (int)want;
+    }
+  }
+  return best;
+}
+
+size_t proj_workspace_bytes(int M, int K, int rank, int num_cus) {
+  if (M <= 16 || (K % kBK) != 0) return 0;
+  const ProjPlan p = plan_proj(M, K, rank, num_cus, ~(size_t)0 >> 8);
+  if (p.slices < 2) return 0;
+  const long tiles = (long)((M + 31) / 32) * ((rank + 32 * p.nt - 1) / (32 * p.nt));
+  return (size_t)tiles * p.slices * p.nt * 1024 * sizeof(float);
+}
+
+template <int NT>
+static hipError_t launch_proj_t(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int slices, void* ws,
+                                hipStream_t stream) {
   const int m_blocks = (M + 31) / 32;
   const size_t lds_x = (size_t)2 * 32 * kPRow * sizeof(half_t);
-  static const bool wide = getenv("GLOWQ_PROJ_WIDE") != nullptr;
-  if (rank > 64 && wide) {
-    constexpr int NT = 4;
-    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
-    static LdsLimit lds_limit;
-    if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), lds, lds_limit); e != hipSuccess) return e;
-    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 127) / 128), dim3(256), lds, stream, x, R, r, M, K, rank);
-  } else if (m_blocks * ((rank + 63) / 64) < num_cus && rank > 32) {
-    // too few workgroups with 64 columns each: 32 columns per workgroup double them (R is small, re-reading it is free)
-    constexpr int NT = 1;
-    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
-    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 31) / 32), dim3(256), lds, stream, x, R, r, M, K, rank);
-  } else {
-    constexpr int NT = 2;
-    const size_t lds = lds_x > (size_t)4 * NT * 16 * 64 * 4 ? lds_x : (size_t)4 * NT * 16 * 64 * 4;
-    hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, (rank + 63) / 64), dim3(256), lds, stream, x, R, r, M, K, rank);
-  }
+  const size_t lds_red = (size_t)4 * NT * 16 * 64 * 4;
+  const size_t lds = lds_x > lds_red ? lds_x : lds_red;
+  static LdsLimit lds_limit;
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), lds, lds_limit); e != hipSuccess) return e;
+  ProjSplit sp = {slices > 1 ? static_cast<float*>(ws) : nullptr};
+  const int col_blocks = (rank + 32 * NT - 1) / (32 * NT);
+  hipLaunchKernelGGL(proj_mfma_kernel<NT>, dim3(m_blocks, col_blocks, slices), dim3(256), lds, stream, x, R, r, M, K, rank, sp);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess || slices == 1) return e;
+  hipLaunchKernelGGL(proj_reduce_kernel, dim3(NT * 4, m_blocks * col_blocks), dim3(256), 0, stream, sp.partials, r, M, rank, NT,
+                     slices, m_blocks);
   return hipGetLastError();
+}
+
+hipError_t launch_shared_proj_mfma(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank, int num_cus,
+                                   hipStream_t stream, void* ws, size_t ws_bytes) {
+  if ((K % kBK) != 0 || K < kBK) return hipErrorInvalidValue;
+  if (ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 15u) != 0) ws_bytes = 0;
+  const ProjPlan p = plan_proj(M, K, rank, num_cus, ws_bytes);
+  if (p.nt == 2) return launch_proj_t<2>(x, R, r, M, K, rank, p.slices, ws, stream);
+  return launch_proj_t<1>(x, R, r, M, K, rank, p.slices, ws, stream);
 }
 
 }  // namespace glowq

@@ -47,6 +47,10 @@ _SIGNATURES = {
     "glowq_w4a16_dequant": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "glowq_unpack_int4": (_I, [_P, _P, _I, _I, _I, _P]),
     "glowq_shared_proj": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "glowq_shared_proj_ws": (_I, [_P, _P, _P, _I, _I, _I, _P, ctypes.c_size_t, _P]),
+    "glowq_proj_workspace_bytes": (ctypes.c_size_t, [_I, _I, _I]),
+    "glowq_w4a16_group_forward_fused_ws": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float,
+                                                _P, ctypes.c_size_t, _P]),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
@@ -77,6 +81,7 @@ class W4A16Extension:
             fn.restype = res
             fn.argtypes = args
         self.version = lib.glowq_version()
+        self._workspaces = {}
 
     # ------------------------------------------------------------------ helpers
     def _raise(self, rc: int, what: str):
@@ -86,6 +91,24 @@ class W4A16Extension:
     @staticmethod
     def _stream(dev: torch.device) -> int:
         return torch.cuda.current_stream(dev).cuda_stream
+
+    WORKSPACE_BYTES = 16 << 20
+
+    def _workspace(self, dev: torch.device, rows: int):
+        """(pointer, bytes) of the projection workspace of the current stream of `dev`: one per stream, because calls
+        that share one must not overlap.  Only calls with more than 16 token rows use it.  A stream that meets its
+        first such call while it is being captured into a graph goes without (the buffer would come from the graph's
+        own memory pool)."""
+        if rows <= 16:
+            return None, 0
+        key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev))
+        ws = self._workspaces.get(key)
+        if ws is None:
+            if torch.cuda.is_current_stream_capturing():
+                return None, 0
+            ws = torch.empty(self.WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+            self._workspaces[key] = ws
+        return ws.data_ptr(), ws.numel()
 
     @staticmethod
     def _check_quant(x, qweight, scales, qzeros, group_size):
@@ -181,7 +204,9 @@ class W4A16Extension:
         if out is None:
             out = torch.empty((M, rank), dtype=torch.float16, device=x.device)
         with torch.cuda.device(x.device):
-            rc = self.lib.glowq_shared_proj(x.data_ptr(), R.data_ptr(), out.data_ptr(), M, K, rank, self._stream(x.device))
+            ws, ws_bytes = self._workspace(x.device, M)
+            rc = self.lib.glowq_shared_proj_ws(x.data_ptr(), R.data_ptr(), out.data_ptr(), M, K, rank, ws, ws_bytes,
+                                               self._stream(x.device))
         if rc:
             self._raise(rc, "shared_proj")
         return out
@@ -237,9 +262,10 @@ class W4A16Extension:
             return result
         with torch.cuda.device(x.device):
             if R is not None:
-                rc = self.lib.glowq_w4a16_group_forward_fused(
+                ws, ws_bytes = self._workspace(x.device, M)
+                rc = self.lib.glowq_w4a16_group_forward_fused_ws(
                     x.data_ptr(), R.data_ptr(), r.data_ptr(), arr, len(members), M, K, int(group_size),
-                    int(rank), float(alpha), self._stream(x.device))
+                    int(rank), float(alpha), ws, ws_bytes, self._stream(x.device))
             else:
                 rc = self.lib.glowq_w4a16_group_forward(
                     x.data_ptr(), r.data_ptr() if r is not None else None, arr, len(members), M, K, int(group_size),

@@ -22,6 +22,7 @@
 #ifndef GLOWQ_W4A16_H_
 #define GLOWQ_W4A16_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -100,6 +101,18 @@ int glowq_unpack_int4(const int32_t* packed, uint8_t* codes, int rows, int total
 int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int rank, void* stream);
 
 /*
+ * The same with a caller-provided workspace (same reference lines).  With more than 16 token rows the output [M, rank]
+ * is too small to fill the chip, so K is split over workgroups that leave fp32 partial tiles in `workspace`; a second
+ * small launch adds them in slice order (results do not depend on scheduling) and writes r.
+ * `workspace`: 16-byte aligned device memory, contents irrelevant; glowq_proj_workspace_bytes gives the size that lets
+ * the split go as far as it is useful for a shape -- a smaller one splits less, NULL or 0 bytes is glowq_shared_proj.
+ * Calls that share a workspace must not overlap (one workspace per stream).
+ */
+int glowq_shared_proj_ws(const void* x, const void* R, void* r, int M, int K, int rank, void* workspace,
+                         size_t workspace_bytes, void* stream);
+size_t glowq_proj_workspace_bytes(int M, int K, int rank);
+
+/*
  * One launch for a whole group: for every member i
  *     y_i = fp16( W4A16(x; member i) + bias_i + alpha * r @ L_i^T )
  * with r = the [M, rank] fp16 result of glowq_shared_proj (may be NULL when no member has L).
@@ -120,6 +133,10 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
  */
 int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
                                     int n_members, int M, int K, int group_size, int rank, float alpha, void* stream);
+/* The same with the projection workspace of glowq_shared_proj_ws (used when M > 16). */
+int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                       int n_members, int M, int K, int group_size, int rank, float alpha,
+                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,

@@ -117,3 +117,31 @@ def test_skinny_group_with_correction(ext, small_m_route, M, K, Ns, rank, alpha)
         else:
             want = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha)
         assert_close(y.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"skinny group member {i}")
+
+
+@pytest.mark.parametrize("M,K,rank", [(64, 14336, 128), (40, 8192, 256), (17, 17408, 256), (130, 18944, 64)])
+def test_shared_proj_split_workspace(ext, M, K, rank):
+    """Many-row projection with K split over workgroups through a workspace of any contents: same values on every call
+    (the partials are added in slice order), smaller workspaces split less, none not at all."""
+    g = torch.Generator().manual_seed(M + K + rank)
+    x = torch.randn(M, K, generator=g).half()
+    R = (torch.randn(rank, K, generator=g) * K ** -0.5).half()
+    want = x.numpy().astype(np.float64) @ R.numpy().astype(np.float64).T
+    xd, Rd = dev(x.numpy()), dev(R.numpy())
+    full = int(ext.lib.glowq_proj_workspace_bytes(M, K, rank))
+    assert full > 0
+    results = []
+    for nbytes in (full, full, full // 3, 2 * 4096 * 4, 0):
+        print(f"M={M} K={K} rank={rank} workspace={nbytes}", flush=True)
+        ws = torch.full((max(nbytes, 16),), 0xFF, dtype=torch.uint8, device="cuda")  # NaN patterns
+        out = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        for _ in range(3):  # the same workspace again and again
+            rc = ext.lib.glowq_shared_proj_ws(xd.data_ptr(), Rd.data_ptr(), out.data_ptr(), M, K, rank,
+                                              ws.data_ptr() if nbytes else None, nbytes, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, ext.lib.glowq_last_error()
+            torch.cuda.synchronize()
+            assert_close(out.cpu().numpy(), want, f"shared_proj_ws {nbytes} bytes")
+            results.append((nbytes, out.clone()))
+    first = results[0][1]
+    for nbytes, out in results[1:6]:
+        assert torch.equal(out, first), "same workspace size, different result"
