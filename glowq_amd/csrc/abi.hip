@@ -83,6 +83,8 @@ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 std::atomic<int> g_wave_dot_max_m{clampi(env_or("GLOWQ_WAVEDOT_M", kWaveDotMaxM), 0, kWaveDotMaxM)};
 std::atomic<int> g_quad_max_m{clampi(env_or("GLOWQ_QUAD_M", 4), 0, 16)};
 std::atomic<int> g_quad_min_m{clampi(env_or("GLOWQ_QUAD_MIN_M", 2), 1, 16)};
+//   skinny_max_m    rows up to which the skinny MFMA kernel is preferred over the tiled GEMM (GLOWQ_SKINNY_M)
+std::atomic<int> g_skinny_max_m{clampi(env_or("GLOWQ_SKINNY_M", 64), 0, 64)};
 int wave_dot_pref_m() { return g_wave_dot_max_m.load(std::memory_order_relaxed); }
 bool quad_wanted(int M) {
   return M >= g_quad_min_m.load(std::memory_order_relaxed) && M <= g_quad_max_m.load(std::memory_order_relaxed);
@@ -157,7 +159,9 @@ int pick_route(const GroupDev& g, int force) {
   }
   if (g.M <= wave_dot_pref_m() && force != kRouteSkinny && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
     return kRouteWaveDot;
-  if (skinny_supported(g)) return kRouteSkinny;
+  const bool skinny_ok = skinny_supported(g);
+  if (skinny_ok && (g.M <= g_skinny_max_m.load(std::memory_order_relaxed) || force == kRouteSkinny || !gemm_supported(g)))
+    return kRouteSkinny;
   if (gemm_supported(g)) return kRouteGemm;
   return kRouteGeneric;
 }
@@ -407,6 +411,7 @@ int glowq_set_tuning(const char* key, int value) {
   if (strcmp(key, "wave_dot_max_m") == 0) { slot = &g_wave_dot_max_m; hi = kWaveDotMaxM; }
   else if (strcmp(key, "quad_max_m") == 0) { slot = &g_quad_max_m; }
   else if (strcmp(key, "quad_min_m") == 0) { slot = &g_quad_min_m; lo = 1; }
+  else if (strcmp(key, "skinny_max_m") == 0) { slot = &g_skinny_max_m; hi = 64; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

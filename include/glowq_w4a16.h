@@ -147,9 +147,10 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
 /*
  * Route limits of the process (the reference's counterpart is the W4A16_GEMV_M_MAX family of environment
  * knobs, src/cuda_w4a16/linear.py:21-27,122): "quad_max_m" / "quad_min_m" bound the token rows served by the
- * 4x4x4 matrix-core GEMV (0 for quad_max_m switches it off), "wave_dot_max_m" those of the wave-dot GEMV.
+ * 4x4x4 matrix-core GEMV (0 for quad_max_m switches it off), "wave_dot_max_m" those of the wave-dot GEMV,
+ * "skinny_max_m" (at most 64) those of the skinny MFMA kernel, above which the tiled GEMM takes over.
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
- * GLOWQ_QUAD_MIN_M and GLOWQ_WAVEDOT_M.
+ * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M and GLOWQ_SKINNY_M.
  */
 int glowq_set_tuning(const char* key, int value);
 
