@@ -52,15 +52,15 @@ int fail(int code, const char* fmt, ...) {
 
 int num_cus() {
   // one value per device; the current device is the one the caller's tensors live on
-  static int cached[64] = {0};
+  static std::atomic<int> cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
+    cached[dev].store(n, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return n;
 }
 }  // namespace glowq
 
@@ -313,8 +313,8 @@ int glowq_shared_proj_ws(const void* x, const void* R, void* r, int M, int K, in
 
 size_t glowq_proj_workspace_bytes(int M, int K, int rank) { return proj_workspace_bytes(M, K, rank, num_cus()); }
 
-int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
-                              int K, int group_size, int rank, float alpha, void* stream) {
+static int group_forward_impl(const void* x, const void* r, const glowq_member_t* members, int n_members, int M, int K,
+                              int group_size, int rank, float alpha, void* ws, size_t ws_bytes, void* stream) {
   int rc = check_common(x, M, K, group_size);
   if (rc) return rc;
   if (members == nullptr || n_members < 1 || n_members > GLOWQ_MAX_MEMBERS)
@@ -338,11 +338,24 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
     for (int i = 0; i < n_members; ++i) g.mem[i].L = nullptr;  // alpha == 0: the reference returns z untouched
   }
   g.x = static_cast<const half_t*>(x);
+  g.ws = ws;
+  g.ws_bytes = ws_bytes;
   g.n_members = n_members;
   g.M = M;
   g.K = K;
   g.group_size = group_size;
   return run_group(g, pick_route(g, -1), static_cast<hipStream_t>(stream));
+}
+
+int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
+                              int K, int group_size, int rank, float alpha, void* stream) {
+  return group_forward_impl(x, r, members, n_members, M, K, group_size, rank, alpha, nullptr, 0, stream);
+}
+
+int glowq_w4a16_group_forward_ws(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
+                                 int K, int group_size, int rank, float alpha, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+  return group_forward_impl(x, r, members, n_members, M, K, group_size, rank, alpha, workspace, workspace_bytes, stream);
 }
 
 static int group_forward_fused_impl(const void* x, const void* R, void* r_out, const glowq_member_t* members,

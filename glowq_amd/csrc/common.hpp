@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/glowq_w4a16.h"
 
 namespace glowq {
@@ -52,18 +54,22 @@ int fail(int code, const char* fmt, ...);
 int num_cus();
 
 // Raises a kernel's dynamic LDS limit to `bytes` on the current device when that is above the 48 KB default and above
-// what this call site asked for before.  `raised` is the call site's own table (one slot per device).
+// what this call site asked for before.  `raised` is the call site's own table (one slot per device); host threads may
+// race on a slot, in which case the attribute is set more than once, to values that only grow.
 struct LdsLimit {
-  size_t raised[64] = {};
+  std::atomic<size_t> raised[64] = {};
 };
 inline hipError_t ensure_dynamic_lds(const void* kernel, size_t bytes, LdsLimit& site) {
   if (bytes <= 48 * 1024) return hipSuccess;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-  if (bytes <= site.raised[dev]) return hipSuccess;
+  if (bytes <= site.raised[dev].load(std::memory_order_acquire)) return hipSuccess;
   hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-  if (e == hipSuccess) site.raised[dev] = bytes;
-  return e;
+  if (e != hipSuccess) return e;
+  size_t seen = site.raised[dev].load(std::memory_order_relaxed);
+  while (seen < bytes && !site.raised[dev].compare_exchange_weak(seen, bytes, std::memory_order_release)) {
+  }
+  return hipSuccess;
 }
 
 __device__ __forceinline__ uint32_t nibble(uint32_t word, int idx) { return (word >> (4 * idx)) & 0xFu; }

@@ -18,6 +18,8 @@
 //     fp16 B operand, acc *= alpha, then the quantised K loop accumulates on top.
 #include <cstdlib>
 
+#include <algorithm>
+
 #include "common.hpp"
 
 namespace glowq {
@@ -44,6 +46,10 @@ struct GemmGroup {
   GemmArgs m[GLOWQ_MAX_MEMBERS];
   int blk_end[GLOWQ_MAX_MEMBERS];
   int n;
+  // split K (super-block form only): gridDim.y slices of whole super-blocks; every workgroup leaves its fp32 tile in
+  // `partials` ([slice][tile][BM * BN] in accumulator-register order) and gemm_reduce_kernel adds them in slice order
+  int slices;
+  float* partials;
 };
 
 __device__ __forceinline__ h8 permute_for_nibble_order(const h8& v) {
@@ -176,7 +182,7 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   int stage = 0;
 
   // ---- phase 1: the correction as a K-extension, acc = r . L^T, fp16 B operand ----------------------
-  if (kQuant && a.r != nullptr) {
+  if (kQuant && a.r != nullptr && blockIdx.y == 0) {
     const int steps = a.rank / kBK;
     load_a(a.r, a.rank, 0);
     store_a(stage, false);
@@ -299,12 +305,17 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
       __syncthreads();
       stage ^= 1;
     };
-    load_a_sub(areg, 0);
-    issue_b(0, bl);
-    load_a_sub(areg1, 1);
+    // this workgroup's super-blocks: all of them, or slice blockIdx.y of gg.slices
+    const int sb_total = steps >> 2;  // steps is a multiple of 4 here
+    const int sb_per = (sb_total + gg.slices - 1) / gg.slices;
+    const int ks0 = min((int)blockIdx.y * sb_per, sb_total) * 4;
+    const int ks1 = min(ks0 + sb_per * 4, steps);
+    load_a_sub(areg, ks0);
+    issue_b(ks0 >> 2, bl);
+    load_a_sub(areg1, ks0 + 1);
     store_a_from(areg, stage, true);
     __syncthreads();
-    for (int ks = 0; ks < steps; ks += 4) {  // steps is a multiple of 4 here
+    for (int ks = ks0; ks < ks1; ks += 4) {
       step(ks, 0, areg, areg1);
       step(ks + 1, 1, areg1, areg);
       step(ks + 2, 2, areg, areg1);
@@ -410,6 +421,18 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   }
 
   // ---- epilogue: accumulator register i of a 32x32 tile is row 8*(i/4) + 4*lh + i%4, column ln ---------
+  if constexpr (kQuant && kSuper) {
+    if (gg.slices > 1) {
+      float* part = gg.partials + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (BM * BN);
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) part[((tm * kNT + tn) * 16 + i) * 256 + tid] = acc[tm][tn][i];
+      return;
+    }
+  }
 #pragma unroll
   for (int tn = 0; tn < kNT; ++tn) {
     const int n = bn * BN + wave * (32 * kNT) + tn * 32 + ln;
@@ -421,6 +444,45 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
       for (int i = 0; i < 16; ++i) {
         const int m = m0 + tm * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
         if (m < a.M) a.y[(size_t)m * a.ldy + n] = (half_t)(acc[tm][tn][i] + b);
+      }
+    }
+  }
+}
+
+// y = fp16(sum over the slices, in slice order, of the partial tiles of gemm_mfma_kernel<kMT, kNT> + bias); same grid
+// in x, same workgroup -> (member, row block, column block) map and accumulator-register order as the producer.
+template <int kMT, int kNT>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, const int m_blocks) {
+  GemmArgs a = gg.m[0];
+  int blk_base = 0;
+  for (int i = 1; i < gg.n; ++i)
+    if ((int)blockIdx.x >= gg.blk_end[i - 1]) {
+      a = gg.m[i];
+      blk_base = gg.blk_end[i - 1];
+    }
+  constexpr int BM = 32 * kMT, BN = 128 * kNT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, lh = lane >> 5;
+  const int blk = (int)blockIdx.x - blk_base;
+  const int m0 = (blk % m_blocks) * BM, bn = blk / m_blocks;
+  const size_t slice_stride = (size_t)gridDim.x * (BM * BN);
+  const float* part = gg.partials + (size_t)blockIdx.x * (BM * BN) + tid;
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) {
+    const int n = bn * BN + wave * (32 * kNT) + tn * 32 + ln;
+    const float b = (n < a.N && a.bias) ? (float)a.bias[n] : 0.f;
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm) {
+      float v[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.f;
+      for (int z = 0; z < gg.slices; ++z) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += part[(size_t)z * slice_stride + ((tm * kNT + tn) * 16 + i) * 256];
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + tm * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+        if (m < a.M && n < a.N) a.y[(size_t)m * a.ldy + n] = (half_t)(v[i] + b);
       }
     }
   }
@@ -440,7 +502,10 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
     total += m_blocks * ((gg.m[i].N + BN - 1) / BN);
     gg.blk_end[i] = total;
   }
-  hipLaunchKernelGGL(kern, dim3(total), dim3(256), lds, stream, gg, m_blocks);
+  if (!(kQuant && kSuper)) gg.slices = 1;
+  hipLaunchKernelGGL(kern, dim3(total, gg.slices), dim3(256), lds, stream, gg, m_blocks);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess || gg.slices == 1) return e;
+  hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(total), dim3(256), 0, stream, gg, m_blocks);
   return hipGetLastError();
 }
 
@@ -481,6 +546,29 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stre
   if (force_nt > 0 && force_nt <= nt_cap) nt = force_nt;
   static const int env_super = getenv("GLOWQ_GEMM_SUPER") ? atoi(getenv("GLOWQ_GEMM_SUPER")) : 1;
   const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128;
+  // Split K through the workspace: where even the largest tile the rows allow leaves CUs idle, that tile is kept and K
+  // is cut into slices of at least sixteen super-blocks until the workgroups number about two per CU.
+  static const int env_split = getenv("GLOWQ_GEMM_SPLIT") ? atoi(getenv("GLOWQ_GEMM_SPLIT")) : 1;
+  const int ws_slices_fit = gg.slices;  // on entry: how many slices of the whole output the workspace holds
+  gg.slices = 1;
+  if (super && env_split != 0 && ws_slices_fit >= 2 && mt_cap >= 2 && nt_cap == 2) {
+    const int bmt = mt_cap >= 4 ? 4 : 2;
+    long tiles = 0;
+    for (int i = 0; i < gg.n; ++i) tiles += (long)((M + 32 * bmt - 1) / (32 * bmt)) * ((gg.m[i].N + 255) / 256);
+    const int sb_total = gg.m[0].K >> 8;
+    long want = (2L * num_cus) / tiles;
+    // every slice writes the whole output once more in fp32, the reduction reads it back, and a short K loop is mostly
+    // ramp: only slices of 16 super-blocks and more pay (measured: 2048 x 3584 outputs gain 8 % at K = 18944 in two
+    // slices and lose 12 % at K = 3584; 128..512 rows of K = 4096 lose up to 40 % in slices of four super-blocks)
+    constexpr long min_depth = 16;
+    if (want > sb_total / min_depth) want = sb_total / min_depth;
+    if (want > ws_slices_fit) want = ws_slices_fit;
+    if (tiles < num_cus && want >= 2 && tiles * want * 2 >= num_cus) {
+      mt = bmt;
+      nt = 2;
+      gg.slices = (int)want;
+    }
+  }
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
   if (mt == MT && nt == NT)                                                                \
     return super ? launch_gemm_t<MT, NT, true, true>(gg, stream) : launch_gemm_t<MT, NT, true>(gg, stream);
@@ -531,6 +619,13 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
     a.ldy = m.ldy;
     a.alpha = g.alpha;
   }
+  // slices of the padded output (rows to a multiple of 128, columns of every member to a multiple of 256) that fit the
+  // workspace; launch_gemm_group turns this into the slice count
+  size_t padded = 0;
+  for (int i = 0; i < g.n_members; ++i) padded += (size_t)((g.M + 127) / 128 * 128) * ((g.mem[i].N + 255) / 256 * 256);
+  const bool ws_ok = g.ws != nullptr && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0;
+  gg.slices = ws_ok ? (int)std::min<size_t>(g.ws_bytes / (padded * sizeof(float)), 64) : 0;
+  gg.partials = static_cast<float*>(g.ws);
   return launch_gemm_group(gg, num_cus, stream);
 }
 

@@ -349,9 +349,9 @@ static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int m
   const int threads = waves * kWave;
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
-  // resident workgroups per CU for this block size and LDS footprint; the last answer is remembered
-  static int last_threads = 0, last_occ = 0;
-  static size_t last_lds = 0;
+  // resident workgroups per CU for this block size and LDS footprint; each host thread remembers its last answer
+  static thread_local int last_threads = 0, last_occ = 0;
+  static thread_local size_t last_lds = 0;
   int occ = last_occ;
   if (last_occ == 0 || last_threads != threads || last_lds != lds) {
     hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), threads, lds);

@@ -49,6 +49,8 @@ _SIGNATURES = {
     "glowq_shared_proj": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "glowq_shared_proj_ws": (_I, [_P, _P, _P, _I, _I, _I, _P, ctypes.c_size_t, _P]),
     "glowq_proj_workspace_bytes": (ctypes.c_size_t, [_I, _I, _I]),
+    "glowq_w4a16_group_forward_ws": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P,
+                                          ctypes.c_size_t, _P]),
     "glowq_w4a16_group_forward_fused_ws": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float,
                                                 _P, ctypes.c_size_t, _P]),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
@@ -92,11 +94,11 @@ class W4A16Extension:
     def _stream(dev: torch.device) -> int:
         return torch.cuda.current_stream(dev).cuda_stream
 
-    WORKSPACE_BYTES = 16 << 20
+    WORKSPACE_BYTES = 64 << 20
 
     def _workspace(self, dev: torch.device, rows: int):
-        """(pointer, bytes) of the projection workspace of the current stream of `dev`: one per stream, because calls
-        that share one must not overlap.  Only calls with more than 16 token rows use it.  A stream that meets its
+        """(pointer, bytes) of the workspace of the current stream of `dev` (many-row projection, split-K of the GEMM):
+        one per stream, because calls that share one must not overlap.  Only calls with more than 16 token rows use it.  A stream that meets its
         first such call while it is being captured into a graph goes without (the buffer would come from the graph's
         own memory pool)."""
         if rows <= 16:
@@ -267,9 +269,10 @@ class W4A16Extension:
                     x.data_ptr(), R.data_ptr(), r.data_ptr(), arr, len(members), M, K, int(group_size),
                     int(rank), float(alpha), ws, ws_bytes, self._stream(x.device))
             else:
-                rc = self.lib.glowq_w4a16_group_forward(
+                ws, ws_bytes = self._workspace(x.device, M)
+                rc = self.lib.glowq_w4a16_group_forward_ws(
                     x.data_ptr(), r.data_ptr() if r is not None else None, arr, len(members), M, K, int(group_size),
-                    int(rank), float(alpha), self._stream(x.device))
+                    int(rank), float(alpha), ws, ws_bytes, self._stream(x.device))
         if rc:
             self._raise(rc, "w4a16_group_forward")
         return result

@@ -133,7 +133,16 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
  */
 int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
                                     int n_members, int M, int K, int group_size, int rank, float alpha, void* stream);
-/* The same with the projection workspace of glowq_shared_proj_ws (used when M > 16). */
+/*
+ * The two group entry points with a workspace (16-byte aligned device memory, contents irrelevant, not shared by calls
+ * that overlap).  It serves the many-row projection as in glowq_shared_proj_ws and, on the tiled GEMM route, a split of
+ * K where the output has too few tiles to fill the chip (long K, few columns: o_proj / down_proj at some hundred
+ * rows): partial fp32 tiles, added in slice order by a second launch.  A slice of the split takes
+ * 4 * roundup(M, 128) * sum_i roundup(N_i, 256) bytes; the split goes as far as the workspace holds slices.
+ */
+int glowq_w4a16_group_forward_ws(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
+                                 int K, int group_size, int rank, float alpha, void* workspace, size_t workspace_bytes,
+                                 void* stream);
 int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out, const glowq_member_t* members,
                                        int n_members, int M, int K, int group_size, int rank, float alpha,
                                        void* workspace, size_t workspace_bytes, void* stream);

@@ -145,3 +145,37 @@ def test_shared_proj_split_workspace(ext, M, K, rank):
     first = results[0][1]
     for nbytes, out in results[1:6]:
         assert torch.equal(out, first), "same workspace size, different result"
+
+
+@pytest.mark.parametrize("M,K,Ns,rank", [(512, 16384, [2048], 64), (1024, 8192, [2048, 1024], 128), (300, 17408, [2000], 0),
+                                         (128, 14336, [4096], 128)])
+def test_gemm_split_k_through_workspace(ext, M, K, Ns, rank):
+    """Tiled GEMM with K split over workgroups (few output tiles, long K): against the oracle, the same bits on every
+    call, and with workspaces that hold fewer slices or none."""
+    x, members, R = make_group(5 + M + K, M, K, Ns, rank, with_bias=True)
+    xd = dev(x)
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]),
+            "L": dev(m["L"]) if rank else None, "bias": dev(m["bias"])} for m in members]
+    if rank:
+        r = ext.shared_proj(xd, dev(R))
+        want = [oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0) for m in members]
+    else:
+        r = None
+        want = [oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128) for m in members]
+    want = [w + m["bias"].astype(np.float64)[None, :] for w, m in zip(want, members)]
+    slice_bytes = 4 * ((M + 127) // 128 * 128) * sum((N + 255) // 256 * 256 for N in Ns)
+    seen = {}
+    for nbytes in (64 << 20, 64 << 20, 2 * slice_bytes, slice_bytes, 0):
+        print(f"M={M} K={K} Ns={Ns} rank={rank} workspace={nbytes}", flush=True)
+        ext.WORKSPACE_BYTES = max(nbytes, 16)
+        ext._workspaces.clear()
+        outs = ext.group_forward(xd, r, mem, 128, 1.0)
+        torch.cuda.synchronize()
+        for i, y in enumerate(outs):
+            assert_close(y.cpu().numpy(), want[i], f"member {i}, workspace {nbytes}")
+        if nbytes in seen:
+            for a, b in zip(outs, seen[nbytes]):
+                assert torch.equal(a, b), "same workspace size, different bits"
+        seen[nbytes] = [o.clone() for o in outs]
+    ext.WORKSPACE_BYTES = 64 << 20
+    ext._workspaces.clear()
