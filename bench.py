@@ -243,6 +243,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill leg and print it (profiling runs)")
     ap.add_argument("--selective-only", action="store_true", help="run only the GlowQ-S leg and print it")
+    ap.add_argument("--no-decode-loop", action="store_true", help="skip the full decode loop leg (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of known size (256 MiB read + 256 MiB written each) so that "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiling run can be scaled")
@@ -402,6 +403,14 @@ def main():
     del layers, graph, gdom
     torch.cuda.empty_cache()
     selective = selective_leg(torch, ext, dev)
+    # the whole decode loop of the same benchmark (32-layer random-init model, 512-token prompt, 256 new tokens, greedy)
+    torch.cuda.empty_cache()
+    decode = None
+    if not args.no_decode_loop:
+        import contextlib
+        from glowq_amd import decode as decode_loop
+        with contextlib.redirect_stdout(sys.stderr):  # the patcher reports what it wrapped; stdout carries the JSON line only
+            decode = decode_loop.measure(32, 512, 256)
 
     result = {
         "metric": "W4A16+GlowQ decode linears, microseconds per layer (Llama-3.1-8B shape, batch 1)",
@@ -430,6 +439,7 @@ def main():
         "batched_rows_us_per_layer": batched,
         "prefill": prefill,
         "selective": selective,
+        "decode_loop": decode,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",

@@ -424,6 +424,31 @@ class GreedyDecoder:
         return out.cpu(), ttfb, decode_s
 
 
+def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
+            fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 4) -> dict:
+    """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
+    second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798)."""
+    import os
+
+    os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    cfg = DecoderConfig(layers=layers, vocab=vocab, max_len=max(1024, prompt_tokens + new_tokens + 8))
+    t0 = time.perf_counter()
+    model, _, _ = build_decoder(cfg, with_correction=correction)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits)
+    g = torch.Generator().manual_seed(3)
+    prompt = torch.randint(0, cfg.vocab, (prompt_tokens,), generator=g)
+    dec.generate(prompt, 4)  # warm-up (also captures the graph)
+    _, ttfb, decode_s = dec.generate(prompt, new_tokens)
+    return {
+        "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
+                    f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + (f" + GlowQ r={cfg.rank}" if correction else ""),
+        "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "graph": graph, "fused_step": fused, "group_sharing": share,
+        "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((new_tokens - 1) / decode_s, 1),
+        "ms_per_token": round(decode_s * 1e3 / (new_tokens - 1), 3), "build_s": round(build_s, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--layers", type=int, default=32)
@@ -436,26 +461,9 @@ def main():
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--attention-splits", type=int, default=4, help="workgroups per head in the fused step's attention")
     args = ap.parse_args()
-    import os
-
-    os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
-    cfg = DecoderConfig(layers=args.layers, vocab=args.vocab, max_len=max(1024, args.prompt + args.new + 8))
-    t0 = time.perf_counter()
-    model, _, _ = build_decoder(cfg, with_correction=not args.no_correction)
-    torch.cuda.synchronize()
-    build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=not args.no_graph, fused=not args.module_path, share=not args.no_sharing,
-                        attention_splits=args.attention_splits)
-    g = torch.Generator().manual_seed(3)
-    prompt = torch.randint(0, cfg.vocab, (args.prompt,), generator=g)
-    dec.generate(prompt, 4)  # warm-up (also captures the graph)
-    _, ttfb, decode_s = dec.generate(prompt, args.new)
-    print(json.dumps({
-        "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
-                    f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + ("" if args.no_correction else f" + GlowQ r={cfg.rank}"),
-        "prompt_tokens": args.prompt, "new_tokens": args.new, "graph": not args.no_graph, "fused_step": not args.module_path, "group_sharing": not args.no_sharing,
-        "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((args.new - 1) / decode_s, 1),
-        "ms_per_token": round(decode_s * 1e3 / (args.new - 1), 3), "build_s": round(build_s, 1)}))
+    print(json.dumps(measure(args.layers, args.prompt, args.new, vocab=args.vocab, graph=not args.no_graph,
+                             fused=not args.module_path, share=not args.no_sharing, correction=not args.no_correction,
+                             attention_splits=args.attention_splits)))
 
 
 if __name__ == "__main__":
