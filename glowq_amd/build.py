@@ -28,6 +28,9 @@ HIPCC_FLAGS = [
     "-Wno-unused-function",
     # keep hipcc from forming packed-fp32 instructions out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first kernel arguments arrive in scalar registers with the wave instead of through a load from the argument
+    # buffer (a memory round trip at the head of every wave; kernels keep a prologue for firmware without the feature)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 

@@ -370,7 +370,8 @@ static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int m
     const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
     wgs_needed += (blocks + waves - 1) / waves;
   }
-  const int rounds = wgs_needed > resident ? (wgs_needed + resident - 1) / resident : 1;
+  static const int persist = env_int("GLOWQ_GEMV_PERSIST", 1);
+  const int rounds = (persist != 0 && wgs_needed > resident) ? (wgs_needed + resident - 1) / resident : 1;
   GroupDev gl = g;
   int grid = 0;
   for (int i = 0; i < g.n_members; ++i) {
