@@ -98,7 +98,12 @@ struct Prefetch {
 // scalar registers and nothing is looked up in memory between two prefetches.
 template <int kM, int kRows, int kLW, bool kWide>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(((kM >= 2 || kRows >= 4) ? 4 : 6), 8)))
-void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
+void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const int head_ldw, const int head_rows,
+                          const int head_blocks, const int head_wg_end, const int head_units, const int head_waves,
+                          const GroupDev g, const int kit) {
+  // The head_* arguments repeat what a workgroup of the FIRST member needs to request the weights of its first step:
+  // plain leading arguments reach the wave in scalar registers, everything inside `g` takes a load from the argument
+  // buffer (a memory round trip).  Those workgroups -- all of them for a group of one -- start that much earlier.
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int U = g.K >> 5;                                  // 16-byte units per weight row
   const int upg_shift = __builtin_ctz(g.group_size >> 5);  // units per quantisation group = 1 << upg_shift
@@ -108,6 +113,17 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  Prefetch<kRows, kLW, kWide> buf0, buf1;
+  const bool head = (int)blockIdx.x < head_wg_end;
+  if (head) {
+    const int n0 = min((int)blockIdx.x * head_waves + wave, head_blocks - 1) * kRows;
+    const int u = min(lane, head_units - 1);
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const int n = min(n0 + r, head_rows - 1);
+      buf0.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(head_qweight + (size_t)n * head_ldw) + u);
+    }
+  }
   const int waves_per_block = blockDim.x >> 6;
 
   // member of this workgroup: every candidate field comes from a fixed kernel-argument offset and is
@@ -136,14 +152,15 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   };
   const int side_row = min(lane >> 4, kRows - 1), side_idx = lane & 15;
   const int gps_shift = 6 - upg_shift;  // log2 of the groups per row and step
-  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kWide>& p) {
+  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kWide>& p, const bool weights_requested = false) {
     const int n0 = min(c.blk, total_blocks - 1) * kRows;
     const int u = min(lane + c.it * kWave, U - 1);
     const int grp = u >> upg_shift;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
       const int n = min(n0 + r, mem.N - 1);
-      p.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw) + u);
+      if (!weights_requested)
+        p.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw) + u);
       if constexpr (!kWide) {
         p.sc[r] = mem.scales[(size_t)n * mem.lds + grp];
         p.zw[r] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (grp >> 3)];
@@ -256,8 +273,7 @@ void gemv_wave_dot_kernel(const GroupDev g, const int kit) {
   Cursor ahead;
   ahead.blk = ((int)blockIdx.x - wg_begin) * waves_per_block + wave;
   ahead.it = 0;
-  Prefetch<kRows, kLW, kWide> buf0, buf1;
-  issue(ahead, buf0);
+  issue(ahead, buf0, head);
 
   stage_activations<kM>(g, U, xs, sig, rs);
   __syncthreads();
@@ -380,7 +396,8 @@ static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int m
     grid += wg_i < 1 ? 1 : wg_i;
     gl.wg_end[i] = grid;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl, kit);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl.mem[0].qweight, gl.mem[0].ldw, gl.mem[0].N, gl.task_end[0],
+                     gl.wg_end[0], gl.K >> 5, waves, gl, kit);
   return hipGetLastError();
 }
 
