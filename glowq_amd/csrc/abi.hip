@@ -13,6 +13,7 @@ namespace glowq {
 hipError_t launch_wave_dot(GroupDev& g, int rows_per_task, int num_cus, hipStream_t stream);
 hipError_t launch_generic(GroupDev& g, int num_cus, hipStream_t stream);
 int wave_dot_rows(long total_rows);
+int wave_dot_rows_single(long total_rows);
 bool wave_dot_supported(int M, int K, int rank, bool has_r);
 // gemv_quad.hip
 int quad_capacity(int M, int K, int rank, bool has_r);
@@ -201,7 +202,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
       g.x = x0 + (size_t)m0 * g.K;
       g.r = r0 ? r0 + (size_t)m0 * g.rank : nullptr;
       for (int i = 0; i < g.n_members; ++i) g.mem[i].y = y0[i] + (size_t)m0 * g.mem[i].ldy;
-      e = (route == kRouteWaveDot) ? launch_wave_dot(g, wave_dot_rows(rows), cus, stream)
+      e = (route == kRouteWaveDot) ? launch_wave_dot(g, g.M == 1 ? wave_dot_rows_single(rows) : wave_dot_rows(rows), cus, stream)
           : (route == kRouteQuad)  ? launch_quad(g, cus, stream)
                                    : launch_generic(g, cus, stream);
     }

@@ -362,40 +362,76 @@ template <int kM, int kRows, int kLW, bool kWide>
 static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int max_wg_per_cu, int num_cus, size_t lds,
                                     hipStream_t stream) {
   auto kern = gemv_wave_dot_kernel<kM, kRows, kLW, kWide>;
-  const int threads = waves * kWave;
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
-  // resident workgroups per CU for this block size and LDS footprint; each host thread remembers its last answer
-  static thread_local int last_threads = 0, last_occ = 0;
-  static thread_local size_t last_lds = 0;
-  int occ = last_occ;
-  if (last_occ == 0 || last_threads != threads || last_lds != lds) {
-    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), threads, lds);
-    if (e != hipSuccess) return e;
-    if (occ < 1) occ = 1;
-    last_threads = threads;
-    last_lds = lds;
-    last_occ = occ;
-  }
-  if (max_wg_per_cu > 0 && occ > max_wg_per_cu) occ = max_wg_per_cu;
+  // resident workgroups per CU for a block size and LDS footprint; each host thread remembers its last answers
+  auto occupancy = [&](int threads, int& occ) -> hipError_t {
+    static thread_local int last_threads[2] = {0, 0}, last_occ[2] = {0, 0};
+    static thread_local size_t last_lds[2] = {0, 0};
+    const int slot = threads == 8 * kWave ? 0 : 1;
+    if (last_occ[slot] == 0 || last_threads[slot] != threads || last_lds[slot] != lds) {
+      int o = 0;
+      hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, reinterpret_cast<const void*>(kern), threads, lds);
+      if (e != hipSuccess) return e;
+      last_threads[slot] = threads;
+      last_lds[slot] = lds;
+      last_occ[slot] = o < 1 ? 1 : o;
+    }
+    occ = last_occ[slot];
+    if (max_wg_per_cu > 0 && occ > max_wg_per_cu) occ = max_wg_per_cu;
+    return hipSuccess;
+  };
   // Split the grid between the members in proportion to their row blocks; when everything does not
   // fit on the chip at once the waves become persistent and walk an equal number of row blocks.
-  const int resident = num_cus * occ;
-  int wgs_needed = 0;
-  for (int i = 0; i < g.n_members; ++i) {
-    const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
-    wgs_needed += (blocks + waves - 1) / waves;
-  }
   static const int persist = env_int("GLOWQ_GEMV_PERSIST", 1);
-  const int rounds = (persist != 0 && wgs_needed > resident) ? (wgs_needed + resident - 1) / resident : 1;
-  GroupDev gl = g;
-  int grid = 0;
-  for (int i = 0; i < g.n_members; ++i) {
-    const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
-    const int wg_i = ((blocks + waves - 1) / waves + rounds - 1) / rounds;
-    grid += wg_i < 1 ? 1 : wg_i;
-    gl.wg_end[i] = grid;
+  struct Plan {
+    int grid, rounds, wg_end[GLOWQ_MAX_MEMBERS];
+    double cost;  // time of the most loaded CU over the mean, times the same for the most loaded wave
+  };
+  auto plan = [&](int w, int occ) {
+    Plan p;
+    const int resident = num_cus * occ;
+    int wgs_needed = 0;
+    for (int i = 0; i < g.n_members; ++i) {
+      const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
+      wgs_needed += (blocks + w - 1) / w;
+    }
+    p.rounds = (persist != 0 && wgs_needed > resident) ? (wgs_needed + resident - 1) / resident : 1;
+    p.grid = 0;
+    double wave_imbalance = 1.0;
+    for (int i = 0; i < g.n_members; ++i) {
+      const int blocks = g.task_end[i] - (i ? g.task_end[i - 1] : 0);
+      int wg_i = ((blocks + w - 1) / w + p.rounds - 1) / p.rounds;
+      if (wg_i < 1) wg_i = 1;
+      p.grid += wg_i;
+      p.wg_end[i] = p.grid;
+      const long slots = (long)wg_i * w;
+      const double imb = (double)((blocks + slots - 1) / slots * slots) / (double)blocks;
+      wave_imbalance = imb > wave_imbalance ? imb : wave_imbalance;
+    }
+    const int per_cu = (p.grid + num_cus - 1) / num_cus;
+    p.cost = wave_imbalance * (double)per_cu * num_cus / (double)p.grid;
+    return p;
+  };
+  int occ = 1;
+  if (hipError_t e = occupancy(waves * kWave, occ); e != hipSuccess) return e;
+  Plan chosen = plan(waves, occ);
+  // A long single-row group (persistent waves): 7 waves per workgroup where that spreads the workgroups evenly over
+  // the CUs and the row blocks evenly over the waves and 8 do not (28672 rows: 512 workgroups of 7 waves, two on every
+  // CU, against 448 of 8, two on three quarters of the CUs: 14.5 against 15.1 us).
+  if (kM == 1 && waves == 8 && chosen.rounds > 1 && tuning_override().waves == 0) {
+    int occ7 = 1;
+    if (hipError_t e = occupancy(7 * kWave, occ7); e != hipSuccess) return e;
+    const Plan alt = plan(7, occ7);
+    if (alt.rounds > 1 && alt.cost < 0.97 * chosen.cost) {
+      chosen = alt;
+      waves = 7;
+    }
   }
+  const int threads = waves * kWave;
+  GroupDev gl = g;
+  const int grid = chosen.grid;
+  for (int i = 0; i < g.n_members; ++i) gl.wg_end[i] = chosen.wg_end[i];
   hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl.mem[0].qweight, gl.mem[0].ldw, gl.mem[0].N, gl.task_end[0],
                      gl.wg_end[0], gl.K >> 5, waves, gl, kit);
   return hipGetLastError();
@@ -415,6 +451,14 @@ int wave_dot_rows(long total_rows) {
   const int o = tuning_override().rows;
   if (o == 1 || o == 2 || o == 4) return o;
   return total_rows >= 8192 ? 4 : 2;
+}
+// Single-row decode: two rows per row block throughout (four measured 2 % slower on the long groups once the first
+// request of a wave no longer waits for the argument buffer).
+int wave_dot_rows_single(long total_rows) {
+  const int o = tuning_override().rows;
+  if (o == 1 || o == 2 || o == 4) return o;
+  (void)total_rows;
+  return 2;
 }
 
 hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStream_t stream) {
