@@ -378,19 +378,34 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
     }
   }
   __syncthreads();
+  // the waves' partials meet: the first nw lanes of wave 0 turn the waves' maxima into weights (and the sum of the
+  // weighted sums), then one thread per dimension adds the weighted accumulators
+  if (wave == 0) {
+    const float mw = lane < nw ? wave_m[lane] : -INFINITY;
+    float mx = mw;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float wgt = (mw == -INFINITY) ? 0.f : __expf(mw - mx);
+    float sum = lane < nw ? wave_l[lane] * wgt : 0.f;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o);
+    if (lane < nw) wave_m[lane] = wgt;  // from here on: the wave's weight
+    if (lane == 0) {
+      wave_l[0] = sum;
+      wave_l[1] = mx;
+    }
+  }
+  __syncthreads();
   float* mine = part ? part + ((size_t)head * splits + split) * (d + 4) : nullptr;
-  float mx = -INFINITY;
-  for (int w = 0; w < nw; ++w) mx = fmaxf(mx, wave_m[w]);
-  float sum = 0.f;
-  for (int w = 0; w < nw; ++w) sum += (wave_m[w] == -INFINITY) ? 0.f : wave_l[w] * __expf(wave_m[w] - mx);
+  const float sum = wave_l[0];
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
     float t = 0.f;
-    for (int w = 0; w < nw; ++w) t += (wave_m[w] == -INFINITY) ? 0.f : acc_part[w * d + i] * __expf(wave_m[w] - mx);
+    for (int w = 0; w < nw; ++w) t = __builtin_fmaf(acc_part[w * d + i], wave_m[w], t);
     if (part) mine[4 + i] = t;
     else out[(size_t)head * d + i] = (half_t)(t / sum);
   }
   if (part && threadIdx.x == 0) {
-    mine[0] = mx;   // -inf for a split without rows: its weight in the combination is exp(-inf) = 0
+    mine[0] = wave_l[1];  // -inf for a split without rows: its weight in the combination is exp(-inf) = 0
     mine[1] = sum;
   }
 }
