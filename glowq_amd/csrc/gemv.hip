@@ -55,6 +55,47 @@ __device__ __forceinline__ void stage_activations(const GroupDev& g, int U, h8* 
   }
 }
 
+// The same staging for one token row in two halves: the loads go out at the head of the kernel, from pointers that
+// arrive in scalar registers, and are written to LDS when the rest of the set-up is done.  Thread t holds words
+// t, t + blockDim, ... (at most kXWords) and two halves of r.
+constexpr int kXWords = 4;
+struct XRegs {
+  h8 v[kXWords];
+  uint32_t r;
+};
+__device__ __forceinline__ bool early_staging_fits(int K, int rank, const half_t* r, int threads) {
+  return (K >> 3) <= kXWords * threads && (r == nullptr || (rank <= 2 * threads && (reinterpret_cast<uintptr_t>(r) & 3u) == 0));
+}
+__device__ __forceinline__ void load_activations(const half_t* x, const half_t* r, int K, int rank, int threads, XRegs& xr) {
+  const int words = K >> 3;
+  const h8* xrow = reinterpret_cast<const h8*>(x);
+#pragma unroll
+  for (int i = 0; i < kXWords; ++i) xr.v[i] = xrow[min((int)threadIdx.x + i * threads, words - 1)];
+  xr.r = 0u;
+  if (r != nullptr) xr.r = reinterpret_cast<const uint32_t*>(r)[min((int)threadIdx.x, (rank >> 1) - 1)];
+}
+__device__ __forceinline__ void store_activations(const half_t* r, int K, int rank, int threads, int U, const XRegs& xr,
+                                                  h8* xs, float* sig, half_t* rs) {
+  const int words = K >> 3;
+#pragma unroll
+  for (int i = 0; i < kXWords; ++i) {
+    const int w = threadIdx.x + i * threads;
+    const h8 v = xr.v[i];
+    float s = ((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3]) +
+              (((float)v[4] + (float)v[5]) + ((float)v[6] + (float)v[7]));
+    s = quad_sum(s);  // threads and words are multiples of 4: a quad lies inside the row or outside as a whole
+    if (w < words) {
+      h8 p;
+      p[0] = v[0]; p[1] = v[4]; p[2] = v[1]; p[3] = v[5];
+      p[4] = v[2]; p[5] = v[6]; p[6] = v[3]; p[7] = v[7];
+      const int u = w >> 2, j = w & 3;
+      xs[(size_t)j * U + u] = p;
+      if (j == 0) sig[u] = s * 0x1p-24f;
+    }
+  }
+  if (r != nullptr && (int)threadIdx.x < (rank >> 1)) reinterpret_cast<uint32_t*>(rs)[threadIdx.x] = xr.r;
+}
+
 __device__ __forceinline__ void dot_word(uint32_t w, const h8& xq, float& accA, float& accB) {
   // nibbles (0,4) and (2,6) land in mantissa bits 0-3, nibbles (1,5) and (3,7) in bits 4-7.
   const uint32_t hi = w >> 8;
@@ -98,9 +139,10 @@ struct Prefetch {
 // scalar registers and nothing is looked up in memory between two prefetches.
 template <int kM, int kRows, int kLW, bool kWide>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(((kM >= 2 || kRows >= 4) ? 4 : 6), 8)))
-void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const int head_ldw, const int head_rows,
+void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t* __restrict__ head_x,
+                          const half_t* __restrict__ head_r, const int head_ldw, const int head_rows,
                           const int head_blocks, const int head_wg_end, const int head_units, const int head_waves,
-                          const GroupDev g, const int kit) {
+                          const int head_rank, const GroupDev g, const int kit) {
   // The head_* arguments repeat what a workgroup of the FIRST member needs to request the weights of its first step:
   // plain leading arguments reach the wave in scalar registers, everything inside `g` takes a load from the argument
   // buffer (a memory round trip).  Those workgroups -- all of them for a group of one -- start that much earlier.
@@ -124,6 +166,10 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const int he
       buf0.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(head_qweight + (size_t)n * head_ldw) + u);
     }
   }
+  // single token row: the activations (and r) are requested here as well, from leading arguments
+  XRegs xr;
+  const bool early_x = kM == 1 && early_staging_fits(head_units << 5, head_rank, head_r, head_waves * kWave);
+  if (kM == 1 && early_x) load_activations(head_x, head_r, head_units << 5, head_rank, head_waves * kWave, xr);
   const int waves_per_block = blockDim.x >> 6;
 
   // member of this workgroup: every candidate field comes from a fixed kernel-argument offset and is
@@ -275,7 +321,8 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const int he
   ahead.it = 0;
   issue(ahead, buf0, head);
 
-  stage_activations<kM>(g, U, xs, sig, rs);
+  if (kM == 1 && early_x) store_activations(head_r, head_units << 5, head_rank, head_waves * kWave, U, xr, xs, sig, rs);
+  else stage_activations<kM>(g, U, xs, sig, rs);
   __syncthreads();
 
   while (ahead.blk < total_blocks) {
@@ -432,8 +479,8 @@ static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int m
   GroupDev gl = g;
   const int grid = chosen.grid;
   for (int i = 0; i < g.n_members; ++i) gl.wg_end[i] = chosen.wg_end[i];
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl.mem[0].qweight, gl.mem[0].ldw, gl.mem[0].N, gl.task_end[0],
-                     gl.wg_end[0], gl.K >> 5, waves, gl, kit);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, stream, gl.mem[0].qweight, gl.x, gl.r, gl.mem[0].ldw, gl.mem[0].N,
+                     gl.task_end[0], gl.wg_end[0], gl.K >> 5, waves, gl.r ? gl.rank : 0, gl, kit);
   return hipGetLastError();
 }
 
