@@ -49,11 +49,16 @@ __device__ __forceinline__ h8 nibble_order(const u32x4& v) {
 }
 
 __device__ __forceinline__ h8 dequant_word_sk(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2) {
+  // the two exponent patterns (1024.0 and 64.0 in both halves) are held in vector registers: with the nibble mask as
+  // the one scalar operand each mask-and-merge is a single v_and_or_b32 instead of an AND and an OR
+  uint32_t e1024, e64;
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(e1024));
+  asm("v_mov_b32 %0, 0x54005400" : "=v"(e64));
   const uint32_t hi = w >> 8;
-  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | 0x64006400u);
-  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | 0x54005400u);
-  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | 0x64006400u);
-  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | 0x54005400u);
+  const h2 q0 = bitcast_u32<h2>((w & 0x000F000Fu) | e1024);
+  const h2 q1 = bitcast_u32<h2>((w & 0x00F000F0u) | e64);
+  const h2 q2 = bitcast_u32<h2>((hi & 0x000F000Fu) | e1024);
+  const h2 q3 = bitcast_u32<h2>((hi & 0x00F000F0u) | e64);
   const h2 d0 = (q0 + zb_lo) * s2;
   const h2 d1 = (q1 + zb_hi) * s2;
   const h2 d2 = (q2 + zb_lo) * s2;
@@ -365,17 +370,19 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     for (int q = 0; q < kMT * 8; ++q) {
       const int seg = q * 8 + (lane >> 3);             // (token row, half of the super-block)
       const int row = min(seg >> 1, g.M - 1);
-      // loads whose four token rows all lie past M are skipped: their accumulator rows are never stored
+      // loads whose four token rows all lie past M are skipped, and so is their staging: those rows of the tile keep
+      // whatever the LDS held, and the accumulator rows they feed are never stored
       if (q * 4 < g.M) ra.a[q] = *reinterpret_cast<const u32x4*>(g.x + (size_t)row * g.K + kbase + (seg & 1) * 128);
-      else ra.a[q] = u32x4{0u, 0u, 0u, 0u};
+      else ra.a[q] = __builtin_nondeterministic_value(ra.a[q]);  // no value carried round the loop: nothing to wait for
     }
   };
   auto stage_a = [&](const ARegs& ra) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous half are done
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int q = 0; q < kMT * 8; ++q)
-      *reinterpret_cast<u32x4*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = ra.a[q];
+    for (int q = 0; q < kMT * 8; ++q)  // staged in the order of the weight nibbles, so that fragment reads need no permute
+      if (q * 4 < g.M)
+        *reinterpret_cast<h8*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = nibble_order(ra.a[q]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -399,7 +406,7 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     for (int t = 0; t < 4; ++t) {
 #pragma unroll
       for (int tm = 0; tm < kMT; ++tm) {
-        const h8 af = nibble_order(*reinterpret_cast<const u32x4*>(atile + (((tm * 32 + ln) * 2 + lh) * kSegStride) + (4 * (j & 1) + t) * 16));
+        const h8 af = *reinterpret_cast<const h8*>(atile + (((tm * 32 + ln) * 2 + lh) * kSegStride) + (4 * (j & 1) + t) * 16);
 #pragma unroll
         for (int tn = 0; tn < kNT; ++tn) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf[tn][t], acc[tm][tn], 0, 0, 0);
       }
@@ -426,27 +433,29 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
 #undef GLOWQ_PIN_LOADS
   __syncthreads();  // the reduction buffer below overlays the staging tiles
 
-  // ---- the waves' partial tiles meet in LDS: [wave][tm][tn][16 regs][64 lanes] floats --------------------------
+  // ---- the waves' partial tiles meet in LDS: [wave][tm][tn][16 regs][64 lanes] floats; only registers and slots of
+  // token rows below M take part ----------------------------------------------------------------------------------
   float* red = reinterpret_cast<float*>(smem);
   constexpr int kTile = kMT * kNT * 16 * 64;
 #pragma unroll
   for (int tm = 0; tm < kMT; ++tm)
 #pragma unroll
-    for (int tn = 0; tn < kNT; ++tn)
+    for (int i = 0; i < 16; ++i)
+      if (tm * 32 + 8 * (i >> 2) < g.M) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) red[(size_t)wave * kTile + ((tm * kNT + tn) * 16 + i) * 64 + lane] = acc[tm][tn][i];
+        for (int tn = 0; tn < kNT; ++tn) red[(size_t)wave * kTile + ((tm * kNT + tn) * 16 + i) * 64 + lane] = acc[tm][tn][i];
+      }
   __syncthreads();
-  const int slots = kMT * kNT * 16 * 64;
+  const int slots = g.M * (32 * kNT);  // (token row, column of the workgroup's tile), column fastest
   for (int sidx = threadIdx.x; sidx < slots; sidx += blockDim.x) {
+    const int m = sidx / (32 * kNT), col = sidx - m * (32 * kNT);
+    const int tm = m >> 5, mm = m & 31, tn = col >> 5;
+    const int reg = ((mm >> 3) << 2) | (mm & 3);
+    const int at = ((tm * kNT + tn) * 16 + reg) * 64 + ((mm >> 2) & 1) * 32 + (col & 31);
     float v = 0.f;
-    for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + sidx];
-    const int l = sidx & 63;
-    const int i = (sidx >> 6) & 15;
-    const int tt = sidx >> 10;
-    const int tm = tt / kNT, tn = tt - tm * kNT;
-    const int n = n0 + tn * 32 + (l & 31);
-    const int m = tm * 32 + 8 * (i >> 2) + 4 * (l >> 5) + (i & 3);
-    if (m < g.M && n < mem.N) {
+    for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + at];
+    const int n = n0 + col;
+    if (n < mem.N) {
       const float b = mem.bias ? (float)mem.bias[n] : 0.f;
       mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
     }
