@@ -254,7 +254,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
 // order (8 lanes per segment, every line requested once per instruction) and reads the fragments back in MFMA lane
 // order.  Loading the fragments straight from memory (one 16-byte request per lane and line) cost 22 us of the 45 us
 // of a 28672 x 4096 layer at 32 rows: every request pulls a whole line out of L2.
-template <int kMT, int kNT>
+template <int kMT, int kNT, bool kBulk>
 __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63;
@@ -337,7 +337,42 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   const int per = (sblocks + waves - 1) / waves;
   const int first = wave * per;
   const int mine = max(0, min(per, sblocks - first));
-  uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point word of the super-block being computed
+  uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point of the super-block being computed
+
+  // With groups of 128 columns a lane's scales and zero-points of eight consecutive super-blocks are 32 and 8
+  // contiguous bytes of its weight row: they are fetched once per eight super-blocks (runs counted from the wave's
+  // first super-block; one that would pass the end of the row is moved back to end with it) and kept in registers,
+  // the lane's own half of every super-block picked out.  One scattered 2-byte and one 4-byte request per
+  // super-block otherwise cost as much address processing as the super-block's weights.
+  // The host picks this form (kBulk) where it applies; with five requests per run it is not worth it for waves with
+  // fewer than four super-blocks.
+  constexpr bool bulk = kBulk;
+  u32x4 run_s[kNT];     // own scale of super-block j of the run: half j % 2 of dword j / 2
+  uint64_t run_z[kNT];  // own zero-point of super-block j: byte j
+  int run_start = 0;    // first super-block of the run held
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) {
+    run_s[tn] = u32x4{0u, 0u, 0u, 0u};
+    run_z[tn] = 0;
+  }
+  auto fetch_run = [&](int start) {
+    run_start = start;
+    const int zword = start >> 2, zlast = (2 * sblocks - 1) >> 3;  // sixteen groups from group 2 start: two or three words
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      const uint32_t* srow = reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned short*>(mem.scales) + (size_t)ncol[tn] * mem.lds) + start;
+      const u32x4 s0 = *reinterpret_cast<const u32x4*>(srow), s1 = *reinterpret_cast<const u32x4*>(srow + 4);
+      const int32_t* zrow = mem.qzeros + (size_t)ncol[tn] * mem.ldz;
+      const uint32_t z0 = (uint32_t)zrow[zword], z1 = (uint32_t)zrow[min(zword + 1, zlast)], z2 = (uint32_t)zrow[min(zword + 2, zlast)];
+      const uint32_t sel = lh ? 0x07060302u : 0x05040100u;  // upper or lower half of both dwords
+      run_s[tn] = u32x4{__builtin_amdgcn_perm(s0.y, s0.x, sel), __builtin_amdgcn_perm(s0.w, s0.z, sel),
+                        __builtin_amdgcn_perm(s1.y, s1.x, sel), __builtin_amdgcn_perm(s1.w, s1.z, sel)};
+      const int sh = 4 * ((2 * start) & 7) + 4 * lh;  // nibble of group 2 start + lh
+      const uint64_t lo = ((uint64_t)z1 << 32) | z0;
+      const uint64_t a = sh ? (lo >> sh) | ((uint64_t)z2 << (64 - sh)) : lo;  // groups 2 start + lh + 0..15, a nibble each
+      run_z[tn] = a & 0x0F0F0F0F0F0F0F0Full;
+    }
+  };
   auto issue_b = [&](int i, BRegs& rb) {
     const int sb = min(first + i, sblocks - 1);  // past-the-end prefetches re-read the last one
     const int grp = (sb * 256 + lh * 128) >> g.gs_shift;
@@ -348,20 +383,37 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
         const int n = min(n0 + tn * 32 + q * 8 + (lane >> 3), mem.N - 1);
         rb.b[tn * 4 + q] = *reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw + sb * 32 + (lane & 7) * 4);
       }
-      rb.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
-      rb.z[tn] = (uint32_t)mem.qzeros[(size_t)ncol[tn] * mem.ldz + (grp >> 3)];
+      if (!bulk) {
+        rb.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
+        rb.z[tn] = (uint32_t)mem.qzeros[(size_t)ncol[tn] * mem.ldz + (grp >> 3)];
+      } else {
+        rb.s[tn] = __builtin_nondeterministic_value(rb.s[tn]);
+        rb.z[tn] = __builtin_nondeterministic_value(rb.z[tn]);
+      }
     }
   };
-  auto stage_b = [&](const BRegs& rb) {
+  auto stage_b = [&](const BRegs& rb, int i) {
+    if (bulk) {
+      const int start = min(first + (i & ~7), sblocks - 8);  // runs of eight from the wave's first super-block
+      if (start != run_start) fetch_run(start);
+    }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous super-block are done
     __builtin_amdgcn_wave_barrier();
+    const int j = first + i - run_start;
 #pragma unroll
     for (int tn = 0; tn < kNT; ++tn) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         *reinterpret_cast<u32x4*>(btile + (tn * 32 + q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = rb.b[tn * 4 + q];
-      cur_s[tn] = rb.s[tn];
-      cur_z[tn] = rb.z[tn];
+      if (bulk) {
+        const u32x4 rs = run_s[tn];
+        const uint32_t sp = (j & 4) ? ((j & 2) ? rs.w : rs.z) : ((j & 2) ? rs.y : rs.x);
+        cur_s[tn] = (j & 1) ? sp >> 16 : sp & 0xFFFFu;
+        cur_z[tn] = (uint32_t)(run_z[tn] >> (8 * j)) & 0xFu;
+      } else {
+        cur_s[tn] = rb.s[tn];
+        cur_z[tn] = nibble(rb.z[tn], (((first + i) * 256 + lh * 128) >> g.gs_shift) & 7);
+      }
     }
   };
   auto issue_a = [&](int i, int jj, ARegs& ra) {  // jj: first or second half of every lane's 128 columns
@@ -388,11 +440,10 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
   auto compute = [&](int i, int j) {
-    const int grp = ((first + i) * 256 + lh * 128) >> g.gs_shift;
     h8 bf[kNT][4];
 #pragma unroll
     for (int tn = 0; tn < kNT; ++tn) {
-      const half_t z = (half_t)(float)nibble(cur_z[tn], grp & 7);
+      const half_t z = (half_t)(float)cur_z[tn];
       const half_t zl = (half_t)(-1024.0f) - z, zh = (half_t)(-64.0f) - z;
       const h2 zb_lo = {zl, zl}, zb_hi = {zh, zh};
       const h2 s2 = bitcast_u32<h2>(cur_s[tn] | (cur_s[tn] << 16));
@@ -419,11 +470,12 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
 #define GLOWQ_PIN_LOADS() asm volatile("" ::: "memory")
   BRegs B;
   ARegs A;
+  if (bulk) fetch_run(min(first, sblocks - 8));
   issue_b(0, B);
   issue_a(0, 0, A);
   GLOWQ_PIN_LOADS();
   for (int i = 0; i < mine; ++i) {
-    stage_b(B); stage_a(A);
+    stage_b(B, i); stage_a(A);
     issue_a(i, 1, A); issue_b(i + 1, B); GLOWQ_PIN_LOADS();
     compute(i, 0); compute(i, 1);
     stage_a(A);
@@ -483,13 +535,25 @@ bool skinny_supported(const GroupDev& g) {
   return true;
 }
 
+// Scales and zero-points in runs of eight super-blocks: groups of 128 columns, rows of eight super-blocks or more, four
+// or more super-blocks per wave, and scale rows that start on a 4-byte boundary.
+static bool skinny_bulk_runs(const SkinnyArgs& a, int waves) {
+  const int sblocks = a.K >> 8;
+  if (a.gs_shift != 7 || sblocks < 8 || (sblocks + waves - 1) / waves < 4) return false;
+  for (int i = 0; i < a.n_members; ++i)
+    if ((a.mem[i].lds & 1) != 0 || (reinterpret_cast<uintptr_t>(a.mem[i].scales) & 3u) != 0) return false;
+  return true;
+}
+
 template <int kMT, int kNT, bool kGroupForm>
 static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) {
-  auto kern = kGroupForm ? skinny_group_kernel<kMT, kNT> : skinny_mfma_kernel<kMT, kNT>;
+  const bool bulk = kGroupForm && skinny_bulk_runs(a, waves);
+  auto kern = !kGroupForm ? skinny_mfma_kernel<kMT, kNT>
+              : bulk ? skinny_group_kernel<kMT, kNT, true> : skinny_group_kernel<kMT, kNT, false>;
   size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
   if (kGroupForm && lds < (size_t)waves * (kMT * 64 + kNT * 32) * 144) lds = (size_t)waves * (kMT * 64 + kNT * 32) * 144;
-  static LdsLimit lds_limit;
-  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
+  static LdsLimit lds_limit[2];  // one per kernel this site launches
+  if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit[bulk]); e != hipSuccess) return e;
   int total = 0;
   for (int i = 0; i < a.n_members; ++i) {
     total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);

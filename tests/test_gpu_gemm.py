@@ -77,7 +77,8 @@ def test_group_forward_large_m(ext, M, K, Ns, rank, alpha):
 
 # ---------------------------------------------------------------- skinny MFMA route (5 <= M <= 64)
 @pytest.mark.parametrize("M,K,N,gs", [(5, 512, 64, 128), (8, 4096, 1024, 128), (16, 1024, 300, 128), (32, 2048, 96, 64),
-                                      (33, 1024, 200, 128), (64, 14336, 128, 128), (64, 64, 32, 32), (7, 192, 40, 64)])
+                                      (33, 1024, 200, 128), (64, 14336, 128, 128), (64, 64, 32, 32), (7, 192, 40, 64),
+                                      (8, 2816, 200, 128), (24, 5632, 96, 128), (16, 18944, 64, 128), (40, 2304, 72, 128)])
 def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     print(f"case M={M} K={K} N={N} gs={gs}", flush=True)
     assert ext.lib.glowq_w4a16_route(M, K, N, gs, K // 8) == (4 if small_m_route == "quad" and M <= 16 else 1)
@@ -88,13 +89,16 @@ def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     assert_close(y.cpu().numpy(), x.astype(np.float64) @ w.T, f"skinny M={M} K={K} N={N}")
 
 
-def test_skinny_identity_block_is_exact(ext, small_m_route):
-    """64 rows of the identity select 64 weight columns: the in-register dequantisation and the activation
-    permutation of the skinny kernel, bit for bit."""
-    K, N, gs = 256, 96, 128
+@pytest.mark.parametrize("K,k0s", [(256, (0, 64, 192)), (2816, (0, 192, 832, 1728, 2048, 2560, 2752)),
+                                   (19456, (0, 2304, 4864, 9984, 19392))])
+def test_skinny_identity_block_is_exact(ext, small_m_route, K, k0s):
+    """64 rows of the identity select 64 weight columns: the in-register dequantisation, the activation permutation
+    and the choice of every super-block's scale and zero-point in the skinny kernel, bit for bit.  The longer rows have
+    scales and zero-points fetched in runs of eight super-blocks, with runs that start off a multiple of four."""
+    N, gs = 96, 128
     _, (m,), _ = make_group(23, 1, K, [N], 0, group_size=gs)
     want = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], K, gs)
-    for k0 in (0, 64, 192):
+    for k0 in k0s:
         x = np.zeros((64, K), dtype=np.float16)
         x[np.arange(64), k0 + np.arange(64)] = 1.0
         y = ext.w4a16_gemv_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs).cpu().numpy()
