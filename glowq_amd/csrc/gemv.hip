@@ -116,14 +116,17 @@ __device__ __forceinline__ void dot_word(uint32_t w, const h8& xq, float& accA, 
 // What a wave loads for one row block, all of it issued before anything is used: per row one
 // 16-byte unit of 32 int4 codes, the raw scale and zero-point word of the unit's quantisation group,
 // and kLW dwords (two halves each) of the row of the left factor L.
-// kWide: a step holds at most 16 quantisation groups per row (group_size >= 128); then lane 16r + i loads the
+// kSide 1: a step holds at most 16 quantisation groups per row (group_size >= 128); then lane 16r + i loads the
 // scale and zero-point of group i of row r once per step and the lanes that need it fetch it with ds_bpermute,
 // instead of every lane loading its own copy for every row.
-template <int kRows, int kLW, bool kWide>
+// kSide 2 (at most two rows per block, an even number of steps per row block): lane 32r + i loads group i of row r
+// of a PAIR of steps with the first step of the pair; the second step issues no scale or zero-point request at all.
+// The steps of a pair always sit in the same two prefetch buffers, so every step has a fixed number of loads.
+template <int kRows, int kLW, int kSide>
 struct Prefetch {
   u32x4 w[kRows];
-  half_t sc[kWide ? 1 : kRows];
-  uint32_t zw[kWide ? 1 : kRows];
+  half_t sc[kSide ? 1 : kRows];
+  uint32_t zw[kSide ? 1 : kRows];
   uint32_t l[kRows][kLW > 0 ? kLW : 1];
 };
 
@@ -137,7 +140,7 @@ struct Prefetch {
 // Every workgroup serves ONE member for its whole life (the host splits the grid between the members in
 // proportion to their row blocks), so the member's pointers and strides are loop invariants held in
 // scalar registers and nothing is looked up in memory between two prefetches.
-template <int kM, int kRows, int kLW, bool kWide>
+template <int kM, int kRows, int kLW, int kSide>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(((kM >= 2 || kRows >= 4) ? 4 : 6), 8)))
 void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t* __restrict__ head_x,
                           const half_t* __restrict__ head_r, const int head_ldw, const int head_rows,
@@ -146,6 +149,8 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
   // The head_* arguments repeat what a workgroup of the FIRST member needs to request the weights of its first step:
   // plain leading arguments reach the wave in scalar registers, everything inside `g` takes a load from the argument
   // buffer (a memory round trip).  Those workgroups -- all of them for a group of one -- start that much earlier.
+  constexpr bool kWide = kSide != 0, kPair = kSide == 2;
+  static_assert(!kPair || kRows <= 2, "a pair of steps of one row fills 32 lanes");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int U = g.K >> 5;                                  // 16-byte units per weight row
   const int upg_shift = __builtin_ctz(g.group_size >> 5);  // units per quantisation group = 1 << upg_shift
@@ -155,7 +160,7 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  Prefetch<kRows, kLW, kWide> buf0, buf1;
+  Prefetch<kRows, kLW, kSide> buf0, buf1;
   const bool head = (int)blockIdx.x < head_wg_end;
   if (head) {
     const int n0 = min((int)blockIdx.x * head_waves + wave, head_blocks - 1) * kRows;
@@ -196,9 +201,11 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
   struct Cursor {
     int blk, it;
   };
-  const int side_row = min(lane >> 4, kRows - 1), side_idx = lane & 15;
+  const int side_row = min(kPair ? lane >> 5 : lane >> 4, kRows - 1), side_idx = kPair ? lane & 31 : lane & 15;
   const int gps_shift = 6 - upg_shift;  // log2 of the groups per row and step
-  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kWide>& p, const bool weights_requested = false) {
+  // first group of the step (of the pair of steps) whose scales and zero-points the side lanes hold
+  auto side_base = [&](int it) { return kPair ? (it >> 1) << (gps_shift + 1) : it << gps_shift; };
+  auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kSide>& p, const bool weights_requested, const bool with_side) {
     const int n0 = min(c.blk, total_blocks - 1) * kRows;
     const int u = min(lane + c.it * kWave, U - 1);
     const int grp = u >> upg_shift;
@@ -220,10 +227,12 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
       }
     }
     if constexpr (kWide) {
-      const int n = min(n0 + side_row, mem.N - 1);
-      const int sg = min((c.it << gps_shift) + side_idx, (U - 1) >> upg_shift);
-      p.sc[0] = mem.scales[(size_t)n * mem.lds + sg];
-      p.zw[0] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (sg >> 3)];
+      if (!kPair || with_side) {  // a constant at every call site
+        const int n = min(n0 + side_row, mem.N - 1);
+        const int sg = min(side_base(c.it) + side_idx, (U - 1) >> upg_shift);
+        p.sc[0] = mem.scales[(size_t)n * mem.lds + sg];
+        p.zw[0] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (sg >> 3)];
+      }
     }
   };
   auto advance = [&](Cursor& c) {
@@ -239,19 +248,26 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
 #pragma unroll
     for (int m = 0; m < kM; ++m) tot[r][m] = 0.f;
 
-  auto compute = [&](const Cursor& c, const Prefetch<kRows, kLW, kWide>& p) {
+  uint32_t side_held = 0;  // kSide 2: scale and zero-point of this lane's group, packed, kept from the first step of a pair
+  auto compute = [&](const Cursor& c, const Prefetch<kRows, kLW, kSide>& p, const bool with_side) {
     const int uraw = lane + c.it * kWave;
     const bool active = uraw < U;
     const int u = active ? uraw : U - 1;
     const int grp = u >> upg_shift;
     float sc[kRows], zp[kRows];
     if constexpr (kWide) {
-      const int sg = min((c.it << gps_shift) + side_idx, (U - 1) >> upg_shift);
-      const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, p.sc[0]) | (nibble(p.zw[0], sg & 7) << 16);
-      const int grel = grp - (c.it << gps_shift);
+      const int sg = min(side_base(c.it) + side_idx, (U - 1) >> upg_shift);
+      uint32_t packed;
+      if (!kPair || with_side) {
+        packed = (uint32_t)__builtin_bit_cast(uint16_t, p.sc[0]) | (nibble(p.zw[0], sg & 7) << 16);
+        side_held = packed;
+      } else {
+        packed = side_held;
+      }
+      const int grel = grp - side_base(c.it);
 #pragma unroll
       for (int r = 0; r < kRows; ++r) {
-        const uint32_t sv = (uint32_t)__builtin_amdgcn_ds_bpermute((16 * r + grel) << 2, (int)packed);
+        const uint32_t sv = (uint32_t)__builtin_amdgcn_ds_bpermute(((kPair ? 32 : 16) * r + grel) << 2, (int)packed);
         sc[r] = active ? (float)__builtin_bit_cast(half_t, (uint16_t)(sv & 0xFFFFu)) : 0.f;
         zp[r] = (float)(sv >> 16);
       }
@@ -319,7 +335,7 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
   Cursor ahead;
   ahead.blk = ((int)blockIdx.x - wg_begin) * waves_per_block + wave;
   ahead.it = 0;
-  issue(ahead, buf0, head);
+  issue(ahead, buf0, head, true);
 
   if (kM == 1 && early_x) store_activations(head_r, head_units << 5, head_rank, head_waves * kWave, U, xr, xs, sig, rs);
   else stage_activations<kM>(g, U, xs, sig, rs);
@@ -328,13 +344,13 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
   while (ahead.blk < total_blocks) {
     Cursor cur = ahead;
     advance(ahead);
-    issue(ahead, buf1);
-    compute(cur, buf0);
+    issue(ahead, buf1, false, false);
+    compute(cur, buf0, true);
     if (ahead.blk >= total_blocks) break;
     cur = ahead;
     advance(ahead);
-    issue(ahead, buf0);
-    compute(cur, buf1);
+    issue(ahead, buf0, false, true);
+    compute(cur, buf1, false);
   }
 }
 
@@ -405,10 +421,10 @@ static const WaveDotTuning& tuning_override() {
   return t;
 }
 
-template <int kM, int kRows, int kLW, bool kWide>
+template <int kM, int kRows, int kLW, int kSide>
 static hipError_t launch_wave_dot_t(const GroupDev& g, int kit, int waves, int max_wg_per_cu, int num_cus, size_t lds,
                                     hipStream_t stream) {
-  auto kern = gemv_wave_dot_kernel<kM, kRows, kLW, kWide>;
+  auto kern = gemv_wave_dot_kernel<kM, kRows, kLW, kSide>;
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   // resident workgroups per CU for a block size and LDS footprint; each host thread remembers its last answers
@@ -525,10 +541,14 @@ hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStre
   const int max_wg = tuning_override().max_wg_per_cu;
   // the shared scale / zero-point loads pay for single-row decode; the multi-row instantiations keep per-lane loads
   const bool wide = g.M == 1 && g.group_size >= 128;
-#define GLOWQ_CASE(MM, RR, LL)                                                                   \
-  if (g.M == MM && rows_per_block == RR && lw == LL)                                             \
-    return (MM == 1 && wide) ? launch_wave_dot_t<MM, RR, LL, (MM == 1)>(g, kit, waves, max_wg, num_cus, lds, stream) \
-                             : launch_wave_dot_t<MM, RR, LL, false>(g, kit, waves, max_wg, num_cus, lds, stream);
+  static const int env_pair = env_int("GLOWQ_GEMV_PAIR", 1);
+  const bool pair = wide && rows_per_block <= 2 && (kit & 1) == 0 && env_pair != 0;
+#define GLOWQ_CASE(MM, RR, LL)                                                                                   \
+  if (g.M == MM && rows_per_block == RR && lw == LL) {                                                           \
+    if (MM == 1 && pair) return launch_wave_dot_t<MM, RR, LL, (MM == 1 && RR <= 2) ? 2 : 0>(g, kit, waves, max_wg, num_cus, lds, stream); \
+    if (MM == 1 && wide) return launch_wave_dot_t<MM, RR, LL, (MM == 1) ? 1 : 0>(g, kit, waves, max_wg, num_cus, lds, stream);           \
+    return launch_wave_dot_t<MM, RR, LL, 0>(g, kit, waves, max_wg, num_cus, lds, stream);                         \
+  }
 #define GLOWQ_CASES(MM, RR) GLOWQ_CASE(MM, RR, 0) GLOWQ_CASE(MM, RR, 1) GLOWQ_CASE(MM, RR, 2)
   GLOWQ_CASES(1, 1) GLOWQ_CASES(1, 2) GLOWQ_CASES(1, 4)
   GLOWQ_CASES(2, 1) GLOWQ_CASES(2, 2)

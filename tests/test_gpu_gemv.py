@@ -20,6 +20,7 @@ def _run_single(ext, x, m, gs=128, entry="gemv"):
 @pytest.mark.parametrize("M,K,N,gs", [
     (1, 2048, 2048, 128), (1, 4096, 1024, 128), (2, 4096, 512, 128), (3, 1024, 300, 128), (4, 5120, 256, 128),
     (1, 14336, 128, 128), (1, 3584, 130, 128), (1, 4096, 4096, 128), (1, 256, 7, 64), (1, 512, 33, 32),
+    (1, 8192, 96, 256), (1, 6144, 70, 128), (1, 16384, 40, 512), (1, 12288, 37, 128),
 ])
 def test_gemv_matches_oracle(ext, small_m_route, M, K, N, gs):
     print(f"case M={M} K={K} N={N} gs={gs}", flush=True)
