@@ -204,6 +204,7 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
   const int side_row = min(kPair ? lane >> 5 : lane >> 4, kRows - 1), side_idx = kPair ? lane & 31 : lane & 15;
   const int gps_shift = 6 - upg_shift;  // log2 of the groups per row and step
   // first group of the step (of the pair of steps) whose scales and zero-points the side lanes hold
+  auto l_step = [&](int it) { return kPair ? it >> 1 : it; };
   auto side_base = [&](int it) { return kPair ? (it >> 1) << (gps_shift + 1) : it << gps_shift; };
   auto issue = [&](const Cursor& c, Prefetch<kRows, kLW, kSide>& p, const bool weights_requested, const bool with_side) {
     const int n0 = min(c.blk, total_blocks - 1) * kRows;
@@ -219,11 +220,13 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
         p.zw[r] = (uint32_t)mem.qzeros[(size_t)n * mem.ldz + (grp >> 3)];
       }
       if constexpr (kLW > 0) {
-        // a member without L reads r itself (valid memory) and is weighted by zero
-        const uint32_t* lrow = mem.L ? reinterpret_cast<const uint32_t*>(mem.L + (size_t)n * g.rank)
-                                     : reinterpret_cast<const uint32_t*>(g.r);
+        if (!kPair || with_side) {  // kSide 2: the L row is spread over the first steps of the pairs only
+          // a member without L reads r itself (valid memory) and is weighted by zero
+          const uint32_t* lrow = mem.L ? reinterpret_cast<const uint32_t*>(mem.L + (size_t)n * g.rank)
+                                       : reinterpret_cast<const uint32_t*>(g.r);
 #pragma unroll
-        for (int j = 0; j < kLW; ++j) p.l[r][j] = lrow[min((c.it * kLW + j) * kWave + lane, ldw_half - 1)];
+          for (int j = 0; j < kLW; ++j) p.l[r][j] = lrow[min((l_step(c.it) * kLW + j) * kWave + lane, ldw_half - 1)];
+        }
       }
     }
     if constexpr (kWide) {
@@ -296,10 +299,10 @@ void gemv_wave_dot_kernel(const int32_t* __restrict__ head_qweight, const half_t
         tot[r][m] = __builtin_fmaf(sc[r], v, tot[r][m]);
       }
     }
-    if constexpr (kLW > 0) {
+    if (kLW > 0 && (!kPair || with_side)) {
 #pragma unroll
       for (int j = 0; j < kLW; ++j) {
-        const int idx = (c.it * kLW + j) * kWave + lane;
+        const int idx = (l_step(c.it) * kLW + j) * kWave + lane;
         const float a = idx < ldw_half ? alpha_scaled : 0.f;
         const int ic = min(idx, ldw_half - 1);
 #pragma unroll
@@ -534,7 +537,7 @@ hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStre
   }
   const int kit = (g.K / 32 + kWave - 1) / kWave;
   const bool has_r = g.r != nullptr;
-  const int lw = has_r ? (g.rank + 128 * kit - 1) / (128 * kit) : 0;
+  int lw = has_r ? (g.rank + 128 * kit - 1) / (128 * kit) : 0;
   const size_t lds = wave_dot_lds_bytes(g.M, g.K, g.rank, has_r);
   int waves = tuning_override().waves;
   if (waves < 1 || waves > 16) waves = 8;
@@ -542,7 +545,10 @@ hipError_t launch_wave_dot(GroupDev& g, int rows_per_block, int num_cus, hipStre
   // the shared scale / zero-point loads pay for single-row decode; the multi-row instantiations keep per-lane loads
   const bool wide = g.M == 1 && g.group_size >= 128;
   static const int env_pair = env_int("GLOWQ_GEMV_PAIR", 1);
-  const bool pair = wide && rows_per_block <= 2 && (kit & 1) == 0 && env_pair != 0;
+  // in pairs the L row rides on every other step: twice the dwords per lane there
+  const int lw_pair = has_r ? (g.rank + 64 * kit - 1) / (64 * kit) : 0;
+  const bool pair = wide && rows_per_block <= 2 && (kit & 1) == 0 && lw_pair <= 2 && env_pair != 0;
+  if (pair) lw = lw_pair;
 #define GLOWQ_CASE(MM, RR, LL)                                                                                   \
   if (g.M == MM && rows_per_block == RR && lw == LL) {                                                           \
     if (MM == 1 && pair) return launch_wave_dot_t<MM, RR, LL, (MM == 1 && RR <= 2) ? 2 : 0>(g, kit, waves, max_wg, num_cus, lds, stream); \
