@@ -218,16 +218,37 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
     // its [BM][64] shape with octets 0-3 = half 0 and octets 4-7 = half 1, so the fragment reads do not change.
     constexpr int kSeg = 144;  // bytes per row segment in the weight tile: 128 + 16, conflict-free fragment reads
     unsigned char* btile = smem + (size_t)2 * BM * kARow * sizeof(half_t) + (size_t)wave * (32 * kNT) * kSeg;
+    // Every load of the loop is a buffer load: a uniform descriptor and a uniform byte offset that advances per step
+    // (scalar registers) plus a 32-bit byte offset that a lane computes once.  With 64-bit addresses per lane and load
+    // the address pairs alone spill the register file of the large tiles, and every reload of a spilled pair waits
+    // for all loads in flight.  (The host keeps tensors whose byte extent does not fit 32 bits off this route.)
+    const auto rsrc = [](const void* p, size_t bytes) {
+      return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(uint32_t)bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t rs_x = rsrc(a.x, (size_t)a.M * a.K * 2);
+    const __amdgpu_buffer_rsrc_t rs_w = rsrc(a.qweight, ((size_t)(a.N - 1) * a.ldw + (a.K >> 3)) * 4);
+    const __amdgpu_buffer_rsrc_t rs_s = rsrc(a.scales, ((size_t)(a.N - 1) * a.lds + (a.K >> gs_shift)) * 2);
+    const __amdgpu_buffer_rsrc_t rs_z = rsrc(a.qzeros, ((size_t)(a.N - 1) * a.ldz + (((a.K >> gs_shift) + 7) >> 3)) * 4);
+    uint32_t a_off[kMT], b_off[kNT * 4], s_off[kNT], z_off[kNT];
+#pragma unroll
+    for (int i = 0; i < kMT; ++i) {
+      const int q = tid + 256 * i;
+      const int oct = q & 7;
+      a_off[i] = ((uint32_t)min(m0 + (q >> 3), a.M - 1) * (uint32_t)a.K + (oct >> 2) * 128 + (oct & 3) * 8) * 2u;
+    }
+#pragma unroll
+    for (int q = 0; q < kNT * 4; ++q)
+      b_off[q] = ((uint32_t)min(bn * BN + wave * (32 * kNT) + q * 8 + (lane >> 3), a.N - 1) * (uint32_t)a.ldw + (lane & 7) * 4) * 4u;
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      s_off[tn] = (uint32_t)ncol[tn] * (uint32_t)a.lds * 2u;
+      z_off[tn] = (uint32_t)ncol[tn] * (uint32_t)a.ldz * 4u;
+    }
     auto load_a_sub = [&](ARegs& dst, int ks) {
       const int kc = min(ks, steps - 1);
-      const int kbase = (kc >> 2) * 256 + (kc & 3) * 32;
+      const int step_off = ((kc >> 2) * 256 + (kc & 3) * 32) * 2;
 #pragma unroll
-      for (int i = 0; i < kMT; ++i) {
-        const int q = tid + 256 * i;
-        const int row = min(m0 + (q >> 3), a.M - 1);
-        const int oct = q & 7;
-        dst.v[i] = *reinterpret_cast<const u32x4*>(a.x + (size_t)row * a.K + kbase + (oct >> 2) * 128 + (oct & 3) * 8);
-      }
+      for (int i = 0; i < kMT; ++i) dst.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, (int)a_off[i], step_off, 0);
     };
     struct BLoad {
       u32x4 w[kNT * 4];  // a super-block of the wave's 32 kNT weight rows in load order: row 8 q + lane / 8, piece lane % 8
@@ -236,16 +257,13 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
     uint32_t cur_s[kNT], cur_z[kNT];
     auto issue_b = [&](int sb, BLoad& bl) {
       const int sbc = min(sb, (steps >> 2) - 1);
-      const int grp = (sbc * 256 + lh * 128) >> gs_shift;
+      const uint32_t grp = (uint32_t)((sbc * 256 + lh * 128) >> gs_shift);
 #pragma unroll
-      for (int q = 0; q < kNT * 4; ++q) {
-        const int n = min(bn * BN + wave * (32 * kNT) + q * 8 + (lane >> 3), a.N - 1);
-        bl.w[q] = *reinterpret_cast<const u32x4*>(a.qweight + (size_t)n * a.ldw + sbc * 32 + (lane & 7) * 4);
-      }
+      for (int q = 0; q < kNT * 4; ++q) bl.w[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)b_off[q], sbc * 128, 0);
 #pragma unroll
       for (int tn = 0; tn < kNT; ++tn) {
-        bl.s[tn] = reinterpret_cast<const unsigned short*>(a.scales)[(size_t)ncol[tn] * a.lds + grp];
-        bl.z[tn] = (uint32_t)a.qzeros[(size_t)ncol[tn] * a.ldz + (grp >> 3)];
+        bl.s[tn] = (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rs_s, (int)(s_off[tn] + grp * 2u), 0, 0);
+        bl.z[tn] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs_z, (int)(z_off[tn] + (grp >> 3) * 4u), 0, 0);
       }
     };
     auto stage_b = [&](const BLoad& bl) {
@@ -545,7 +563,13 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stre
   if (force_mt > 0 && force_mt <= mt_cap) mt = force_mt;
   if (force_nt > 0 && force_nt <= nt_cap) nt = force_nt;
   static const int env_super = getenv("GLOWQ_GEMM_SUPER") ? atoi(getenv("GLOWQ_GEMM_SUPER")) : 1;
-  const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128;
+  // the super-block form addresses its operands with 32-bit byte offsets
+  bool fits32 = (size_t)M * gg.m[0].K * 2 < (1ull << 32);
+  for (int i = 0; i < gg.n; ++i) {
+    const size_t rows = (size_t)gg.m[i].N;
+    fits32 = fits32 && rows * gg.m[i].ldw * 4 < (1ull << 32) && rows * gg.m[i].lds * 2 < (1ull << 32) && rows * gg.m[i].ldz * 4 < (1ull << 32);
+  }
+  const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128 && fits32;
   // Split K through the workspace: where even the largest tile the rows allow leaves CUs idle, that tile is kept and K
   // is cut into slices of at least sixteen super-blocks until the workgroups number about two per CU.
   static const int env_split = getenv("GLOWQ_GEMM_SPLIT") ? atoi(getenv("GLOWQ_GEMM_SPLIT")) : 1;
