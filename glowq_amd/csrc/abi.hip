@@ -86,6 +86,19 @@ std::atomic<int> g_quad_max_m{clampi(env_or("GLOWQ_QUAD_M", 4), 0, 16)};
 std::atomic<int> g_quad_min_m{clampi(env_or("GLOWQ_QUAD_MIN_M", 2), 1, 16)};
 //   skinny_max_m    rows up to which the skinny MFMA kernel is preferred over the tiled GEMM (GLOWQ_SKINNY_M)
 std::atomic<int> g_skinny_max_m{clampi(env_or("GLOWQ_SKINNY_M", 64), 0, 64)};
+//   small_group_mb  3..4 rows: groups whose int4 weights are smaller than this many MB go to the skinny MFMA kernel (or
+//                   stay on the wave-dot GEMV), which start up faster than the 4x4x4 GEMV; at two rows they stay on the
+//                   wave-dot GEMV and the limit is 40/17 of it (GLOWQ_SMALL_GROUP_MB; default 17; 0 switches the rule off).  8B-shape layers at two rows: q|k|v 8.9 -> 7.8 us, o_proj 7.2 -> 5.6,
+//                   down_proj (29 MB) 13.1 -> 11.2, while gate|up (59 MB) is 1.6 us faster on the 4x4x4 kernel
+std::atomic<int> g_small_group_mb{clampi(env_or("GLOWQ_SMALL_GROUP_MB", 17), 0, 4096)};
+bool small_group_prefers_wave_dot(const GroupDev& g) {
+  if (g.M < 2 || g.M > 4) return false;
+  const size_t mb = (size_t)g_small_group_mb.load(std::memory_order_relaxed);
+  const size_t limit = (g.M == 2 ? mb * 40 / 17 : mb) << 20;
+  size_t bytes = 0;
+  for (int i = 0; i < g.n_members; ++i) bytes += (size_t)g.mem[i].N * (size_t)(g.K >> 1);
+  return bytes < limit;
+}
 int wave_dot_pref_m() { return g_wave_dot_max_m.load(std::memory_order_relaxed); }
 bool quad_wanted(int M) {
   return M >= g_quad_min_m.load(std::memory_order_relaxed) && M <= g_quad_max_m.load(std::memory_order_relaxed);
@@ -152,6 +165,13 @@ int pick_route(const GroupDev& g, int force) {
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
   const bool quad_rows = quad_wanted(g.M) ||
                          (g.M > 1 && g.M <= 16 && g_quad_max_m.load(std::memory_order_relaxed) > 0 && !(skinny_supported(g) && skinny_group_form(g)));
+  if (force < 0 && small_group_prefers_wave_dot(g)) {
+    // two rows: the wave-dot GEMV; three and four: the skinny MFMA kernel where its super-block form applies
+    // (8B-shape q|k|v at four rows: 10.5 us on the 4x4x4 GEMV, 10.0 on the wave-dot GEMV, 8.0 on the skinny kernel)
+    if (g.M > 2 && skinny_supported(g) && skinny_group_form(g)) return kRouteSkinny;
+    if (g.M <= wave_dot_pref_m() && wave_dot_supported(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr))
+      return kRouteWaveDot;
+  }
   if (quad_rows && force != kRouteSkinny && quad_capacity(g.M, g.K, g.rank, g.r != nullptr || g.R != nullptr) > 0) {
     bool ok = true;
     for (int i = 0; i < g.n_members; ++i)  // 16-byte L rows; 32-bit byte offsets inside every buffer of a member
@@ -426,6 +446,7 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "quad_max_m") == 0) { slot = &g_quad_max_m; }
   else if (strcmp(key, "quad_min_m") == 0) { slot = &g_quad_min_m; lo = 1; }
   else if (strcmp(key, "skinny_max_m") == 0) { slot = &g_skinny_max_m; hi = 64; }
+  else if (strcmp(key, "small_group_mb") == 0) { slot = &g_small_group_mb; hi = 4096; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

@@ -413,8 +413,8 @@ class W4A16Extension:
         return names[self.lib.glowq_w4a16_route(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
 
     def set_tuning(self, key: str, value: int) -> int:
-        """Sets a route limit of the process ("quad_max_m", "quad_min_m", "wave_dot_max_m", "skinny_max_m"); returns the
-        old value."""
+        """Sets a route limit of the process ("quad_max_m", "quad_min_m", "wave_dot_max_m", "skinny_max_m",
+        "small_group_mb"); returns the old value."""
         old = self.lib.glowq_set_tuning(key.encode(), int(value))
         if old < 0:
             raise ValueError(self.lib.glowq_last_error().decode())

@@ -158,8 +158,11 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * knobs, src/cuda_w4a16/linear.py:21-27,122): "quad_max_m" / "quad_min_m" bound the token rows served by the
  * 4x4x4 matrix-core GEMV (0 for quad_max_m switches it off), "wave_dot_max_m" those of the wave-dot GEMV,
  * "skinny_max_m" (at most 64) those of the skinny MFMA kernel, above which the tiled GEMM takes over.
+ * "small_group_mb": at 3..4 token rows a group whose int4 weights are smaller than this many MB goes to the
+ * skinny MFMA kernel (or stays on the wave-dot GEMV) instead of the 4x4x4 GEMV, which starts up more slowly; at 2
+ * rows it stays on the wave-dot GEMV and the limit is 40/17 of it; 0 = never.
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
- * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M and GLOWQ_SKINNY_M.
+ * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M and GLOWQ_SMALL_GROUP_MB.
  */
 int glowq_set_tuning(const char* key, int value);
 

@@ -33,6 +33,8 @@ def small_m_route(request, ext):
     off (wave-dot GEMV for 1..4 rows, skinny MFMA kernel above)."""
     old = ext.set_tuning("quad_max_m", 16 if request.param == "quad" else 0)
     old_min = ext.set_tuning("quad_min_m", 1)
+    old_small = ext.set_tuning("small_group_mb", 0)  # no shape-dependent choice between the two at 2..4 rows
     yield request.param
     ext.set_tuning("quad_max_m", old)
     ext.set_tuning("quad_min_m", old_min)
+    ext.set_tuning("small_group_mb", old_small)

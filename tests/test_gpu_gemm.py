@@ -89,6 +89,23 @@ def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     assert_close(y.cpu().numpy(), x.astype(np.float64) @ w.T, f"skinny M={M} K={K} N={N}")
 
 
+@pytest.mark.parametrize("M,K,Ns,rank", [(3, 4096, [512, 128, 128], 128), (4, 2048, [300], 64), (4, 5632, [96, 40], 128), (2, 4096, [256], 128)])
+def test_small_groups_at_two_to_four_rows(ext, M, K, Ns, rank):
+    """Default route limits: a small group at three or four rows runs on the skinny MFMA kernel, at two rows on the
+    wave-dot GEMV; both against the oracle, with the shared correction."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    assert ext.lib.glowq_w4a16_route(M, K, sum(Ns), 128, K // 8) == (0 if M == 2 else 1)
+    x, members, R = make_group(311 + M + K, M, K, Ns, rank, with_bias=True)
+    r = torch.empty(M, rank, dtype=torch.float16, device="cuda")
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]), "L": dev(m["L"]),
+            "bias": dev(m["bias"])} for m in members]
+    outs = ext.group_forward(dev(x), r, mem, 128, 1.0, R=dev(R))
+    torch.cuda.synchronize()
+    for i, (m, y) in enumerate(zip(members, outs)):
+        want = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0)
+        assert_close(y.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"small group member {i} at M={M}")
+
+
 @pytest.mark.parametrize("K,k0s", [(256, (0, 64, 192)), (2816, (0, 192, 832, 1728, 2048, 2560, 2752)),
                                    (19456, (0, 2304, 4864, 9984, 19392))])
 def test_skinny_identity_block_is_exact(ext, small_m_route, K, k0s):
