@@ -56,6 +56,57 @@ template <int kM>
 __device__ __forceinline__ void stage_quad(const GroupDev& g, const QuadLds& l, h8* xs, float* sig, half_t* rs) {
   const int words = g.K >> 3;
   const int U = g.K >> 5;
+  if constexpr (kM <= 4) {
+    // Up to four token rows: every request of the staging goes out before anything is used -- one memory round trip
+    // instead of two per token row (x, then r), which is most of what a short launch costs.
+    constexpr int kMaxW = 4;                 // 16-byte words of a token row per thread
+    constexpr int kTok4 = (kM + 3) & ~3;
+    const int rd = g.rank >> 1;              // dwords of a row of r
+    if (words <= kMaxW * (int)blockDim.x && (g.r == nullptr || rd <= (int)blockDim.x)) {
+      h8 v[kM][kMaxW];
+      uint32_t rv[kTok4];
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+        const h8* xrow = reinterpret_cast<const h8*>(g.x + (size_t)min(m, g.M - 1) * g.K);
+#pragma unroll
+        for (int c = 0; c < kMaxW; ++c) {
+          const int w = (int)threadIdx.x + c * (int)blockDim.x;
+          if (w < words) v[m][c] = xrow[w];
+          else v[m][c] = __builtin_nondeterministic_value(v[m][c]);  // never used
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < kTok4; ++m)
+        rv[m] = (g.r != nullptr && (int)threadIdx.x < rd)
+                    ? reinterpret_cast<const uint32_t*>(g.r + (size_t)min(m, g.M - 1) * g.rank)[threadIdx.x] : 0u;
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+#pragma unroll
+        for (int c = 0; c < kMaxW; ++c) {
+          const int w = (int)threadIdx.x + c * (int)blockDim.x;
+          if (w < words) {  // the four words of a unit sit in one quad of threads: whole quads take this branch
+            const h8 q = v[m][c];
+            h8 p;
+            p[0] = q[0]; p[1] = q[4]; p[2] = q[2]; p[3] = q[6];
+            p[4] = q[1]; p[5] = q[5]; p[6] = q[3]; p[7] = q[7];
+            const int u = w >> 2, t = w & 3;
+            xs[(size_t)m * l.x_stride + t * U + u] = p;
+            float sum = ((float)q[0] + (float)q[1]) + ((float)q[2] + (float)q[3]) +
+                        (((float)q[4] + (float)q[5]) + ((float)q[6] + (float)q[7]));
+            sum = quad_sum(sum);
+            if (t == 0) sig[u * l.tok4 + m] = sum * 0x1p-24f;
+          }
+        }
+      }
+      for (int m = kM; m < kTok4; ++m)
+        for (int u = threadIdx.x; u < U; u += blockDim.x) sig[u * l.tok4 + m] = 0.f;
+      if (g.r != nullptr && (int)threadIdx.x < rd) {
+#pragma unroll
+        for (int m = 0; m < kTok4; ++m) reinterpret_cast<uint32_t*>(rs + m * l.r_stride)[threadIdx.x] = rv[m];
+      }
+      return;
+    }
+  }
 #pragma unroll 1
   for (int m = 0; m < l.tok4; ++m) {
     const int src = min(m, g.M - 1);
