@@ -35,6 +35,46 @@ __host__ __device__ inline size_t wave_dot_lds_total(int M, int K, int rank) {
 template <int kM>
 __device__ __forceinline__ void stage_activations(const GroupDev& g, int U, h8* xs, float* sig, half_t* rs) {
   const int words = g.K >> 3;  // 8 halves each
+  constexpr int kMaxW = 4;     // words of a token row per thread on the short path
+  const int rd = g.rank >> 1;
+  if (words <= kMaxW * (int)blockDim.x &&
+      (g.r == nullptr || ((g.rank & 1) == 0 && rd <= (int)blockDim.x && (reinterpret_cast<uintptr_t>(g.r) & 3u) == 0))) {
+    // every request of the staging goes out before anything is used: one memory round trip, not two per token row
+    h8 v[kM][kMaxW];
+    uint32_t rv[kM];
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+      const h8* xrow = reinterpret_cast<const h8*>(g.x + (size_t)m * g.K);
+#pragma unroll
+      for (int c = 0; c < kMaxW; ++c) {
+        const int w = (int)threadIdx.x + c * (int)blockDim.x;
+        if (w < words) v[m][c] = xrow[w];
+        else v[m][c] = __builtin_nondeterministic_value(v[m][c]);  // never used
+      }
+      rv[m] = (g.r != nullptr && (int)threadIdx.x < rd) ? reinterpret_cast<const uint32_t*>(g.r + (size_t)m * g.rank)[threadIdx.x] : 0u;
+    }
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+#pragma unroll
+      for (int c = 0; c < kMaxW; ++c) {
+        const int w = (int)threadIdx.x + c * (int)blockDim.x;
+        if (w < words) {  // words is a multiple of 4: whole quads of threads take this branch
+          const h8 q = v[m][c];
+          h8 p;
+          p[0] = q[0]; p[1] = q[4]; p[2] = q[1]; p[3] = q[5];
+          p[4] = q[2]; p[5] = q[6]; p[6] = q[3]; p[7] = q[7];
+          const int u = w >> 2, j = w & 3;
+          xs[((size_t)m * 4 + j) * U + u] = p;
+          float sum = ((float)q[0] + (float)q[1]) + ((float)q[2] + (float)q[3]) +
+                      (((float)q[4] + (float)q[5]) + ((float)q[6] + (float)q[7]));
+          sum = quad_sum(sum);
+          if (j == 0) sig[m * U + u] = sum * 0x1p-24f;
+        }
+      }
+      if (g.r != nullptr && (int)threadIdx.x < rd) reinterpret_cast<uint32_t*>(rs + m * g.rank)[threadIdx.x] = rv[m];
+    }
+    return;
+  }
   for (int m = 0; m < kM; ++m) {
     const h8* xrow = reinterpret_cast<const h8*>(g.x + (size_t)m * g.K);
     for (int w = threadIdx.x; w < words; w += blockDim.x) {
