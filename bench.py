@@ -59,7 +59,7 @@ SELECTIVE_GROUPS = {
     "down_proj": (17408, [5120]),
 }
 DOMINANT = "gate_up"
-DOMINANT_TRAFFIC_BYTES = 68708000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
+DOMINANT_TRAFFIC_BYTES = 68884000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
 
 
 def algorithmic_bytes(M, K, N, rank, gs=GROUP_SIZE):
