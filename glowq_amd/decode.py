@@ -339,9 +339,14 @@ class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
     def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True,
-                 attention_splits: int = 4):
+                 attention_splits: int = 0):
         self.model = model
         cfg = model.cfg
+        if attention_splits <= 0:
+            # workgroups per head in the fused step's attention: 4 up to 2048 positions of cache, 8 beyond
+            # (measured at 32 heads: 2.34 -> 2.28 ms per token at 3.6k tokens of context, 2.73 -> 2.57 at 7.7k;
+            # 16 is slower than either, and at 0.5k to 0.8k tokens 4 beats 8)
+            attention_splits = 4 if cfg.max_len <= 2048 else 8
         dev = model.lm_head.weight.device
         self.dev = dev
         self.caches = [(torch.zeros(cfg.kv_heads, cfg.max_len, cfg.head_dim, dtype=torch.float16, device=dev),
@@ -425,7 +430,7 @@ class GreedyDecoder:
 
 
 def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
-            fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 4) -> dict:
+            fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0) -> dict:
     """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
     second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798)."""
     import os
@@ -459,7 +464,8 @@ def main():
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
     ap.add_argument("--vocab", type=int, default=128256)
-    ap.add_argument("--attention-splits", type=int, default=4, help="workgroups per head in the fused step's attention")
+    ap.add_argument("--attention-splits", type=int, default=0,
+                    help="workgroups per head in the fused step's attention (0: by the cache length)")
     args = ap.parse_args()
     print(json.dumps(measure(args.layers, args.prompt, args.new, vocab=args.vocab, graph=not args.no_graph,
                              fused=not args.module_path, share=not args.no_sharing, correction=not args.no_correction,
