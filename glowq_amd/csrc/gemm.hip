@@ -584,7 +584,10 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stre
     // every slice writes the whole output once more in fp32, the reduction reads it back, and a short K loop is mostly
     // ramp: only slices of 16 super-blocks and more pay (measured: 2048 x 3584 outputs gain 8 % at K = 18944 in two
     // slices and lose 12 % at K = 3584; 128..512 rows of K = 4096 lose up to 40 % in slices of four super-blocks)
-    constexpr long min_depth = 16;
+    // ... unless the output has so few tiles that most of the chip would otherwise sit idle for the whole of a long K
+    // (4096 outputs of K = 14336 at 65..256 rows: 16 to 32 tiles, 97 -> 75..80 us with slices of four to eight)
+    static const int env_depth = getenv("GLOWQ_GEMM_MIN_DEPTH") ? atoi(getenv("GLOWQ_GEMM_MIN_DEPTH")) : 0;
+    const long min_depth = env_depth > 0 ? env_depth : (tiles >= 64 ? 16 : (tiles >= 32 ? 8 : 4));
     if (want > sb_total / min_depth) want = sb_total / min_depth;
     if (want > ws_slices_fit) want = ws_slices_fit;
     if (tiles < num_cus && want >= 2 && tiles * want * 2 >= num_cus) {
