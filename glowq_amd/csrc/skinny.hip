@@ -36,6 +36,10 @@ struct SkinnyArgs {
   int n_members;
   int M, K, rank, gs_shift;
   float alpha;
+  // second form only: gridDim.y slices of whole super-blocks; with more than one, every workgroup leaves its fp32
+  // tile in `partials` ([slice][workgroup][M][32 kNT]) and skinny_reduce_kernel adds the slices in order
+  int slices;
+  float* partials;
 };
 
 __device__ __forceinline__ h8 nibble_order(const u32x4& v) {
@@ -291,7 +295,7 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
 
   // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
-  const bool corrected = mem.L != nullptr && g.r != nullptr;
+  const bool corrected = mem.L != nullptr && g.r != nullptr && blockIdx.y == 0;  // the first slice carries the correction
   if (corrected) {
     const int lblocks = g.rank >> 6;
     for (int jb = wave; jb < lblocks; jb += waves) {
@@ -334,9 +338,12 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   unsigned char* atile = smem + (size_t)wave * (kATile + kBTile);
   unsigned char* btile = atile + kATile;
   const int sblocks = g.K >> 8;
-  const int per = (sblocks + waves - 1) / waves;
-  const int first = wave * per;
-  const int mine = max(0, min(per, sblocks - first));
+  // this workgroup's super-blocks: all of them, or slice blockIdx.y of g.slices; its waves split that range
+  const int sb_slice = (sblocks + g.slices - 1) / g.slices;
+  const int sb_begin = min((int)blockIdx.y * sb_slice, sblocks), sb_end = min(sb_begin + sb_slice, sblocks);
+  const int per = (sb_end - sb_begin + waves - 1) / waves;
+  const int first = sb_begin + wave * per;
+  const int mine = max(0, min(per, sb_end - first));
   uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point of the super-block being computed
 
   // With groups of 128 columns a lane's scales and zero-points of eight consecutive super-blocks are 32 and 8
@@ -507,10 +514,39 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     float v = 0.f;
     for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + at];
     const int n = n0 + col;
-    if (n < mem.N) {
+    if (g.slices > 1) {
+      g.partials[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * g.M + m) * (32 * kNT) + col] = v;
+    } else if (n < mem.N) {
       const float b = mem.bias ? (float)mem.bias[n] : 0.f;
       mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
     }
+  }
+}
+
+// Adds the K slices of skinny_group_kernel in slice order, then bias, and writes y.  One workgroup per tile.
+template <int kNT>
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const SkinnyArgs g) {
+  SkinnyMember mem = g.mem[0];
+  int blk_base = 0;
+#define GLOWQ_PICK(i)                                          \
+  if (g.n_members > i && (int)blockIdx.x >= g.blk_end[i - 1]) { \
+    mem = g.mem[i];                                            \
+    blk_base = g.blk_end[i - 1];                               \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
+  const int n0 = ((int)blockIdx.x - blk_base) * (32 * kNT);
+  const int slots = g.M * (32 * kNT);
+  for (int sidx = threadIdx.x; sidx < slots; sidx += blockDim.x) {
+    const int m = sidx / (32 * kNT), col = sidx - m * (32 * kNT);
+    const int n = n0 + col;
+    if (n >= mem.N) continue;
+    float v = 0.f;
+    for (int sl = 0; sl < g.slices; ++sl) v += g.partials[(((size_t)sl * gridDim.x + blockIdx.x) * g.M + m) * (32 * kNT) + col];
+    const float b = mem.bias ? (float)mem.bias[n] : 0.f;
+    mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
   }
 }
 
@@ -539,14 +575,34 @@ bool skinny_supported(const GroupDev& g) {
 // or more super-blocks per wave, and scale rows that start on a 4-byte boundary.
 static bool skinny_bulk_runs(const SkinnyArgs& a, int waves) {
   const int sblocks = a.K >> 8;
-  if (a.gs_shift != 7 || sblocks < 8 || (sblocks + waves - 1) / waves < 4) return false;
+  const int sb_slice = (sblocks + a.slices - 1) / a.slices;
+  if (a.gs_shift != 7 || sblocks < 8 || (sb_slice + waves - 1) / waves < 4) return false;
   for (int i = 0; i < a.n_members; ++i)
     if ((a.mem[i].lds & 1) != 0 || (reinterpret_cast<uintptr_t>(a.mem[i].scales) & 3u) != 0) return false;
   return true;
 }
 
+// ws_bytes: room behind a.partials (0: none).  The second form cuts K into slices through it where the column tiles
+// alone leave half of the CUs or more without a workgroup and every wave still keeps three super-blocks and more
+// (4096 outputs of K = 14336: 128 workgroups -> 2 x 128; 8 rows 16.6 -> about 14.5 us, 64 rows 41 -> about 28).
 template <int kMT, int kNT, bool kGroupForm>
-static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) {
+static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t ws_bytes, hipStream_t stream) {
+  int total = 0;
+  for (int i = 0; i < a.n_members; ++i) {
+    total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
+    a.blk_end[i] = total;
+  }
+  a.slices = 1;
+  static const int env_split = getenv("GLOWQ_SKINNY_SPLIT") ? atoi(getenv("GLOWQ_SKINNY_SPLIT")) : 1;
+  if (kGroupForm && env_split != 0 && a.partials != nullptr && total * 2 <= num_cus) {
+    const int sblocks = a.K >> 8;
+    int s = num_cus / total;
+    if (s > sblocks / (3 * waves)) s = sblocks / (3 * waves);
+    if (s > 8) s = 8;
+    const size_t per_slice = (size_t)total * a.M * (32 * kNT) * sizeof(float);
+    if (per_slice > 0 && (size_t)s > ws_bytes / per_slice) s = (int)(ws_bytes / per_slice);
+    if (s >= 2) a.slices = s;
+  }
   const bool bulk = kGroupForm && skinny_bulk_runs(a, waves);
   auto kern = !kGroupForm ? skinny_mfma_kernel<kMT, kNT>
               : bulk ? skinny_group_kernel<kMT, kNT, true> : skinny_group_kernel<kMT, kNT, false>;
@@ -554,12 +610,9 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, hipStream_t stream) 
   if (kGroupForm && lds < (size_t)waves * (kMT * 64 + kNT * 32) * 144) lds = (size_t)waves * (kMT * 64 + kNT * 32) * 144;
   static LdsLimit lds_limit[2];  // one per kernel this site launches
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit[bulk]); e != hipSuccess) return e;
-  int total = 0;
-  for (int i = 0; i < a.n_members; ++i) {
-    total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
-    a.blk_end[i] = total;
-  }
-  hipLaunchKernelGGL(kern, dim3(total), dim3(waves * 64), lds, stream, a);
+  hipLaunchKernelGGL(kern, dim3(total, a.slices), dim3(waves * 64), lds, stream, a);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess || a.slices == 1) return e;
+  hipLaunchKernelGGL(skinny_reduce_kernel<kNT>, dim3(total), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 
@@ -573,6 +626,10 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
   a.rank = g.rank;
   a.gs_shift = __builtin_ctz(g.group_size);
   a.alpha = g.alpha;
+  a.slices = 1;
+  const bool ws_ok = g.ws != nullptr && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0;
+  a.partials = ws_ok ? static_cast<float*>(g.ws) : nullptr;
+  const size_t ws_bytes = ws_ok ? g.ws_bytes : 0;
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
     SkinnyMember& s = a.mem[i];
@@ -598,10 +655,10 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
     const bool wide = cols >= 64L * num_cus;
     if (env_waves < 1) waves = wide ? 4 : (g.M <= 32 ? 8 : 6);  // staging tiles: 18 / 13.5 / 22.5 KB of LDS per wave
     if (waves > (g.K >> 8)) waves = g.K >> 8;
-    if (g.M <= 32) return wide ? launch_skinny_t<1, 2, true>(a, waves, stream) : launch_skinny_t<1, 1, true>(a, waves, stream);
+    if (g.M <= 32) return wide ? launch_skinny_t<1, 2, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true>(a, waves, num_cus, ws_bytes, stream);
     if (!wide) {
       if (waves > 6) waves = 6;
-      return launch_skinny_t<2, 1, true>(a, waves, stream);  // 2 x 2 tiles do not fit the register file with the staging
+      return launch_skinny_t<2, 1, true>(a, waves, num_cus, ws_bytes, stream);  // 2 x 2 tiles do not fit the register file with the staging
     }
     // many columns and more than 32 rows: two passes of 32 rows over the wide tile beat one pass over the narrow one
     for (int m0 = 0; m0 < g.M; m0 += 32) {
@@ -610,15 +667,15 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
       c.x = a.x + (size_t)m0 * g.K;
       c.r = a.r ? a.r + (size_t)m0 * g.rank : nullptr;
       for (int i = 0; i < g.n_members; ++i) c.mem[i].y = a.mem[i].y + (size_t)m0 * a.mem[i].ldy;
-      hipError_t e = launch_skinny_t<1, 2, true>(c, waves, stream);
+      hipError_t e = launch_skinny_t<1, 2, true>(c, waves, num_cus, ws_bytes, stream);
       if (e != hipSuccess) return e;
     }
     return hipSuccess;
   }
   const int kblocks = g.K >> 6;
   if (waves > kblocks) waves = kblocks;
-  if (g.M <= 32) return launch_skinny_t<1, 2, false>(a, waves, stream);
-  return launch_skinny_t<2, 2, false>(a, waves, stream);
+  if (g.M <= 32) return launch_skinny_t<1, 2, false>(a, waves, num_cus, ws_bytes, stream);
+  return launch_skinny_t<2, 2, false>(a, waves, num_cus, ws_bytes, stream);
 }
 
 }  // namespace glowq

@@ -97,11 +97,11 @@ class W4A16Extension:
     WORKSPACE_BYTES = 64 << 20
 
     def _workspace(self, dev: torch.device, rows: int):
-        """(pointer, bytes) of the workspace of the current stream of `dev` (many-row projection, split-K of the GEMM):
-        one per stream, because calls that share one must not overlap.  Only calls with more than 16 token rows use it.  A stream that meets its
-        first such call while it is being captured into a graph goes without (the buffer would come from the graph's
-        own memory pool)."""
-        if rows <= 16:
+        """(pointer, bytes) of the workspace of the current stream of `dev` (many-row projection, split-K of the GEMM
+        and of the skinny kernel): one per stream, because calls that share one must not overlap.  Only calls with more
+        than 4 token rows use it.  A stream that meets its first such call while it is being captured into a graph goes
+        without (the buffer would come from the graph's own memory pool)."""
+        if rows <= 4:
             return None, 0
         key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev))
         ws = self._workspaces.get(key)

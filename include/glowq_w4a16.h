@@ -139,6 +139,8 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
  * K where the output has too few tiles to fill the chip (long K, few columns: o_proj / down_proj at some hundred
  * rows): partial fp32 tiles, added in slice order by a second launch.  A slice of the split takes
  * 4 * roundup(M, 128) * sum_i roundup(N_i, 256) bytes; the split goes as far as the workspace holds slices.
+ * The skinny MFMA route (5..64 rows) splits K the same way where its column tiles cover half of the CUs or fewer and
+ * K is 12288 columns or longer (down_proj): 4 * M * sum_i roundup(N_i, 32) bytes per slice, at most 8 slices.
  */
 int glowq_w4a16_group_forward_ws(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
                                  int K, int group_size, int rank, float alpha, void* workspace, size_t workspace_bytes,

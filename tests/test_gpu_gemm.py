@@ -89,6 +89,37 @@ def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     assert_close(y.cpu().numpy(), x.astype(np.float64) @ w.T, f"skinny M={M} K={K} N={N}")
 
 
+@pytest.mark.parametrize("M,K,Ns,rank", [(8, 14336, [256, 64], 128), (16, 14336, [4096], 128), (33, 14336, [128], 64),
+                                         (64, 12288, [96], 128), (5, 18432, [40, 300], 0)])
+def test_skinny_split_k_through_workspace(ext, M, K, Ns, rank):
+    """Few column tiles and a long K: the skinny kernel cuts K into slices through the workspace (the correction rides
+    on the first slice only) and a second launch adds them up; without a workspace the same call runs unsplit."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    assert ext.lib.glowq_w4a16_route(M, K, sum(Ns), 128, K // 8) == 1
+    x, members, R = make_group(733 + M, M, K, Ns, rank, with_bias=True)
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]),
+            "L": dev(m["L"]) if rank else None, "bias": dev(m["bias"])} for m in members]
+    want = [(oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 0.5) if rank else
+             oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)) + m["bias"].astype(np.float64)[None, :] for m in members]
+    r = torch.empty(M, rank, dtype=torch.float16, device="cuda") if rank else None
+    outs = ext.group_forward(dev(x), r, mem, 128, 0.5, R=dev(R) if rank else None)
+    torch.cuda.synchronize()
+    for i, (w, y) in enumerate(zip(want, outs)):
+        assert_close(y.cpu().numpy(), w, f"split skinny member {i}")
+    saved = ext.WORKSPACE_BYTES, dict(ext._workspaces)
+    try:
+        ext.WORKSPACE_BYTES = 64  # too small for a single slice: the call must fall back to the unsplit launch
+        ext._workspaces.clear()
+        outs2 = ext.group_forward(dev(x), r, mem, 128, 0.5, R=dev(R) if rank else None)
+        torch.cuda.synchronize()
+        for i, (w, y) in enumerate(zip(want, outs2)):
+            assert_close(y.cpu().numpy(), w, f"unsplit skinny member {i}")
+    finally:
+        ext.WORKSPACE_BYTES = saved[0]
+        ext._workspaces.clear()
+        ext._workspaces.update(saved[1])
+
+
 @pytest.mark.parametrize("M,K,Ns,rank", [(3, 4096, [512, 128, 128], 128), (4, 2048, [300], 64), (4, 5632, [96, 40], 128), (2, 4096, [256], 128)])
 def test_small_groups_at_two_to_four_rows(ext, M, K, Ns, rank):
     """Default route limits: a small group at three or four rows runs on the skinny MFMA kernel, at two rows on the
