@@ -560,9 +560,11 @@ bool skinny_group_form(const GroupDev& g) {
 bool skinny_supported(const GroupDev& g) {
   if (g.M < 1 || g.M > 64) return false;
   if ((g.K & 63) != 0 || (g.group_size & 31) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
-  if (g.r != nullptr && (g.rank & 63) != 0) return false;
+  // r is either given or still to be produced from R into r_out by the projection launch that goes ahead
+  const half_t* r = g.r != nullptr ? g.r : (g.R != nullptr ? g.r_out : nullptr);
+  if (r != nullptr && (g.rank & 63) != 0) return false;
   if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
-  if (g.r != nullptr && (reinterpret_cast<uintptr_t>(g.r) & 15u) != 0) return false;
+  if (r != nullptr && (reinterpret_cast<uintptr_t>(r) & 15u) != 0) return false;
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
     if ((reinterpret_cast<uintptr_t>(m.qweight) & 15u) != 0 || (m.ldw & 3) != 0) return false;
