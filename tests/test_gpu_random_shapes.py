@@ -39,9 +39,23 @@ def random_cases(n, seed=20240):
     return cases
 
 
+@pytest.fixture(params=["default", "quad", "classic"])
+def route_mode(request, ext):
+    """The library's own route limits, the 4x4x4 matrix-core GEMV for every case of 1..16 rows it can take, or that
+    kernel switched off (wave-dot GEMV up to 4 rows, skinny MFMA kernel above)."""
+    if request.param == "default":
+        yield request.param
+        return
+    old = [ext.set_tuning("quad_max_m", 16 if request.param == "quad" else 0), ext.set_tuning("quad_min_m", 1),
+           ext.set_tuning("small_group_mb", 0)]
+    yield request.param
+    for key, value in zip(("quad_max_m", "quad_min_m", "small_group_mb"), old):
+        ext.set_tuning(key, value)
+
+
 # GLOWQ_RANDOM_CASES / GLOWQ_RANDOM_SEED widen or move the sweep for a hunting run; the defaults are what the suite runs
-@pytest.mark.parametrize("case", random_cases(int(os.environ.get("GLOWQ_RANDOM_CASES", "48")), int(os.environ.get("GLOWQ_RANDOM_SEED", "20240"))), ids=lambda c: f"{c[0]}-M{c[1]}-K{c[2]}-N{'_'.join(map(str, c[3]))}-r{c[4]}-g{c[5]}")
-def test_random_group_matches_oracle(ext, case):
+@pytest.mark.parametrize("case", random_cases(int(os.environ.get("GLOWQ_RANDOM_CASES", "32")), int(os.environ.get("GLOWQ_RANDOM_SEED", "20240"))), ids=lambda c: f"{c[0]}-M{c[1]}-K{c[2]}-N{'_'.join(map(str, c[3]))}-r{c[4]}-g{c[5]}")
+def test_random_group_matches_oracle(ext, route_mode, case):
     i, M, K, Ns, rank, gs, alpha, bias, bare = case
     print(f"case {case}", flush=True)
     x, members, R = make_group(9000 + i, M, K, Ns, rank, group_size=gs, with_bias=bias)
@@ -59,7 +73,7 @@ def test_random_group_matches_oracle(ext, case):
     route = ROUTES.get(ext.lib.glowq_w4a16_route(M, K, sum(Ns), gs, members[0]["qweight"].shape[1]), "?")
     for j, (w, y) in enumerate(zip(want, outs)):
         assert y.shape == (M, Ns[j])
-        assert_close(y.cpu().numpy(), w, f"case {i} member {j} route {route}")
+        assert_close(y.cpu().numpy(), w, f"case {i} member {j} route {route} ({route_mode})")
     if rank:
         want_r = x.astype(np.float64) @ R.astype(np.float64).T
         assert_close(r.cpu().numpy(), want_r, f"case {i} shared projection")
