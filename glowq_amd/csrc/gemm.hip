@@ -154,7 +154,6 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
       *reinterpret_cast<h8*>(dst) = permute ? permute_for_nibble_order(v) : v;
     }
   };
-  auto load_a = [&](const half_t* src, int ld, int kb) { load_a_to(areg, src, ld, kb); };
   auto store_a = [&](int stage, bool permute) { store_a_from(areg, stage, permute); };
   // A fragment of MFMA step t for row tile tm: octet (4*lh + t) of row tm*32 + ln
   auto read_a = [&](int stage, int tm, int t) {
@@ -183,8 +182,20 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
 
   // ---- phase 1: the correction as a K-extension, acc = r . L^T, fp16 B operand ----------------------
   if (kQuant && a.r != nullptr && blockIdx.y == 0) {
-    const int steps = a.rank / kBK;
-    load_a(a.r, a.rank, 0);
+    // ranks are multiples of 8: in a partial last block the octets of r past the rank count as zero and L is read
+    // from the row's last octet (finite values)
+    const int steps = (a.rank + kBK - 1) / kBK;
+    auto load_r = [&](int kb) {
+#pragma unroll
+      for (int i = 0; i < kMT; ++i) {
+        const int q = tid + 256 * i;
+        const int row = min(m0 + (q >> 3), a.M - 1);
+        const int k = kb + (q & 7) * 8;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(a.r + (size_t)row * a.rank + min(k, a.rank - 8));
+        areg.v[i] = k < a.rank ? v : u32x4{0u, 0u, 0u, 0u};
+      }
+    };
+    load_r(0);
     store_a(stage, false);
     __syncthreads();
     for (int ks = 0; ks < steps; ++ks) {
@@ -193,8 +204,8 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
       for (int tn = 0; tn < kNT; ++tn)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + ks * kBK + 32 * lh + 8 * t);
-      if (ks + 1 < steps) load_a(a.r, a.rank, (ks + 1) * kBK);
+          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + min(ks * kBK + 32 * lh + 8 * t, a.rank - 8));
+      if (ks + 1 < steps) load_r((ks + 1) * kBK);
       mma_step(stage, bfrag);
       if (ks + 1 < steps) store_a(stage ^ 1, false);
       __syncthreads();
@@ -611,7 +622,7 @@ bool gemm_supported(const GroupDev& g) {
   if ((g.K % kBK) != 0 || (g.group_size % 32) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
   // r is either given or still to be produced from R into r_out by the projection launch that goes ahead
   const half_t* r = g.r != nullptr ? g.r : (g.R != nullptr ? g.r_out : nullptr);
-  if (r != nullptr && (g.rank % kBK) != 0) return false;
+  if (r != nullptr && ((g.rank & 7) != 0 || g.rank < 8)) return false;
   if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
   if (r != nullptr && (reinterpret_cast<uintptr_t>(r) & 15u) != 0) return false;
   for (int i = 0; i < g.n_members; ++i) {

@@ -10,7 +10,7 @@
 //   * A operand: the lane's 8 activations per MFMA step straight from global memory (x is a few hundred KB at
 //     most and lives in L2), permuted in registers into the order the nibble masks deliver the codes.  With
 //     kNT >= 2 every A fragment feeds two MFMAs, which keeps the L1 traffic per weight byte low enough.
-// The correction is a K-extension in front: the rank/64 blocks of [r | L] are dealt to the waves first,
+// The correction is a K-extension in front: the ceil(rank/64) blocks of [r | L] are dealt to the waves first,
 // acc *= alpha, then the weight blocks accumulate on top.  The waves' partial tiles meet in LDS once.
 #include <cstdlib>
 
@@ -122,18 +122,22 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
   // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
   const bool corrected = mem.L != nullptr && g.r != nullptr;
   if (corrected) {
-    const int lblocks = g.rank >> 6;
+    const int lblocks = (g.rank + 63) >> 6;  // ranks are multiples of 8: the last block may be partial
     for (int jb = wave; jb < lblocks; jb += waves) {
       const int kb = jb * 64;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
+        // octets past the rank: r counts as zero there, L is read from the row's last octet (finite values)
+        const int k = kb + 32 * lh + 8 * t;
+        const bool live = k < g.rank;
+        const int kc = min(k, g.rank - 8);
         h8 af[kMT];
 #pragma unroll
         for (int tm = 0; tm < kMT; ++tm)
-          af[tm] = *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kb + 32 * lh + 8 * t);
+          af[tm] = live ? *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kc) : h8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int tn = 0; tn < kNT; ++tn) {
-          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kb + 32 * lh + 8 * t);
+          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kc);
 #pragma unroll
           for (int tm = 0; tm < kMT; ++tm) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf, acc[tm][tn], 0, 0, 0);
         }
@@ -297,18 +301,22 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
   const bool corrected = mem.L != nullptr && g.r != nullptr && blockIdx.y == 0;  // the first slice carries the correction
   if (corrected) {
-    const int lblocks = g.rank >> 6;
+    const int lblocks = (g.rank + 63) >> 6;  // ranks are multiples of 8: the last block may be partial
     for (int jb = wave; jb < lblocks; jb += waves) {
       const int kb = jb * 64;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
+        // octets past the rank: r counts as zero there, L is read from the row's last octet (finite values)
+        const int k = kb + 32 * lh + 8 * t;
+        const bool live = k < g.rank;
+        const int kc = min(k, g.rank - 8);
         h8 af[kMT];
 #pragma unroll
         for (int tm = 0; tm < kMT; ++tm)
-          af[tm] = *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kb + 32 * lh + 8 * t);
+          af[tm] = live ? *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kc) : h8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int tn = 0; tn < kNT; ++tn) {
-          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kb + 32 * lh + 8 * t);
+          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kc);
 #pragma unroll
           for (int tm = 0; tm < kMT; ++tm) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf, acc[tm][tn], 0, 0, 0);
         }
@@ -562,7 +570,7 @@ bool skinny_supported(const GroupDev& g) {
   if ((g.K & 63) != 0 || (g.group_size & 31) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
   // r is either given or still to be produced from R into r_out by the projection launch that goes ahead
   const half_t* r = g.r != nullptr ? g.r : (g.R != nullptr ? g.r_out : nullptr);
-  if (r != nullptr && (g.rank & 63) != 0) return false;
+  if (r != nullptr && ((g.rank & 7) != 0 || g.rank < 8)) return false;
   if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
   if (r != nullptr && (reinterpret_cast<uintptr_t>(r) & 15u) != 0) return false;
   for (int i = 0; i < g.n_members; ++i) {
