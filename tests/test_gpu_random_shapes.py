@@ -31,7 +31,7 @@ def random_cases(n, seed=20240):
             K = max(gs, K // gs * gs)  # most cases keep whole groups; the rest exercise the zero-padded tail group
         M = int(rng.choice(ROWS))
         Ns = [int(rng.integers(1, 700)) for _ in range(int(rng.integers(1, 5)))]
-        rank = int(rng.choice([0, 0, 8, 24, 64, 96, 128, 256]))
+        rank = int(rng.choice([0, 0, 5, 8, 12, 24, 64, 96, 128, 256]))
         alpha = float(rng.choice([1.0, 0.5, 2.0]))
         bias = bool(rng.random() < 0.4)
         bare = [bool(rank and rng.random() < 0.2) for _ in Ns]  # members of a corrected group without their own L
