@@ -51,6 +51,14 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// r = x R^T on the one-workgroup-per-row-of-R kernel (chunks of four token rows) or on the MFMA projection with its sum
+// over K slices: the first up to 16 rows always, and up to 64 rows while M K rank stays below 60 M multiply-adds
+// (K = 4096, rank 128: 3.9 us against 6.4 at 20 rows, 4.4 against 6.6 at 32, level at 64; K = 14336: 7.2 against 8.2 at
+// 32 rows, 9.4 against 8.4 at 48; K = 17408, rank 256: level at 20 rows, 16.3 against 11.4 at 32).
+bool proj_on_small_kernel(int M, int K, int rank) {
+  return M <= 16 || (M <= 64 && (long)M * K * rank <= 60L * 1000 * 1000);
+}
+
 int num_cus() {
   // one value per device; the current device is the one the caller's tensors live on
   static std::atomic<int> cached[64] = {};
@@ -195,7 +203,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   if (g.R != nullptr) {
     // r = x R^T goes ahead as a launch of its own.  (Folding it into the group kernel was measured: the
     // R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch costs.)
-    if (g.M > 16 && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
+    if (!proj_on_small_kernel(g.M, g.K, g.rank) && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
       e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream, g.ws, g.ws_bytes);
     else
       e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
@@ -312,7 +320,7 @@ static int shared_proj_impl(const void* x, const void* R, void* r, int M, int K,
   const half_t* Rp = static_cast<const half_t*>(R);
   half_t* rp = static_cast<half_t*>(r);
   hipError_t e;
-  if (M > 16 && (K & 63) == 0 && aligned16(x) && aligned16(R)) {
+  if (!proj_on_small_kernel(M, K, rank) && (K & 63) == 0 && aligned16(x) && aligned16(R)) {
     e = launch_shared_proj_mfma(xp, Rp, rp, M, K, rank, num_cus(), static_cast<hipStream_t>(stream), ws, ws_bytes);
   } else {
     if ((K & 7) == 0 && (!aligned16(x) || !aligned16(R)))
