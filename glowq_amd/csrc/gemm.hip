@@ -692,6 +692,8 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
                                                         half_t* __restrict__ r, int M, int K, int rank, ProjSplit sp) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* lds_x = reinterpret_cast<half_t*>(smem);  // [2][32][kPRow]; reused for the final reduction
+  constexpr size_t kLdsX = (size_t)2 * 32 * kPRow * sizeof(half_t), kLdsRed = (size_t)4 * kNT * 16 * 64 * 4;
+  constexpr size_t b_tile_offset = kLdsX > kLdsRed ? kLdsX : kLdsRed;  // the waves' B tiles lie behind both
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -703,10 +705,6 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
   const int per_slice = (all_blocks + slices - 1) / slices;
   const int blk_begin = min((int)blockIdx.z * per_slice, all_blocks);
   const int blocks = min(blk_begin + per_slice, all_blocks);  // this workgroup walks blocks [blk_begin, blocks)
-
-  int ncol[kNT];
-#pragma unroll
-  for (int tn = 0; tn < kNT; ++tn) ncol[tn] = min(n0 + tn * 32 + ln, rank - 1);
 
   f16v acc[kNT];
 #pragma unroll
@@ -734,39 +732,54 @@ __global__ __launch_bounds__(256) void proj_mfma_kernel(const half_t* __restrict
       *reinterpret_cast<u32x4*>(lds_x + ((size_t)stage * 32 + (q >> 5)) * kPRow + (q & 31) * 8) = xr.v[i];
     }
   };
+  // R reaches the B operand through a wave-private LDS tile: the wave's 128-byte row segments (its 64-column slice of
+  // 32 kNT rows of R) are loaded in memory order, 8 lanes per segment, and read back in MFMA lane order.  Fragment
+  // loads straight from memory put every lane of a request on a line of its own.
+  constexpr int kSeg = 144;  // bytes per row segment in the tile: 128 + 16, conflict-free fragment reads
+  unsigned char* btile = smem + b_tile_offset + (size_t)wave * (32 * kNT) * kSeg;
   struct BRegs {
-    u32x4 v[kNT][4];
+    u32x4 w[kNT * 4];  // row 8 q + lane / 8 of the tile, piece lane % 8
   };
   // this wave's slice of a block: columns kb + 64*wave .. +63; a slice past the end of K is weighted by zero
   auto load_b = [&](int kb, BRegs& br) {
     const int ks = min(kb + 64 * wave, K - 64);
 #pragma unroll
-    for (int tn = 0; tn < kNT; ++tn)
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-        br.v[tn][t] = *reinterpret_cast<const u32x4*>(R + (size_t)ncol[tn] * K + ks + 32 * lh + 8 * t);
+    for (int q = 0; q < kNT * 4; ++q)
+      br.w[q] = *reinterpret_cast<const u32x4*>(R + (size_t)min(n0 + q * 8 + (lane >> 3), rank - 1) * K + ks + (lane & 7) * 8);
   };
-  auto mma_block = [&](int stage, int kb, const BRegs& br) {
+  auto stage_b = [&](const BRegs& br) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous block are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < kNT * 4; ++q)
+      *reinterpret_cast<u32x4*>(btile + (q * 8 + (lane >> 3)) * kSeg + (lane & 7) * 16) = br.w[q];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto mma_block = [&](int stage, int kb) {
     if (kb + 64 * wave >= K) return;  // wave-uniform: nothing of this slice lies inside K
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const h8 af = *reinterpret_cast<const h8*>(lds_x + ((size_t)stage * 32 + ln) * kPRow + 64 * wave + (4 * lh + t) * 8);
 #pragma unroll
-      for (int tn = 0; tn < kNT; ++tn)
-        acc[tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, __builtin_bit_cast(h8, br.v[tn][t]), acc[tn], 0, 0, 0);
+      for (int tn = 0; tn < kNT; ++tn) {
+        const h8 bf = *reinterpret_cast<const h8*>(btile + (tn * 32 + ln) * kSeg + lh * 64 + t * 16);
+        acc[tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[tn], 0, 0, 0);
+      }
     }
   };
 
   int stage = 0;
-  // Block s: copy B(s) out of its register set, refill that set with B(s+2) and the matching x set with
+  // Block s: move B(s) out of its register set into the wave's LDS tile, refill that set with B(s+2) and the matching x set with
   // x(s+2), run the MFMAs of block s on LDS stage s%2, then move x(s+1) (loaded one block ago) into the other
   // stage.  Two blocks of loads are in flight at any time.
   auto block = [&](int blk, BRegs& br, XRegs& x_fill, const XRegs& x_store) {
-    BRegs cur = br;
+    stage_b(br);
     const int kn = min(blk + 2, all_blocks - 1) * kPK;
     load_b(kn, br);
     load_x(kn, x_fill);
-    mma_block(stage, blk * kPK, cur);
+    mma_block(stage, blk * kPK);
     store_x(stage ^ 1, x_store);
     __syncthreads();
     stage ^= 1;
@@ -892,7 +905,7 @@ static hipError_t launch_proj_t(const half_t* x, const half_t* R, half_t* r, int
   const int m_blocks = (M + 31) / 32;
   const size_t lds_x = (size_t)2 * 32 * kPRow * sizeof(half_t);
   const size_t lds_red = (size_t)4 * NT * 16 * 64 * 4;
-  const size_t lds = lds_x > lds_red ? lds_x : lds_red;
+  const size_t lds = (lds_x > lds_red ? lds_x : lds_red) + (size_t)4 * (32 * NT) * 144;  // + the four waves' B tiles
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(proj_mfma_kernel<NT>), lds, lds_limit); e != hipSuccess) return e;
   ProjSplit sp = {slices > 1 ? static_cast<float*>(ws) : nullptr};
