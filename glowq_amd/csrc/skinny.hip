@@ -299,24 +299,50 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
 
   // ---- phase 1: correction blocks [r | L], fp16 B operand, dealt round-robin to the waves ----------------
+  constexpr int kSegStride = 144;                      // 128 bytes of a row segment + 16: conflict-free fragment reads
+  constexpr int kATile = kMT * 64 * kSegStride;        // bytes per wave
+  constexpr int kBTile = kNT * 32 * kSegStride;
+  unsigned char* atile = smem + (size_t)wave * (kATile + kBTile);
+  unsigned char* btile = atile + kATile;
   const bool corrected = mem.L != nullptr && g.r != nullptr && blockIdx.y == 0;  // the first slice carries the correction
   if (corrected) {
+    // A 64-column block of [r | L] reaches the operands like the weights below: its 128-byte row segments are loaded in
+    // memory order, 8 lanes per segment, into the wave's LDS tiles and read back in MFMA lane order.
     const int lblocks = (g.rank + 63) >> 6;  // ranks are multiples of 8: the last block may be partial
     for (int jb = wave; jb < lblocks; jb += waves) {
-      const int kb = jb * 64;
+      // octets past the rank: r counts as zero there, L is read from the row's last octet (finite values)
+      const int k = jb * 64 + (lane & 7) * 8;
+      const bool live = k < g.rank;
+      const int kc = min(k, g.rank - 8);
+      u32x4 lreg[kNT * 4], rreg[kMT * 4];
+#pragma unroll
+      for (int q = 0; q < kMT * 4; ++q) {
+        rreg[q] = *reinterpret_cast<const u32x4*>(g.r + (size_t)min(q * 8 + (lane >> 3), g.M - 1) * g.rank + kc);
+        if (!live) rreg[q] = u32x4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int q = 0; q < kNT * 4; ++q)
+        lreg[q] = *reinterpret_cast<const u32x4*>(mem.L + (size_t)min(n0 + q * 8 + (lane >> 3), mem.N - 1) * g.rank + kc);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous block are done
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int q = 0; q < kMT * 4; ++q)
+        *reinterpret_cast<u32x4*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = rreg[q];
+#pragma unroll
+      for (int q = 0; q < kNT * 4; ++q)
+        *reinterpret_cast<u32x4*>(btile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = lreg[q];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        // octets past the rank: r counts as zero there, L is read from the row's last octet (finite values)
-        const int k = kb + 32 * lh + 8 * t;
-        const bool live = k < g.rank;
-        const int kc = min(k, g.rank - 8);
         h8 af[kMT];
 #pragma unroll
         for (int tm = 0; tm < kMT; ++tm)
-          af[tm] = live ? *reinterpret_cast<const h8*>(g.r + (size_t)mrow[tm] * g.rank + kc) : h8{0, 0, 0, 0, 0, 0, 0, 0};
+          af[tm] = *reinterpret_cast<const h8*>(atile + (tm * 32 + ln) * kSegStride + lh * 64 + t * 16);
 #pragma unroll
         for (int tn = 0; tn < kNT; ++tn) {
-          const h8 bf = *reinterpret_cast<const h8*>(mem.L + (size_t)ncol[tn] * g.rank + kc);
+          const h8 bf = *reinterpret_cast<const h8*>(btile + (tn * 32 + ln) * kSegStride + lh * 64 + t * 16);
 #pragma unroll
           for (int tm = 0; tm < kMT; ++tm) acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tm], bf, acc[tm][tn], 0, 0, 0);
         }
@@ -340,11 +366,6 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   struct ARegs {
     u32x4 a[kMT * 8];  // half a super-block in load order: segment 8 q + lane / 8, piece lane % 8
   };
-  constexpr int kSegStride = 144;                      // 128 bytes of a row segment + 16: conflict-free fragment reads
-  constexpr int kATile = kMT * 64 * kSegStride;        // bytes per wave
-  constexpr int kBTile = kNT * 32 * kSegStride;
-  unsigned char* atile = smem + (size_t)wave * (kATile + kBTile);
-  unsigned char* btile = atile + kATile;
   const int sblocks = g.K >> 8;
   // this workgroup's super-blocks: all of them, or slice blockIdx.y of g.slices; its waves split that range
   const int sb_slice = (sblocks + g.slices - 1) / g.slices;
