@@ -200,11 +200,35 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
     __syncthreads();
     for (int ks = 0; ks < steps; ++ks) {
       h8 bfrag[kNT][4];
+      if constexpr (kSuper) {
+        // the wave's 32 kNT rows of L, 128 bytes of this block each, in memory order (8 lanes per row) through its LDS
+        // tile, as the weights of the main loop: fragment loads straight from memory cost a line per lane
+        unsigned char* ltile = smem + (size_t)2 * BM * kARow * sizeof(half_t) + (size_t)wave * (32 * kNT) * 144;
+        u32x4 lreg[kNT * 4];
 #pragma unroll
-      for (int tn = 0; tn < kNT; ++tn)
+        for (int q = 0; q < kNT * 4; ++q)
+          lreg[q] = *reinterpret_cast<const u32x4*>(a.bmat + (size_t)min(bn * BN + wave * (32 * kNT) + q * 8 + (lane >> 3), a.N - 1) * a.ldb +
+                                                    min(ks * kBK + (lane & 7) * 8, a.rank - 8));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // fragment reads of the previous block are done
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-          bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + min(ks * kBK + 32 * lh + 8 * t, a.rank - 8));
+        for (int q = 0; q < kNT * 4; ++q)
+          *reinterpret_cast<u32x4*>(ltile + (q * 8 + (lane >> 3)) * 144 + (lane & 7) * 16) = lreg[q];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            bfrag[tn][t] = *reinterpret_cast<const h8*>(ltile + (tn * 32 + ln) * 144 + lh * 64 + t * 16);
+      } else {
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            bfrag[tn][t] = *reinterpret_cast<const h8*>(a.bmat + (size_t)ncol[tn] * a.ldb + min(ks * kBK + 32 * lh + 8 * t, a.rank - 8));
+      }
       if (ks + 1 < steps) load_r((ks + 1) * kBK);
       mma_step(stage, bfrag);
       if (ks + 1 < steps) store_a(stage ^ 1, false);
