@@ -489,14 +489,24 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const half_t* __re
   float best = -INFINITY;
   int idx = 0x7fffffff;
   const int n8 = (reinterpret_cast<uintptr_t>(logits) & 15) == 0 ? n / 8 : 0;  // 16-byte pieces, then the tail
-  for (int i = threadIdx.x; i < n8; i += blockDim.x) {
-    const h8 v = reinterpret_cast<const h8*>(logits)[i];
+  // batches of eight pieces per thread, all requested before the first is looked at: a round trip per batch, not per piece
+  constexpr int kBatch = 8;
+  for (int i0 = threadIdx.x; i0 < n8; i0 += kBatch * blockDim.x) {
+    h8 v[kBatch];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if ((float)v[j] > best) {  // ascending index per thread: the first maximum wins
-        best = (float)v[j];
-        idx = 8 * i + j;
+    for (int b = 0; b < kBatch; ++b) v[b] = reinterpret_cast<const h8*>(logits)[min(i0 + b * (int)blockDim.x, n8 - 1)];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int i = i0 + b * (int)blockDim.x;
+      if (i < n8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if ((float)v[b][j] > best) {  // ascending index per thread: the first maximum wins
+            best = (float)v[b][j];
+            idx = 8 * i + j;
+          }
       }
+    }
   }
   for (int i = 8 * n8 + threadIdx.x; i < n; i += blockDim.x) {
     const float v = (float)logits[i];

@@ -167,6 +167,17 @@ def test_glue_kernels_match_torch(ext, fp16_out):
     pos.fill_(41)
     ext.argmax_advance(logits, nxt, tok, pos)
     assert (int(nxt), int(tok), int(pos)) == (1234, 1234, 42)
+    # a vocabulary-sized vector (several batches of pieces per thread, then a tail) with the tie far apart
+    big = torch.randn(128256 + 3, device="cuda", generator=g).half()
+    big[100003] = 11.0
+    big[9001] = 11.0
+    big[128258] = 11.0
+    ext.argmax_advance(big.reshape(1, -1), nxt, tok, pos)
+    assert (int(nxt), int(tok), int(pos)) == (9001, 9001, 43)
+    big[9001] = 0.0
+    big[100003] = 0.0
+    ext.argmax_advance(big.reshape(1, -1), nxt, tok, pos)
+    assert (int(nxt), int(pos)) == (128258, 44)      # the maximum in the tail behind the last whole piece
 
 
 @pytest.mark.parametrize("d,max_len,pos", [(64, 320, 0), (64, 320, 1), (64, 320, 37), (64, 320, 300), (128, 2100, 257),
