@@ -21,6 +21,10 @@ __device__ __forceinline__ float block_sum(float v, float* red, int nwaves) {
   return t;
 }
 
+// x * sigmoid(x) in fp32: one exponential and one reciprocal (the hardware approximations, about 1 ulp each: far inside
+// the fp16 rounding that follows); a full-precision division costs ten instructions more per element.
+__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
@@ -77,7 +81,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(half_t* __restrict__ 
 // follows needs no projection launch of its own.  One workgroup per row j of R: every workgroup recomputes the (cheap)
 // elementwise result, dots it with R[j] and writes r[j]; the elementwise outputs are written in 8-element chunks dealt
 // round robin over the workgroups.  x_out must not alias x_in (other workgroups still read it).
-__global__ __launch_bounds__(256) void add_rmsnorm_proj_kernel(const half_t* __restrict__ x_in, const half_t* __restrict__ delta,
+template <int kMax>  // chunks of 8 per thread: H <= 8 * blockDim.x * kMax
+__global__ __launch_bounds__(512) void add_rmsnorm_proj_kernel(const half_t* __restrict__ x_in, const half_t* __restrict__ delta,
                                                                const half_t* __restrict__ w, half_t* __restrict__ x_out,
                                                                half_t* __restrict__ h, const half_t* __restrict__ R,
                                                                half_t* __restrict__ r, int H, int rank, float eps) {
@@ -85,7 +90,6 @@ __global__ __launch_bounds__(256) void add_rmsnorm_proj_kernel(const half_t* __r
   const int j = blockIdx.x;
   const int nw = blockDim.x >> 6;
   const int chunks = H >> 3;
-  constexpr int kMax = 4;  // chunks per thread: H <= 8 * 256 * 4
   h8 xv[kMax], wv[kMax], rv[kMax];
   // every load goes out before the first reduction: one memory round trip for the whole kernel
 #pragma unroll
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_proj_kernel(const half_t* __r
 }
 
 // 1024 threads, at most kMax chunks of 8 per thread, all loads first.
+template <int kMax>  // chunks of 8 per thread: n <= 8 * 1024 * kMax
 __global__ __launch_bounds__(1024) void silu_mul_proj_kernel(const half_t* __restrict__ gate, const half_t* __restrict__ up,
                                                              half_t* __restrict__ out, const half_t* __restrict__ R,
                                                              half_t* __restrict__ r, int n, int rank) {
@@ -141,7 +146,6 @@ __global__ __launch_bounds__(1024) void silu_mul_proj_kernel(const half_t* __res
   const int j = blockIdx.x;
   const int nw = blockDim.x >> 6;
   const int chunks = n >> 3;
-  constexpr int kMax = 4;  // n <= 8 * 1024 * 4
   h8 gv[kMax], uv[kMax], rv[kMax];
 #pragma unroll
   for (int c = 0; c < kMax; ++c) {
@@ -159,7 +163,7 @@ __global__ __launch_bounds__(1024) void silu_mul_proj_kernel(const half_t* __res
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float gf = (float)gv[c][e];
-        o[e] = (half_t)((float)(half_t)(gf / (1.f + __expf(-gf))) * (float)uv[c][e]);
+        o[e] = (half_t)((float)(half_t)silu_f32(gf) * (float)uv[c][e]);
         dot = __builtin_fmaf((float)o[e], (float)rv[c][e], dot);
       }
       if (i % rank == j) reinterpret_cast<h8*>(out)[i] = o;
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const half_t* __restrict_
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float gf = (float)g[j];
-      o[j] = (half_t)((float)(half_t)(gf / (1.f + __expf(-gf))) * (float)u[j]);
+      o[j] = (half_t)((float)(half_t)silu_f32(gf) * (float)u[j]);
     }
     reinterpret_cast<h8*>(out)[i] = o;
   }
@@ -563,13 +567,27 @@ hipError_t launch_silu_mul(const half_t* gate, const half_t* up, half_t* out, lo
 
 hipError_t launch_add_rmsnorm_proj(const half_t* x_in, const half_t* delta, const half_t* w, half_t* x_out, half_t* h,
                                    const half_t* R, half_t* r, int H, int rank, float eps, hipStream_t stream) {
-  hipLaunchKernelGGL(add_rmsnorm_proj_kernel, dim3(rank), dim3(256), 0, stream, x_in, delta, w, x_out, h, R, r, H, rank, eps);
+  // 512 threads and as few chunk slots per thread as H needs: every workgroup redoes the whole elementwise part, so
+  // slots that only repeat the last chunk are instructions on its critical path
+  const int slots = ((H >> 3) + 511) / 512;
+  if (slots <= 1)
+    hipLaunchKernelGGL(add_rmsnorm_proj_kernel<1>, dim3(rank), dim3(512), 0, stream, x_in, delta, w, x_out, h, R, r, H, rank, eps);
+  else if (slots == 2)
+    hipLaunchKernelGGL(add_rmsnorm_proj_kernel<2>, dim3(rank), dim3(512), 0, stream, x_in, delta, w, x_out, h, R, r, H, rank, eps);
+  else
+    hipLaunchKernelGGL(add_rmsnorm_proj_kernel<4>, dim3(rank), dim3(512), 0, stream, x_in, delta, w, x_out, h, R, r, H, rank, eps);
   return hipGetLastError();
 }
 
 hipError_t launch_silu_mul_proj(const half_t* gate, const half_t* up, half_t* out, const half_t* R, half_t* r, int n, int rank,
                                 hipStream_t stream) {
-  hipLaunchKernelGGL(silu_mul_proj_kernel, dim3(rank), dim3(1024), 0, stream, gate, up, out, R, r, n, rank);
+  const int slots = ((n >> 3) + 1023) / 1024;
+  if (slots <= 1)
+    hipLaunchKernelGGL(silu_mul_proj_kernel<1>, dim3(rank), dim3(1024), 0, stream, gate, up, out, R, r, n, rank);
+  else if (slots == 2)
+    hipLaunchKernelGGL(silu_mul_proj_kernel<2>, dim3(rank), dim3(1024), 0, stream, gate, up, out, R, r, n, rank);
+  else
+    hipLaunchKernelGGL(silu_mul_proj_kernel<4>, dim3(rank), dim3(1024), 0, stream, gate, up, out, R, r, n, rank);
   return hipGetLastError();
 }
 
