@@ -418,7 +418,7 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
 // projection r[j] = out . R[j] of the group that consumes it: one workgroup per row of R recomputes the combination
 // (the partials are a few tens of KB) and writes 8-element chunks of `out` dealt round robin, as the other fused
 // glue kernels do.  Without R a few workgroups just write their chunks.
-constexpr int kCombineSplits = 8;  // splits whose partials are all fetched before any is used
+template <int kCombineSplits>  // splits whose partials are all fetched before any is used (more walk them one by one)
 __global__ __launch_bounds__(1024) void attend_combine_proj_kernel(const float* __restrict__ part, half_t* __restrict__ out,
                                                                    const half_t* __restrict__ R, half_t* __restrict__ r,
                                                                    int heads, int d, int splits) {
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(1024) void attend_combine_proj_kernel(const float* 
         for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, ph[s * stride + 4 + i0 + e], acc[e]);
       }
     }
-    const float inv = 1.f / den;
+    const float inv = __builtin_amdgcn_rcpf(den);
     h8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (half_t)(acc[e] * inv);
@@ -629,7 +629,12 @@ hipError_t launch_attend_combine_proj(const float* part, half_t* out, const half
   const int chunks = heads * d / 8;
   int threads = (chunks + 63) / 64 * 64;  // one 8-element chunk per thread where the workgroup size allows
   threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
-  hipLaunchKernelGGL(attend_combine_proj_kernel, dim3(wgs), dim3(threads), 0, stream, part, out, R, r, heads, d, splits);
+  if (splits <= 2)
+    hipLaunchKernelGGL(attend_combine_proj_kernel<2>, dim3(wgs), dim3(threads), 0, stream, part, out, R, r, heads, d, splits);
+  else if (splits <= 4)
+    hipLaunchKernelGGL(attend_combine_proj_kernel<4>, dim3(wgs), dim3(threads), 0, stream, part, out, R, r, heads, d, splits);
+  else
+    hipLaunchKernelGGL(attend_combine_proj_kernel<8>, dim3(wgs), dim3(threads), 0, stream, part, out, R, r, heads, d, splits);
   return hipGetLastError();
 }
 
