@@ -121,11 +121,17 @@ __global__ __launch_bounds__(512) void add_rmsnorm_proj_kernel(const half_t* __r
   for (int c = 0; c < kMax; ++c) {
     const int i = threadIdx.x + c * blockDim.x;
     if (i < chunks) {
+      // fp16(x * inv) in fp32, then the weight as a packed fp16 product (the fp32 product of two halves is exact, so one
+      // rounding either way) and the dot with R two elements at a time in fp32
       h8 o;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        o[e] = (half_t)((float)(half_t)((float)xv[c][e] * inv) * (float)wv[c][e]);
-        dot = __builtin_fmaf((float)o[e], (float)rv[c][e], dot);
+      for (int e = 0; e < 8; e += 2) {
+        const h2 n2 = {(half_t)((float)xv[c][e] * inv), (half_t)((float)xv[c][e + 1] * inv)};
+        const h2 w2 = {wv[c][e], wv[c][e + 1]};
+        const h2 o2 = n2 * w2;
+        o[e] = o2[0];
+        o[e + 1] = o2[1];
+        dot = __builtin_amdgcn_fdot2(o2, h2{rv[c][e], rv[c][e + 1]}, dot, false);
       }
       if (i % rank == j) {
         reinterpret_cast<h8*>(x_out)[i] = xv[c];
