@@ -282,15 +282,32 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
     v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
   }
   const int pos = (int)*pos_p;
+  // A position outside the cache (a caller stepping past max_len - 1): nothing is written -- no cache row, no output,
+  // no partial -- instead of indexing the tables and the caches out of bounds.  Uniform over the grid.
+  if (pos < 0 || pos >= max_len) return;
 
   // rotary embedding of q and k_new: out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i + d/2] cos + x[i] sin
   if (threadIdx.x < half_d) {
     const int i = threadIdx.x;
     // the tables are rounded to fp16 first, as a half-precision model's rotary embedding does
     const float c = (float)(half_t)cos_t[(size_t)pos * d + i], sn = (float)(half_t)sin_t[(size_t)pos * d + i];
-    qs[i] = (float)(half_t)(q0 * c - q1 * sn);
-    qs[i + half_d] = (float)(half_t)(q1 * c + q0 * sn);
-    const half_t r0 = (half_t)(k0 * c - k1 * sn), r1 = (half_t)(k1 * c + k0 * sn);
+    // Two fp32 products and one fp32 sum, each rounded on its own, then one rounding to fp16: what the elementwise
+    // tensor expression x * cos + rotate_half(x) * sin evaluates.  A fused multiply-add skips the rounding of one
+    // product, which now and then lands on the other side of an fp16 rounding boundary (one cached key element in some
+    // thousand rows differed by an fp16 ulp from the tensor expression before contraction was switched off here).
+    float qa, qb, ka, kb;
+    {
+#pragma clang fp contract(off)
+      const float q0c = q0 * c, q1s = q1 * sn, q1c = q1 * c, q0s = q0 * sn;
+      const float k0c = k0 * c, k1s = k1 * sn, k1c = k1 * c, k0s = k0 * sn;
+      qa = q0c - q1s;
+      qb = q1c + q0s;
+      ka = k0c - k1s;
+      kb = k1c + k0s;
+    }
+    qs[i] = (float)(half_t)qa;
+    qs[i + half_d] = (float)(half_t)qb;
+    const half_t r0 = (half_t)ka, r1 = (half_t)kb;
     kn[i] = (float)r0;
     kn[i + half_d] = (float)r1;
     vn[i] = (float)v0;

@@ -264,20 +264,36 @@ class FusedStep:
 
     @staticmethod
     def _group(mods, outs, f16):
-        members, R, alpha, gs = [], None, 1.0, None
+        """Launch description of a group.  The corrected members of one launch must share one right factor and one
+        alpha (the group kernel applies a single r and a single alpha); artifacts with a factor pair per module
+        (layer-wise, non-shared correction) get `per_member` instead: one projection and one launch per module."""
+        members, factors, gs = [], [], None
         for mod in mods:
             inner = mod.inner if isinstance(mod, AddSVDCorrection) else mod
             if not isinstance(inner, CudaW4A16Linear):
                 raise TypeError("FusedStep needs every projection converted to CudaW4A16Linear")
             L = None
             if isinstance(mod, AddSVDCorrection) and mod.alpha_svd != 0.0:
-                L, alpha = mod.A_q, float(mod.alpha_svd)
-                R = mod.B_q if R is None else R
+                L = mod.A_q
+                factors.append((mod.B_q, float(mod.alpha_svd)))
+            else:
+                factors.append(None)
             gs = inner.group_size
             members.append({"qweight": inner.qweight_i32, "scales": inner.scales_f16, "qzeros": inner.qzeros_i32, "L": L,
                             "bias": inner.bias})
-        r = torch.zeros(1, R.size(0), **f16) if R is not None else None
-        return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs}
+        corrected = [f for f in factors if f is not None]
+        R, alpha = (corrected[0] if corrected else (None, 1.0))
+        shared = all(a == alpha and (B.data_ptr() == R.data_ptr() or (B.shape == R.shape and bool(torch.equal(B, R))))
+                     for B, a in corrected)
+        if shared:
+            r = torch.zeros(1, R.size(0), **f16) if R is not None else None
+            return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs, "per_member": None}
+        per_member = []
+        for mem, f, out in zip(members, factors, outs):
+            Ri, ai = f if f is not None else (None, 1.0)
+            per_member.append({"members": [mem], "R": Ri, "r": torch.zeros(1, Ri.size(0), **f16) if Ri is not None else None,
+                               "alpha": ai, "gs": gs, "outs": [out], "per_member": None})
+        return {"members": members, "R": None, "r": None, "alpha": 1.0, "gs": gs, "outs": outs, "per_member": per_member}
 
     def _norm(self, x, delta, ln, grp):
         """Residual add + RMSNorm into self.h; with a shared group behind it the projection r = h R^T comes out of the same
@@ -290,6 +306,10 @@ class FusedStep:
         return x, False
 
     def _linear(self, x, grp, r_ready=False):
+        if grp["per_member"] is not None:
+            for sub in grp["per_member"]:
+                self.ext.group_forward(x, sub["r"], sub["members"], sub["gs"], sub["alpha"], outs=sub["outs"], R=sub["R"])
+            return
         if self.share:
             self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"],
                                    R=None if r_ready else grp["R"])

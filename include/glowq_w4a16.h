@@ -58,10 +58,17 @@ int glowq_version(void);
 const char* glowq_last_error(void);
 
 /*
- * y = fp16( sum_k (code - zero) * scale * x ), fp32 accumulate, weights never rounded to fp16.
+ * y = fp16( sum_k (code - zero) * scale * x ), fp32 accumulate.
  * Replaces `w4a16_gemv_forward_cuda` (src/cuda_w4a16/csrc/gemv_w4a16.cu:146-214; pybind
- * src/cuda_w4a16/csrc/pybind.cpp:19-23).  Any M is accepted; all M rows share one pass over the
- * weights in chunks of the kernel's row capacity.
+ * src/cuda_w4a16/csrc/pybind.cpp:19-23).  Any M is accepted; all M rows share one pass over the weights.
+ * Weight rounding by row count: the GEMV kernels (1 token row; 2..4 rows by group size, see glowq_set_tuning) keep
+ * (code - zero) * scale unrounded, as the reference's GEMV does (gemv_w4a16.cu:96-112).  From the row count at which
+ * the MFMA kernels take over (3..5 rows, glowq_w4a16_route tells) the dequantised weight is rounded once to fp16
+ * before the multiply, which is the arithmetic of the reference's dequantise-then-matmul route (gemm_w4a16.cu:46-49,132)
+ * -- the reference itself switches to that arithmetic only above 128 rows.  On activations of order one the two differ
+ * by far less than 1e-2 + 1e-3 |y|; with outlier channels in the thousands they differ by more than that, in the
+ * reference as here, so compare against the matching one.  glowq_set_tuning("quad_max_m", 16) together with
+ * ("small_group_mb", 0) keeps the unrounded arithmetic (the 4x4x4 GEMV) up to 16 rows.
  */
 int glowq_w4a16_gemv_forward(const void* x, const int32_t* qweight, const void* scales, const int32_t* qzeros,
                              void* y, int M, int K, int N, int group_size, int ldw_i32, int lds, int ldz_i32,
@@ -194,6 +201,8 @@ int glowq_silu_mul_proj(const void* gate, const void* up, void* out, const void*
  * Rotary embedding of q [heads, d] and k_new [kv_heads, d] at position *pos (cos/sin tables [max_len, d] fp32),
  * append of k / v_new to the caches [kv_heads, max_len, d] at *pos, attention of the one query token over positions
  * 0..*pos, out [heads, d].  d = 64 or 128; one pass with a running maximum, so max_len is bounded by the caches alone.
+ * *pos is read on the device: a value outside [0, max_len) makes the launch write nothing at all (no cache row, no
+ * output, no partial), so a replayed graph that steps past the end of the cache cannot write out of bounds.
  */
 int glowq_rope_attend(const void* q, const void* k_new, const void* v_new, const float* cos_table, const float* sin_table,
                       const int64_t* pos, void* cache_k, void* cache_v, void* out, int heads, int kv_heads, int head_dim,

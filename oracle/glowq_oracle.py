@@ -20,8 +20,9 @@ How each function is pinned (tests/test_oracle_*.py):
   * pack / unpack / quantize / dequant / the CPU forward: bit-exact against golden vectors that
     tests/golden/make_golden.py wrote by running the reference's own functions once in the build
     container (tests/golden/*.npz), plus exhaustive brute force over all nibble values/positions.
-  * gemv_ref / gemm_ref: reduce to ``x @ dequant(W).T`` (a library matmul) and to one-hot inputs
-    that select single dequantised columns exactly.
+  * gemv_ref / gemm_ref / linear_exact / linear_rounded_exact: reduce to ``x @ dequant(W).T`` (a library
+    matmul on the golden-pinned dequant) and to one-hot inputs that select single dequantised columns exactly;
+    linear_rounded_exact rounded to fp16 is gemm_ref.
   * correction / group_forward: closed form ``z + alpha * (x R^T) L^T`` against a float64 library
     matmul; alpha = 0 identity; linearity in alpha; group == independent solo results.
   * quantize on constant groups (scale underflows to 0 in fp16 -> NaN zero-point) is UNDEFINED in
@@ -170,6 +171,15 @@ def linear_exact(x, qweight, qzeros, scales, group_size: int) -> np.ndarray:
     return x.astype(np.float64) @ w.T
 
 
+def linear_rounded_exact(x, qweight, qzeros, scales, group_size: int) -> np.ndarray:
+    """float64 value of x @ dequant(W)^T with the dequantised weight rounded to fp16 first and no output rounding:
+    the "dequantise, then matmul" route (src/cuda_w4a16/csrc/gemm_w4a16.cu:46-49,132) without the library GEMM's own
+    rounding.  ``gemm_ref`` is this value rounded to fp16."""
+    x = _h(x)
+    w = dequant(qweight, qzeros, scales, x.shape[1], group_size)
+    return x.astype(np.float64) @ w.astype(np.float64).T
+
+
 # --------------------------------------------------------------------------------------
 # group-shared low-rank correction
 # --------------------------------------------------------------------------------------
@@ -188,6 +198,14 @@ def correction(z, r, L, alpha: float, acc=np.float64) -> np.ndarray:
 def corrected_linear_exact(x, qweight, qzeros, scales, group_size, R, L, alpha) -> np.ndarray:
     """float64, unrounded z + alpha * (x R^T) L^T."""
     z = linear_exact(x, qweight, qzeros, scales, group_size)
+    r = _h(x).astype(np.float64) @ _h(R).astype(np.float64).T
+    return z + float(alpha) * (r @ _h(L).astype(np.float64).T)
+
+
+def corrected_linear_rounded_exact(x, qweight, qzeros, scales, group_size, R, L, alpha) -> np.ndarray:
+    """float64, unrounded x @ fp16(dequant(W))^T + alpha * (x R^T) L^T: the dequantise-then-matmul-plus-correction
+    value (gemm_w4a16.cu:76-135 followed by step3_eval_dataset.py:484-511) before any output rounding."""
+    z = linear_rounded_exact(x, qweight, qzeros, scales, group_size)
     r = _h(x).astype(np.float64) @ _h(R).astype(np.float64).T
     return z + float(alpha) * (r @ _h(L).astype(np.float64).T)
 

@@ -29,6 +29,17 @@ def make_group(seed, M, K, Ns, rank, group_size=128, w_std=0.02, with_bias=False
     return x, members, R
 
 
+def outlier_activations(x, seed, scale=4.0, fraction=0.01, factor=200.0):
+    """x scaled by `scale`, with a seeded `fraction` of its channels (columns) another `factor` times larger, rounded
+    to fp16: a few channels in the thousands among values of order one."""
+    rng = np.random.default_rng(seed)
+    K = x.shape[1]
+    cols = rng.choice(K, size=max(1, int(K * fraction)), replace=False)
+    out = x.astype(np.float32)
+    out[:, cols] *= factor
+    return (out * scale).astype(np.float16)
+
+
 def dev(a, device="cuda"):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device)
 

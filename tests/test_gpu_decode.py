@@ -36,18 +36,23 @@ class _RefLinear(nn.Module):
         return (x.float() @ self.w.T).to(x.dtype)
 
 
-def _effective_weight(mod, with_correction=True):
+def _effective_weight(mod, with_correction=True, deq_cache=None):
     inner = mod.inner if isinstance(mod, corr.AddSVDCorrection) else mod
     assert isinstance(inner, CudaW4A16Linear)
-    w = oracle.dequant(inner.qweight_i32.cpu().numpy(), inner.qzeros_i32.cpu().numpy(), inner.scales_f16.cpu().numpy(),
-                       inner.in_features, inner.group_size)[:, : inner.in_features].astype(np.float32)
-    w = torch.from_numpy(w).cuda()
+    w = deq_cache.get(id(inner)) if deq_cache is not None else None
+    if w is None:
+        w = oracle.dequant(inner.qweight_i32.cpu().numpy(), inner.qzeros_i32.cpu().numpy(), inner.scales_f16.cpu().numpy(),
+                           inner.in_features, inner.group_size)[:, : inner.in_features].astype(np.float32)
+        w = torch.from_numpy(w).cuda()
+        if deq_cache is not None:
+            deq_cache[id(inner)] = w
     if with_correction and isinstance(mod, corr.AddSVDCorrection):
         w = w + float(mod.alpha_svd) * (mod.A_q.float() @ mod.B_q.float())
     return w
 
 
-def _swap_in_reference(model, with_correction=True):
+def _swap_in_reference(model, with_correction=True, deq_cache=None):
+    """`deq_cache` (a dict) keeps the oracle-dequantised weights between calls on the same model."""
     saved = []
     for layer in model.model.layers:
         for owner, names in ((layer.self_attn, ("q_proj", "k_proj", "v_proj", "o_proj")),
@@ -55,7 +60,7 @@ def _swap_in_reference(model, with_correction=True):
             for n in names:
                 mod = getattr(owner, n)
                 saved.append((owner, n, mod))
-                setattr(owner, n, _RefLinear(_effective_weight(mod, with_correction)))
+                setattr(owner, n, _RefLinear(_effective_weight(mod, with_correction, deq_cache)))
     return saved
 
 
@@ -214,6 +219,63 @@ def test_rope_attend_matches_torch(ext, fp16_out, d, max_len, pos):
     assert torch.equal(ck2[:, keep], ck[:, keep]) and torch.equal(cv2[:, keep], cv[:, keep])   # nothing else touched
 
 
+def test_appended_key_is_bit_identical_to_the_tensor_expression(ext, fp16_out):
+    """The rotated key written to the cache equals (k * cos + rotate_half(k) * sin) evaluated op by op in fp32 and
+    rounded once to fp16, bit for bit: first on the one input where a fused multiply-add in the kernel's rotary
+    embedding once landed an fp16 ulp away (head dim 128, 2 KV heads, 16 heads, position 1645 of 4100, generator seed
+    23), then over a seeded sweep of keys and positions; the one-workgroup and the split kernel write the same bits."""
+    def run(d, kvh, heads, max_len, pos, seed, splits):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        q = torch.randn(heads * d, device="cuda", generator=g).half()
+        k = torch.randn(kvh * d, device="cuda", generator=g).half()
+        v = torch.randn(kvh * d, device="cuda", generator=g).half()
+        ck = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+        cv = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+        model = decode.Decoder(decode.DecoderConfig(hidden=heads * d, layers=0, heads=heads, kv_heads=kvh, head_dim=d,
+                                                    intermediate=64, vocab=8, max_len=max_len))
+        cos, sin = model.rope_tables("cuda")
+        c, s = cos[pos].half().float(), sin[pos].half().float()
+        kf = k.view(kvh, d).float()
+        kr = (kf * c + torch.cat((-kf[..., d // 2:], kf[..., :d // 2]), dim=-1) * s).half()
+        p = torch.tensor([pos], device="cuda")
+        ck1, cv1, o1 = ck.clone(), cv.clone(), torch.empty(heads * d, dtype=torch.float16, device="cuda")
+        ext.rope_attend(q, k, v, cos, sin, p, ck1, cv1, o1, d ** -0.5)
+        ck2, cv2 = ck.clone(), cv.clone()
+        part = torch.zeros(heads, splits, d + 4, device="cuda")
+        ext.rope_attend_split(q, k, v, cos, sin, p, ck2, cv2, part, d ** -0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(ck1[:, pos], kr), (d, kvh, pos, seed)
+        assert torch.equal(ck1, ck2) and torch.equal(cv1, cv2)
+
+    run(128, 2, 16, 4100, 1645, 23, 3)
+    rng = np.random.default_rng(8)
+    for i in range(48):
+        d = int(rng.choice([64, 128]))
+        run(d, 8, 8, 200, int(rng.integers(0, 200)), 1000 + i, int(rng.choice([2, 4])))
+
+
+def test_position_outside_the_cache_writes_nothing(ext, fp16_out):
+    heads, kvh, d, max_len = 8, 2, 64, 96
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q = torch.randn(heads * d, device="cuda", generator=g).half()
+    k = torch.randn(kvh * d, device="cuda", generator=g).half()
+    v = torch.randn(kvh * d, device="cuda", generator=g).half()
+    ck = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    cv = torch.randn(kvh, max_len, d, device="cuda", generator=g).half()
+    model = decode.Decoder(decode.DecoderConfig(hidden=heads * d, layers=0, heads=heads, kv_heads=kvh, head_dim=d, intermediate=64,
+                                                vocab=8, max_len=max_len))
+    cos, sin = model.rope_tables("cuda")
+    for bad in (max_len, max_len + 7, -1):
+        p = torch.tensor([bad], device="cuda")
+        ck2, cv2 = ck.clone(), cv.clone()
+        out = torch.full((heads * d,), 7.0, dtype=torch.float16, device="cuda")
+        part = torch.full((heads, 4, d + 4), 7.0, device="cuda")
+        ext.rope_attend(q, k, v, cos, sin, p, ck2, cv2, out, d ** -0.5)
+        ext.rope_attend_split(q, k, v, cos, sin, p, ck2, cv2, part, d ** -0.5)
+        torch.cuda.synchronize()
+        assert torch.equal(ck2, ck) and torch.equal(cv2, cv) and (out == 7.0).all() and (part == 7.0).all()
+
+
 @pytest.mark.parametrize("pos,splits", [(0, 4), (1, 4), (3, 8), (37, 4), (300, 4), (300, 7)])
 def test_split_attention_and_merge_match_single_workgroup(ext, fp16_out, pos, splits):
     heads, kvh, d, max_len, rank = 8, 2, 128, 320, 64
@@ -283,6 +345,88 @@ def test_fused_step_matches_module_path(fp16_out):
     for _ in range(3):
         got, _, _ = graphed.generate(prompt, 10)
         assert torch.equal(got, eager)
+
+
+GEOM_8B = dict(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128, intermediate=14336, vocab=4096, max_len=640,
+               group_size=128, rank=128)
+
+
+def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out):
+    """Two layers of the Llama-3.1-8B geometry (hidden 4096, 32 query / 8 KV heads of 128, SwiGLU 14336, W4A16 g = 128,
+    rank 128) with 512 cached positions: the fused single-token step (group launches, attention split over 4 workgroups
+    per head, glue kernels that carry the projections) against the same network with every quantised module replaced
+    by an fp32 matmul on its effective weight, teacher forced; the cache of both is filled by the yardstick network."""
+    cfg = decode.DecoderConfig(**GEOM_8B)
+    model, _, _ = decode.build_decoder(cfg, seed=21)
+    assert sum(isinstance(m, corr.AddSVDCorrection) for m in model.modules()) == 7 * cfg.layers
+    prompt = torch.randint(0, cfg.vocab, (512,), generator=torch.Generator().manual_seed(6))
+    deq = {}
+    ref = decode.GreedyDecoder(model, use_graph=False)
+    fus = decode.GreedyDecoder(model, use_graph=False, fused=True)     # reads the quantised buffers of the modules
+    bare = decode.GreedyDecoder(model, use_graph=False)
+    saved = _swap_in_reference(model, with_correction=False, deq_cache=deq)
+    bare.prefill(prompt)
+    _restore(saved)
+    saved = _swap_in_reference(model, deq_cache=deq)
+    first = ref.prefill(prompt)
+    fus.prefill(prompt)
+    tok = first.clone()
+    worst = 0.0
+    for step in range(4):
+        print(f"8B-geometry step {step}", flush=True)
+        pos = torch.tensor([prompt.numel() + step], device="cuda")
+        want = model.forward_tokens(tok, pos, ref.caches, ref.cos, ref.sin).float()
+        fus.tok.copy_(tok), fus.pos.copy_(pos)
+        fus.fused.run()
+        got = fus.fused.logits.float()
+        err = float((got - want).abs().max())
+        worst = max(worst, err)
+        assert err <= 1e-2 + 1e-2 * float(want.abs().max()), (step, err)
+        assert int(fus.pos) == int(pos) + 1 and int(fus.tok) == int(got.argmax())
+        # the step left the same key / value rows in its cache as the yardstick network
+        for (ka, va), (kb, vb) in zip(ref.caches, fus.caches):
+            assert (ka[:, int(pos)].float() - kb[:, int(pos)].float()).abs().max() <= 2e-2
+            assert (va[:, int(pos)].float() - vb[:, int(pos)].float()).abs().max() <= 2e-2
+        tok = want.argmax(-1)
+    _restore(saved)
+    # the check discriminates: the same step on the network without the correction is much further away
+    saved = _swap_in_reference(model, with_correction=False, deq_cache=deq)
+    pos = torch.tensor([prompt.numel()], device="cuda")
+    without = model.forward_tokens(first, pos, bare.caches, bare.cos, bare.sin).float()
+    _restore(saved)
+    fus2 = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    saved = _swap_in_reference(model, deq_cache=deq)
+    fus2.prefill(prompt)
+    _restore(saved)
+    fus2.tok.copy_(first), fus2.pos.copy_(pos)
+    fus2.fused.run()
+    assert float((fus2.fused.logits.float() - without).abs().max()) > 5 * max(worst, 1e-3)
+
+
+def test_fused_step_with_a_factor_pair_per_module(fp16_out):
+    """Artifacts whose q / k / v (gate / up) hold different right factors cannot share one group launch: the fused step
+    must run them one by one, each with its own r, and still match the module path."""
+    cfg = decode.DecoderConfig(**TINY)
+    model, _, _ = decode.build_decoder(cfg, seed=13)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    for layer in model.model.layers:
+        for owner, name in ((layer.self_attn, "k_proj"), (layer.mlp, "up_proj")):
+            # a solo wrapper with its own R instead of the group's, as the patcher builds for a key without "B_shared"
+            old = getattr(owner, name)
+            old.group_cache.members.remove(old)
+            R = (torch.randn(old.B_q.shape, device="cuda", generator=g) * old.B_q.size(1) ** -0.5).half()
+            setattr(owner, name, corr.AddSVDCorrection(old.inner, old.A_q, R, "solo", False, None, 1.0))
+    prompt = torch.randint(0, cfg.vocab, (9,), generator=torch.Generator().manual_seed(4))
+    ref = decode.GreedyDecoder(model, use_graph=False)
+    fus = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    assert fus.fused.plan[0]["qkv"]["per_member"] is not None and fus.fused.plan[0]["o"]["per_member"] is None
+    first = ref.prefill(prompt)
+    fus.prefill(prompt)
+    pos = torch.tensor([prompt.numel()], device="cuda")
+    want = model.forward_tokens(first, pos, ref.caches, ref.cos, ref.sin).float()
+    fus.tok.copy_(first), fus.pos.copy_(pos)
+    fus.fused.run()
+    assert (fus.fused.logits.float() - want).abs().max() <= 1e-2 + 1e-2 * want.abs().max()
 
 
 def test_perplexity_windows_and_effective_weight_network(fp16_out, tmp_path):
