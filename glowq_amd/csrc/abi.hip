@@ -42,6 +42,29 @@ thread_local char g_err[512] = "";
 
 }  // namespace
 
+// Scratch of glowq_w4a16_group_forward_fused_static: the workspace of the many-row projection and of the skinny kernel's
+// split of K for callers that cannot bring one.  One copy per GPU the library runs on, held until the process ends.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+// Device address of `scratch` on the current device.  The array's name is a host-side stand-in; the address each GPU
+// keeps its copy at comes from hipGetSymbolAddress, asked once per device with that device current.
+std::atomic<void*> g_scratch_ptr[64] = {};
+
+void* static_scratch() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return nullptr;
+  g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing host threads store the same address
+  return p;
+}
+
+}  // namespace
+
 namespace glowq {
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -432,6 +455,28 @@ int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out
   return group_forward_fused_impl(x, R, r_out, members, n_members, M, K, group_size, rank, alpha, workspace,
                                   workspace_bytes, stream);
 }
+
+int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                           int n_members, int M, int K, int group_size, int rank, float alpha,
+                                           void* stream) {
+  if (M > GLOWQ_STATIC_MAX_ROWS)
+    return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: %d token rows, the static scratch serves at most %d", M,
+                GLOWQ_STATIC_MAX_ROWS);
+  // what the two users of the workspace ask for at this shape: the projection's split of K, and the skinny kernel's
+  // (at most one 32-column fp32 tile per token row for each of num_cus workgroup slots)
+  size_t need = (M > 0 && K > 0 && rank > 0) ? proj_workspace_bytes(M, K, rank, num_cus()) : 0;
+  const size_t skinny_need = M > 4 ? (size_t)num_cus() * (size_t)M * 32 * sizeof(float) : 0;
+  if (skinny_need > need) need = skinny_need;
+  if (need > kStaticScratchBytes)
+    return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: this shape wants %zu bytes of scratch, the static buffer holds %zu",
+                need, kStaticScratchBytes);
+  void* ws = static_scratch();
+  if (ws == nullptr) return fail(GLOWQ_ELAUNCH, "group_forward_fused_static: the address of the static scratch is not available");
+  return group_forward_fused_impl(x, R, r_out, members, n_members, M, K, group_size, rank, alpha, ws, kStaticScratchBytes,
+                                  stream);
+}
+
+size_t glowq_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
   GroupDev g;

@@ -53,6 +53,8 @@ _SIGNATURES = {
                                           ctypes.c_size_t, _P]),
     "glowq_w4a16_group_forward_fused_ws": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float,
                                                 _P, ctypes.c_size_t, _P]),
+    "glowq_w4a16_group_forward_fused_static": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_static_scratch_bytes": (ctypes.c_size_t, []),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),

@@ -157,6 +157,21 @@ int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out
                                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * glowq_w4a16_group_forward_fused_ws for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * glowq_w4a16_group_forward_fused_ws called with a workspace of glowq_static_scratch_bytes() bytes, but the workspace
+ * is a static device array inside the library (8 MiB on every GPU the library runs on, held until the process ends);
+ * the call allocates and frees nothing.  At most GLOWQ_STATIC_MAX_ROWS token rows, and shapes whose projection would
+ * want a larger workspace (glowq_proj_workspace_bytes) are refused with GLOWQ_EUNSUPPORTED.  Every call on a GPU shares
+ * that GPU's array: calls that overlap on one GPU (two streams, two threads) race; nothing in it has to start at zero.
+ */
+#define GLOWQ_STATIC_MAX_ROWS 64
+int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r_out, const glowq_member_t* members,
+                                           int n_members, int M, int K, int group_size, int rank, float alpha,
+                                           void* stream);
+size_t glowq_static_scratch_bytes(void);
+
+/*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
  * 2 = tiled MFMA GEMM, 3 = generic (odd shapes), 4 = 4x4x4 matrix-core GEMV.
  */
