@@ -15,6 +15,9 @@ hipError_t launch_generic(GroupDev& g, int num_cus, hipStream_t stream);
 int wave_dot_rows(long total_rows);
 int wave_dot_rows_single(long total_rows);
 bool wave_dot_supported(int M, int K, int rank, bool has_r);
+// gemv_stream.hip
+bool stream_supported(const GroupDev& g);
+hipError_t launch_stream(GroupDev& g, int num_cus, hipStream_t stream);
 // gemv_quad.hip
 int quad_capacity(int M, int K, int rank, bool has_r);
 hipError_t launch_quad(GroupDev& g, int num_cus, hipStream_t stream);
@@ -234,7 +237,10 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     g.r = g.r_out;
     g.R = nullptr;
   }
-  if (route == kRouteGemm) {
+  static const int use_stream = env_or("GLOWQ_STREAM", 1);
+  if (route == kRouteWaveDot && g.M == 1 && use_stream != 0 && stream_supported(g)) {
+    e = launch_stream(g, cus, stream);
+  } else if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
   } else if (route == kRouteSkinny) {
     e = launch_skinny(g, cus, stream);
