@@ -15,7 +15,9 @@ ramp for 10-20 ms after an idle gap), then the W warm-up steps.
 
 Prints ONE JSON line: the metric (microseconds per layer), the roofline of the dominant kernel (the
 gate|up group GEMV, priced on algorithmic bytes against 8 TB/s) and the CPU baseline (the oracle's
-restatement of the reference's torch path, timed on this box's host cores on a bounded sample).
+restatement of the reference's torch path, timed on this box's host cores on a bounded sample).  Next to the
+metric: the same step with r given (the decode loop's launch structure), every group at 2 / 4 / 8 token rows, the
+prefill configuration (MFMA-bound), the GlowQ-S configuration and the whole decode loop.
 """
 from __future__ import annotations
 
@@ -59,7 +61,10 @@ SELECTIVE_GROUPS = {
     "down_proj": (17408, [5120]),
 }
 DOMINANT = "gate_up"
-DOMINANT_TRAFFIC_BYTES = 68884000  # measured, see profiles/decode_linears_llama8b_hbm_traffic.md
+# HBM bytes per launch of the dominant kernel as counted by rocprofv3 (FETCH_SIZE + WRITE_SIZE, scaled by the same
+# counters on a copy of known size): written by `python bench.py --summarize-pmc FETCH_CSV WRITE_CSV` from the counter
+# files of two profiling runs of this script, read back here for `roofline.traffic` (null when the file is missing)
+TRAFFIC_SIDECAR = os.path.join(ROOT, "profiles", "decode_gemv_gate_up_llama8b_hbm_traffic.json")
 
 
 def algorithmic_bytes(M, K, N, rank, gs=GROUP_SIZE):
@@ -278,6 +283,64 @@ def selective_leg(torch, ext, dev):
     return out
 
 
+def calibrate_copy(torch, dev, graph):
+    """Eight plain device copies of 256 MiB each from cold sources (the kernel shows up in a profile as a copy kernel):
+    262144 KiB read and 262144 KiB written per copy, the yardstick the FETCH_SIZE / WRITE_SIZE counts are scaled by."""
+    srcs = [torch.full((128 * 1024 * 1024,), float(i), dtype=torch.float16, device=dev) for i in range(8)]
+    dst = torch.empty_like(srcs[0])
+    graph.replay()  # push the sources out of the last-level cache
+    torch.cuda.synchronize()
+    for s_ in srcs:
+        dst.copy_(s_)
+    torch.cuda.synchronize()
+
+
+def summarize_pmc(fetch_csv, write_csv):
+    """Reads the per-dispatch counter files of two rocprofv3 --pmc runs of `bench.py --dominant-only --calibrate-copy`
+    (FETCH_SIZE, then WRITE_SIZE) and writes the traffic sidecar: bytes per launch of the dominant kernel, each counter
+    scaled by what it reads for the 256 MiB device copies of the same run."""
+    import csv
+
+    def averages(path, counter):
+        per = {}
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") != counter:
+                    continue
+                per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in per.items()}
+
+    out = {"kernel": None, "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py "
+                                      "--dominant-only --calibrate-copy", "copy_bytes_each_way": 256 << 20}
+    total = 0.0
+    for path, counter in ((fetch_csv, "FETCH_SIZE"), (write_csv, "WRITE_SIZE")):
+        avg = averages(path, counter)
+        copy = [k for k in avg if "copy" in k.lower()]
+        dom = [k for k in avg if "gemv_stream_kernel" in k or "gemv_wave_dot_kernel" in k]
+        if not copy or not dom:
+            raise SystemExit(f"{path}: need the copy kernel and the GEMV kernel in the counter file, found {sorted(avg)}")
+        factor = (256 << 20) / 1024.0 / avg[copy[0]]          # KiB per count
+        kib = avg[dom[0]] * factor
+        out["kernel"] = dom[0][:120]
+        out[counter] = {"count_per_launch": round(avg[dom[0]], 1), "count_per_copy": round(avg[copy[0]], 1),
+                        "KiB_per_count": round(factor, 4), "KiB_per_launch": round(kib, 1)}
+        total += kib * 1024.0
+    out["traffic_bytes_per_launch"] = int(round(total))
+    with open(TRAFFIC_SIDECAR, "w") as f:
+        json.dump(out, f, indent=1)
+        f.write("\n")
+    print(json.dumps(out))
+
+
+def read_traffic_sidecar():
+    try:
+        with open(TRAFFIC_SIDECAR) as f:
+            d = json.load(f)
+        return int(d["traffic_bytes_per_launch"]), os.path.relpath(TRAFFIC_SIDECAR, ROOT)
+    except (OSError, ValueError, KeyError):
+        return None, None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -287,6 +350,10 @@ def main():
     ap.add_argument("--prefill-only", action="store_true", help="run only the prefill leg and print it (profiling runs)")
     ap.add_argument("--selective-only", action="store_true", help="run only the GlowQ-S leg and print it")
     ap.add_argument("--no-decode-loop", action="store_true", help="skip the full decode loop leg (profiling runs)")
+    ap.add_argument("--dominant-only", action="store_true",
+                    help="run only the graph of the dominant kernel (32 launches per replay) and print its timing (profiling runs)")
+    ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter files of two --pmc runs into the traffic sidecar under profiles/")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain device copies of known size (256 MiB read + 256 MiB written each) so that "
                          "FETCH_SIZE / WRITE_SIZE counters of a profiling run can be scaled")
@@ -294,6 +361,9 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU execution (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if args.summarize_pmc:
+        summarize_pmc(*args.summarize_pmc)
+        return
 
     import torch
     from glowq_amd.kernels import load_w4a16_extension
@@ -313,33 +383,51 @@ def main():
         print(json.dumps({"selective": selective_leg(torch, ext, dev)}))
         return
 
+    from glowq_amd.kernels import PreparedGroup
+
     layers = [make_layer(torch, dev, 100 + i) for i in range(LAYERS)]
     g = torch.Generator(device=dev).manual_seed(1)
     xs = {name: torch.randn(M_TOKENS, K, device=dev, generator=g).half() for name, (K, _) in GROUPS.items()}
     rbuf = torch.empty(M_TOKENS, RANK, dtype=torch.float16, device=dev)
     outs = {name: [torch.empty(M_TOKENS, N, dtype=torch.float16, device=dev) for N in Ns] for name, (_, Ns) in GROUPS.items()}
-
-    def run_group(layer, name):
-        members, R = layer[name]
-        # one call: r = x R^T is left in rbuf by the projection launch, the group launch consumes it
-        ext.group_forward(xs[name], rbuf, members, GROUP_SIZE, 1.0, outs=outs[name], R=R)
-
-    def step_eager():
-        for layer in layers:
-            for name in GROUPS:
-                run_group(layer, name)
-
-    # capture one step as a HIP graph (the launches go to torch's current stream = the capture stream)
+    # every group validated once, descriptors built once: a call is one library call
+    calls = [{name: PreparedGroup(ext, layer[name][0], GROUPS[name][0], GROUP_SIZE, 1.0, R=layer[name][1]) for name in GROUPS}
+             for layer in layers]
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        step_eager()
-        torch.cuda.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-            step_eager()
-    torch.cuda.synchronize()
 
+    def capture(run):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            run()  # outside the capture first: kernel attributes of the routes these shapes take
+            torch.cuda.synchronize()
+            with torch.cuda.graph(gr, stream=side):
+                run()
+        torch.cuda.synchronize()
+        return gr
+
+    def run_group(li, name, project=True, x=None, r=None, o=None):
+        # project: one call = the shared-projection launch (r = x R^T left in the r buffer) + the fused group launch;
+        # otherwise the group launch alone on an r that is already there (what a decode loop does, whose glue kernels
+        # produce r together with x)
+        calls[li][name].run(xs[name] if x is None else x, r=rbuf if r is None else r, outs=outs[name] if o is None else o,
+                            project=project)
+
+    # dominant kernel: the gate|up group launch alone (r given), 32 layers of distinct weights back to back in one
+    # graph, HIP events around the replays on the launch stream
+    K_d, Ns_d = GROUPS[DOMINANT]
+    # the group kernel's own bytes: the group total minus R, which the projection launch reads
+    dom_bytes = algorithmic_bytes(M_TOKENS, K_d, sum(Ns_d), RANK) - 2 * RANK * K_d
+    gdom = capture(lambda: [run_group(li, DOMINANT, project=False) for li in range(LAYERS)])
+    if args.dominant_only:
+        dom_us = timed_replays(torch, gdom, max(10, min(args.steps, 50))) * 1e3 / LAYERS
+        if args.calibrate_copy:
+            calibrate_copy(torch, dev, gdom)
+        print(json.dumps({"dominant_kernel_us": round(dom_us, 3), "GBps": round(dom_bytes / dom_us / 1e3, 1),
+                          "algorithmic_bytes_per_launch": dom_bytes}))
+        return
+
+    graph = capture(lambda: [run_group(li, name) for li in range(LAYERS) for name in GROUPS])
     settle(torch, graph)  # clock ramp after the idle gap of the capture, before the warm-up steps
     for _ in range(args.warmup):
         graph.replay()
@@ -358,68 +446,52 @@ def main():
     us_per_layer = ms_per_step * 1e3 / LAYERS
     gbps = bytes_layer / (us_per_layer * 1e-6) / 1e9
 
-    # dominant kernel: the gate|up group launch alone, 32 layers of
-    # distinct weights back to back in one graph, HIP events around the replays on the launch stream
-    K_d, Ns_d = GROUPS[DOMINANT]
-    # the group kernel's own bytes: the group total minus R, which the projection launch reads
-    dom_bytes = algorithmic_bytes(M_TOKENS, K_d, sum(Ns_d), RANK) - 2 * RANK * K_d
-    gdom = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        with torch.cuda.graph(gdom, stream=side):
-            for layer in layers:
-                ext.group_forward(xs[DOMINANT], rbuf, layer[DOMINANT][0], GROUP_SIZE, 1.0, outs=outs[DOMINANT])
-    torch.cuda.synchronize()
     dom_us = timed_replays(torch, gdom, max(10, min(args.steps, 50))) * 1e3 / LAYERS
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+
+    # the same step with r given: 4 group launches per layer, the structure of the decode loop (its glue kernels produce
+    # r together with the activations); the bytes of R belong to those kernels and are left out of this figure's bytes
+    g_given = capture(lambda: [run_group(li, name, project=False) for li in range(LAYERS) for name in GROUPS])
+    given_us = timed_replays(torch, g_given, max(10, min(args.steps, 50))) * 1e3 / LAYERS
+    given_bytes = sum(algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK) - 2 * RANK * K for K, Ns in GROUPS.values())
 
     # per-group split of the step, from graphs of one group kind each (reported, not the metric)
     per_group = {}
     for name in GROUPS:
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(gr, stream=side):
-                for layer in layers:
-                    run_group(layer, name)
-        torch.cuda.synchronize()
-        us = timed_replays(torch, gr, 10) * 1e3 / LAYERS
         K, Ns = GROUPS[name]
         by = algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK)
-        per_group[name] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+        us = timed_replays(torch, capture(lambda: [run_group(li, name) for li in range(LAYERS)]), 10) * 1e3 / LAYERS
+        us_g = timed_replays(torch, capture(lambda: [run_group(li, name, project=False) for li in range(LAYERS)]), 10) * 1e3 / LAYERS
+        per_group[name] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                           "group_launch_only_us": round(us_g, 3),
+                           "group_launch_only_pct_hbm_peak": round((by - 2 * RANK * K) / us_g / 1e3 / HBM_PEAK_GBPS * 100, 2)}
 
-    # the same layers at more token rows per call (batched decode): reported next to the metric, not part of it;
-    # 8 layers of distinct weights (1 GB) per replay keep the last-level cache out of the picture
-    batched = {}
+    # the same layers at more token rows per call (the batch sizes of the configuration, then 16 and 64): projection +
+    # group launch per group as in the step; 8 layers of distinct weights (1 GB) per replay keep the last-level cache
+    # out of the picture.  Fractions are algorithmic bytes at that row count over the time, against the HBM peak.
+    batched, batched_groups = {}, {}
     for rows in (2, 4, 8, 16, 64):
         xb = {name: torch.randn(rows, K, device=dev, generator=g).half() for name, (K, _) in GROUPS.items()}
         rb = torch.empty(rows, RANK, dtype=torch.float16, device=dev)
         ob = {name: [torch.empty(rows, N, dtype=torch.float16, device=dev) for N in Ns] for name, (_, Ns) in GROUPS.items()}
-        gb = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            for name in GROUPS:  # outside the capture first: kernel attributes of the routes these shapes take
-                ext.group_forward(xb[name], rb, layers[0][name][0], GROUP_SIZE, 1.0, outs=ob[name], R=layers[0][name][1])
-            torch.cuda.synchronize()
-            with torch.cuda.graph(gb, stream=side):
-                for layer in layers[:8]:
-                    for name in GROUPS:
-                        ext.group_forward(xb[name], rb, layer[name][0], GROUP_SIZE, 1.0, outs=ob[name], R=layer[name][1])
-        torch.cuda.synchronize()
+        gb = capture(lambda: [run_group(li, name, x=xb[name], r=rb, o=ob[name]) for li in range(8) for name in GROUPS])
         batched[str(rows)] = round(timed_replays(torch, gb, 10) * 1e3 / 8, 2)
+        if rows <= 8:
+            entry = {}
+            for name, (K, Ns) in GROUPS.items():
+                gg = capture(lambda: [run_group(li, name, x=xb[name], r=rb, o=ob[name]) for li in range(8)])
+                us = timed_replays(torch, gg, 10) * 1e3 / 8
+                by = algorithmic_bytes(rows, K, sum(Ns), RANK)
+                entry[name] = {"us": round(us, 2), "route": ext.route(rows, K, sum(Ns), GROUP_SIZE),
+                               "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+            batched_groups[str(rows)] = entry
 
     prefill = prefill_leg(torch, ext, dev)
 
     if args.calibrate_copy:
-        # cold sources: 8 distinct 256 MiB buffers, each copied once (the kernel shows up in a profile as
-        # torch's elementwise copy kernel with 134217728 elements)
-        srcs = [torch.full((128 * 1024 * 1024,), float(i), dtype=torch.float16, device=dev) for i in range(8)]
-        dst = torch.empty_like(srcs[0])
-        graph.replay()  # push the sources out of the last-level cache
-        torch.cuda.synchronize()
-        for s_ in srcs:
-            dst.copy_(s_)
-        torch.cuda.synchronize()
-        del srcs, dst
+        calibrate_copy(torch, dev, graph)
 
-    del layers, graph, gdom
+    del layers, calls, graph, gdom, g_given
     torch.cuda.empty_cache()
     selective = selective_leg(torch, ext, dev)
     # the whole decode loop of the same benchmark (32-layer random-init model, 512-token prompt, 256 new tokens, greedy)
@@ -431,6 +503,7 @@ def main():
         with contextlib.redirect_stdout(sys.stderr):  # the patcher reports what it wrapped; stdout carries the JSON line only
             decode = decode_loop.measure(32, 512, 256)
 
+    traffic, traffic_source = read_traffic_sidecar()
     result = {
         "metric": "W4A16+GlowQ decode linears, microseconds per layer (Llama-3.1-8B shape, batch 1)",
         "value": round(us_per_layer, 3),
@@ -450,29 +523,43 @@ def main():
                         "down 4096x14336), int4 g=128 asym, shared rank-128 correction, batch tokens 1, 32 layers of distinct weights",
             "tokens": M_TOKENS, "rank": RANK, "group_size": GROUP_SIZE, "layers": LAYERS,
             "launches_per_step": 2 * len(GROUPS) * LAYERS, "execution": "HIP graph replay",
+            "structure": "per group one library call = shared-projection launch (r = x R^T) + fused group launch; the "
+                         "figure under r_given is the same step with the 4 group launches alone",
         },
         "hbm_GBps": round(gbps, 1),
         "pct_hbm_peak": round(gbps / HBM_PEAK_GBPS * 100, 2),
         "decode_tok_per_s_linears_only": round(1e3 / ms_per_step, 1),
         "algorithmic_bytes_per_layer": bytes_layer,
+        "r_given": {
+            "structure": "4 group launches per layer on an r that is already there, as in the decode loop, whose glue "
+                         "kernels (norm, attention merge, gating) produce r together with the activations",
+            "us_per_layer": round(given_us, 3), "launches_per_step": len(GROUPS) * LAYERS,
+            "algorithmic_bytes_per_layer": given_bytes,
+            "hbm_GBps": round(given_bytes / given_us / 1e3, 1),
+            "pct_hbm_peak": round(given_bytes / given_us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+        },
         "per_group": per_group,
         "batched_rows_us_per_layer": batched,
+        "batched_rows_per_group": batched_groups,
         "prefill": prefill,
         "selective": selective,
         "decode_loop": decode,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_wave_dot_kernel (gate|up group, N=28672, K=4096, M=1, rank 128)",
+            "kernel": "gemv_stream_kernel (gate|up group launch, N=28672, K=4096, M=1, rank 128, r given)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "avg_launch_us": round(dom_us, 3),
             "algorithmic_bytes_per_launch": dom_bytes,
-            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by the
-            # same counters on a 256 MiB copy (x1.9998 / x1.0): profiles/decode_linears_llama8b_hbm_traffic.md
-            "traffic": DOMINANT_TRAFFIC_BYTES,
+            # the same group with its projection launch: all of the group's bytes over the time of both launches
+            "frac_with_projection_launch": round(per_group[DOMINANT]["pct_hbm_peak"] / 100, 4),
+            # HBM bytes per launch counted by rocprofv3 (FETCH_SIZE + WRITE_SIZE scaled on a copy of known size) in an
+            # earlier profiling run of this script: read from the file named next to it, null without that file
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
     if not args.no_cpu_baseline:

@@ -27,7 +27,8 @@ from typing import Dict, List, Optional
 import torch
 import torch.nn as nn
 
-from .linear import CudaW4A16Linear, _get_kernel_out_dtype
+from . import kernels as _kernels
+from .linear import KNOBS, CudaW4A16Linear, refresh_env_knobs
 
 _LEADER_USES = {"q": 2, "gate": 1}  # followers that will consume what the leader cached
 
@@ -125,18 +126,35 @@ class AddSVDCorrection(nn.Module):
                 and self._same_right_factor(lead))
 
     # -- execution ------------------------------------------------------------------------------------
-    def _run(self, ext, x2d, r, wrappers):
+    def _apply(self, fn, *args, **kwargs):
+        self.__dict__.pop("_prepared_groups", None)  # descriptors hold the addresses of A_q / B_q
+        _kernels.bump_generation()
+        return super()._apply(fn, *args, **kwargs)
+
+    def _prepared(self, ext, wrappers, corrected: bool):
+        """The launch description of `wrappers` (this one first) with this wrapper's right factor: members validated,
+        descriptors and side streams built once and kept until a tensor moves or a factor is replaced."""
+        key = (tuple(id(w) for w in wrappers), float(self.alpha_svd), corrected)
+        cache = self.__dict__.setdefault("_prepared_groups", {})
+        hit = cache.get(key)
+        ptrs = (self.A_q.data_ptr(), self.B_q.data_ptr())
+        if hit is not None and hit[0] == ptrs and hit[1].generation == _kernels.generation():
+            return hit[1]
         members = []
         for w in wrappers:
-            m = w.inner._member(w.A_q if r is not None else None)
+            m = w.inner._member(w.A_q if corrected else None)
             m["bias"] = w.inner.bias.data if w.inner.bias is not None else None
             members.append(m)
-        return ext.group_forward(x2d, r, members, self.inner.group_size, float(self.alpha_svd))
+        pg = _kernels.PreparedGroup(ext, members, self.inner.in_features, self.inner.group_size,
+                                    float(self.alpha_svd) if corrected else 0.0, R=self.B_q if corrected else None)
+        if len(cache) >= 4:
+            cache.clear()
+        cache[key] = (ptrs, pg)
+        return pg
 
     def _finish(self, y2d: torch.Tensor, lead_shape) -> torch.Tensor:
-        out_dtype = _get_kernel_out_dtype()
-        if y2d.dtype != out_dtype:
-            y2d = y2d.to(out_dtype)
+        if y2d.dtype != KNOBS.out_dtype:
+            y2d = y2d.to(KNOBS.out_dtype)
         return y2d.reshape(*lead_shape, self.inner.out_features)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -164,23 +182,31 @@ class AddSVDCorrection(nn.Module):
                 y = cache.take_output(self)
                 if y is not None:
                     return self._finish(y, lead_shape)
-            if not (ok and same_x and r is not None):
-                r = ext.shared_proj(x2d, self.B_q)
-            return self._finish(self._run(ext, x2d, r, [self])[0], lead_shape)
+            pg = self._prepared(ext, [self], True)
+            if ok and same_x and r is not None:
+                return self._finish(pg.run(x2d, r=r, project=False)[0], lead_shape)
+            return self._finish(pg.run(x2d)[0], lead_shape)  # the reference's recompute-on-miss: r from this module's own R
 
-        r = ext.shared_proj(x2d, self.B_q)
         if cache is not None and self.role in _LEADER_USES:
-            followers = [w for w in cache.members if w is not self and w._fusable_with(self)]
-            group = [self] + followers[: ext_max_members() - 1]
-            outs = self._run(ext, x2d, r, group)
+            # who joins the leader's launch is decided once per state of the group (members, their alpha switches,
+            # tensors not moved since), not on every call
+            state = (_kernels.generation(), tuple((id(w), w.alpha_svd) for w in cache.members), self.B_q.data_ptr())
+            memo = self.__dict__.get("_group_memo")
+            if memo is None or memo[0] != state:
+                followers = [w for w in cache.members if w is not self and w._fusable_with(self)]
+                memo = (state, [self] + followers[: ext_max_members() - 1])
+                self.__dict__["_group_memo"] = memo
+            group = memo[1]
+            pg = self._prepared(ext, group, True)
+            outs = pg.run(x2d)  # r = x R^T and every member of the group in one call
             cache.clear()
-            cache.set(r, _LEADER_USES[self.role])
+            cache.set(pg.last_r, _LEADER_USES[self.role])
             cache.x_key = _x_key(x2d)
             cache.x_hold = x2d
             for w, y in zip(group[1:], outs[1:]):
                 cache.outputs[id(w)] = y
             return self._finish(outs[0], lead_shape)
-        return self._finish(self._run(ext, x2d, r, [self])[0], lead_shape)
+        return self._finish(self._prepared(ext, [self], True).run(x2d)[0], lead_shape)
 
 
 def ext_max_members() -> int:
@@ -280,6 +306,7 @@ def _configure_cuda_w4a16_env(args) -> None:
     if getattr(args, "cuda_w4a16_force_gemv", False):
         env["W4A16_FORCE_GEMV"] = "1"
         env.pop("W4A16_FORCE_GEMM", None)
+    refresh_env_knobs()  # the modules read the switches from a cache, not from the environment on every call
     print("[CUDA W4A16] env:"
           f" out_dtype={env.get('W4A16_KERNEL_OUT_DTYPE')}"
           f", gemv_m_max={env.get('W4A16_GEMV_M_MAX', '(default)')}"

@@ -7,6 +7,7 @@
 #include <cstring>
 
 #include "common.hpp"
+#include "side_stream.hpp"
 
 namespace glowq {
 // gemv.hip
@@ -26,6 +27,7 @@ hipError_t launch_dequant(const int32_t*, const half_t*, const int32_t*, half_t*
                           hipStream_t);
 hipError_t launch_unpack(const int32_t*, uint8_t*, int, int, int, int, hipStream_t);
 hipError_t launch_shared_proj_small(const half_t*, const half_t*, half_t*, int, int, int, hipStream_t);
+hipError_t launch_pack_side(const half_t*, const int32_t*, const half_t*, void*, int, int, int, int, int, int, int, hipStream_t);
 // skinny.hip / gemm.hip
 bool skinny_supported(const GroupDev& g);
 bool skinny_group_form(const GroupDev& g);
@@ -187,6 +189,8 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
   d.L = static_cast<const half_t*>(s.L);
   d.bias = static_cast<const half_t*>(s.bias);
   d.y = static_cast<half_t*>(s.y);
+  d.side = aligned16(s.side) ? static_cast<const unsigned char*>(s.side) : nullptr;
+  d.side_rank = s.side_rank;
   d.N = s.N;
   d.ldw = s.ldw_i32;
   d.lds = s.lds;
@@ -238,6 +242,11 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     g.R = nullptr;
   }
   static const int use_stream = env_or("GLOWQ_STREAM", 1);
+  // side streams are used only where every member brings one packed for the rank this launch applies
+  bool packed = true;
+  for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr && g.mem[i].side_rank == (g.r ? g.rank : 0);
+  if (!packed)
+    for (int i = 0; i < g.n_members; ++i) g.mem[i].side = nullptr;
   if (route == kRouteWaveDot && g.M == 1 && use_stream != 0 && stream_supported(g)) {
     e = launch_stream(g, cus, stream);
   } else if (route == kRouteGemm) {
@@ -300,7 +309,7 @@ int forward_single(const void* x, const int32_t* qweight, const void* scales, co
 
 extern "C" {
 
-int glowq_version(void) { return 100; }
+int glowq_version(void) { return 101; }
 
 const char* glowq_last_error(void) { return g_err; }
 
@@ -329,6 +338,27 @@ int glowq_w4a16_dequant(const int32_t* qweight, const void* scales, const int32_
   hipError_t e = launch_dequant(qweight, static_cast<const half_t*>(scales), qzeros, static_cast<half_t*>(out), N, K,
                                 group_size, ldw_i32, lds, ldz_i32, num_cus(), static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "dequant launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+size_t glowq_side_bytes(int N, int K, int group_size, int rank) {
+  SideLayout lay;
+  if (N <= 0 || !side_layout(K, group_size, rank, lay)) return 0;
+  return (size_t)((N + 1) >> 1) * side_block_bytes(lay);
+}
+
+int glowq_pack_side(const void* scales, const int32_t* qzeros, const void* L, void* side, int N, int K, int group_size,
+                    int rank, int lds, int ldz_i32, void* stream) {
+  if (!scales || !qzeros || !side) return fail(GLOWQ_EINVAL, "pack_side: NULL pointer");
+  if (glowq_side_bytes(N, K, group_size, rank) == 0)
+    return fail(GLOWQ_EUNSUPPORTED, "pack_side: no side stream for N=%d K=%d group_size=%d rank=%d", N, K, group_size, rank);
+  const int groups = (K + group_size - 1) / group_size;
+  if (lds < groups || ldz_i32 < (groups + 7) / 8) return fail(GLOWQ_ESHAPE, "pack_side: scales / qzeros rows too short");
+  if (L != nullptr && (rank <= 0 || !aligned4(L))) return fail(GLOWQ_EINVAL, "pack_side: L needs a positive rank and 4-byte alignment");
+  if (!aligned16(side)) return fail(GLOWQ_EINVAL, "pack_side: side must be 16-byte aligned");
+  hipError_t e = launch_pack_side(static_cast<const half_t*>(scales), qzeros, static_cast<const half_t*>(L), side, N, K,
+                                  group_size, rank, lds, ldz_i32, num_cus(), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "pack_side launch failed: %s", hipGetErrorString(e));
   return GLOWQ_OK;
 }
 

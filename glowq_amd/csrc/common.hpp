@@ -29,6 +29,8 @@ struct MemberDev {
   const half_t* L;
   const half_t* bias;
   half_t* y;
+  const unsigned char* side;  // the member's side stream (side_stream.hpp) or nullptr
+  int side_rank;              // the rank it was packed for
   int N, ldw, lds, ldz, ldy;
 };
 

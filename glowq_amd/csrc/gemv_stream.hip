@@ -18,6 +18,7 @@
 #include <utility>
 
 #include "common.hpp"
+#include "side_stream.hpp"
 
 namespace glowq {
 
@@ -58,6 +59,17 @@ __device__ __forceinline__ uint32_t ld_b32_nt(const void* sbase, uint32_t voff) 
   asm volatile("global_load_dword %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
   return v;
 }
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+__device__ __forceinline__ u32x2 ld_b64_nt(const void* sbase, uint32_t voff) {
+  u32x2 v;
+  asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+  return v;
+}
+__device__ __forceinline__ u32x3 ld_b96_nt(const void* sbase, uint32_t voff) {
+  u32x3 v;
+  asm volatile("global_load_dwordx3 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+  return v;
+}
 __device__ __forceinline__ uint32_t ld_u16_nt(const void* sbase, uint32_t voff) {
   uint32_t v;
   asm volatile("global_load_ushort %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
@@ -83,6 +95,16 @@ __device__ __forceinline__ void wait_vm(uint32_t& a) {
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(kN) : "memory");
 }
 template <int kN>
+__device__ __forceinline__ void wait_vm(u32x2& a) {
+  static_assert(kN >= 0 && kN <= 63, "vmcnt is a 6-bit field");
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(kN) : "memory");
+}
+template <int kN>
+__device__ __forceinline__ void wait_vm(u32x3& a) {
+  static_assert(kN >= 0 && kN <= 63, "vmcnt is a 6-bit field");
+  asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(kN) : "memory");
+}
+template <int kN>
 __device__ __forceinline__ void wait_vm(u32x4& a) {
   static_assert(kN >= 0 && kN <= 63, "vmcnt is a 6-bit field");
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(kN) : "memory");
@@ -97,21 +119,40 @@ __device__ __forceinline__ void dot_word2(uint32_t w, const h8& xq, float& accA,
   accB = __builtin_amdgcn_fdot2(bitcast_u32<h2>(hi & 0x00F000F0u), h2{xq[6], xq[7]}, accB, false);
 }
 
-// What a wave holds of one row block: kKit steps of two 16-byte units (32 codes of each row), the scale and the
-// zero-point word of one (row, group) per lane and pair of steps -- lane 32 r + i has group 32 p + i of row r for pair
-// p -- and kLW dwords of each row of L.
-template <int kKit, int kLW>
-struct Slot {
-  static constexpr int kNP = (kKit + 1) / 2;
-  u32x4 w[kKit][kSRows];
-  uint32_t sc[kNP], zw[kNP];
-  uint32_t l[kSRows][kLW > 0 ? kLW : 1];
-};
-template <int kKit, int kLW>
+// What a wave holds of one row block: kKit steps of two 16-byte units (32 codes of each row), and the side data.
+// From the canonical buffers: the scale and the zero-point word of one (row, group) per lane and pair of steps -- lane
+// 32 r + i has group gbase(p) + i of row r for pair p -- and kLW dwords of each row of L.  From a side stream
+// (side_stream.hpp) the same in kDwords = kNP + 2 kLW dwords per lane, fetched as chunks of up to four.
+template <int kSize>
+struct SideChunk;
+template <>
+struct SideChunk<1> { uint32_t v; __device__ __forceinline__ uint32_t get(int) const { return v; } };
+template <>
+struct SideChunk<2> { u32x2 v; __device__ __forceinline__ uint32_t get(int i) const { return v[i]; } };
+template <>
+struct SideChunk<3> { u32x3 v; __device__ __forceinline__ uint32_t get(int i) const { return v[i]; } };
+template <>
+struct SideChunk<4> { u32x4 v; __device__ __forceinline__ uint32_t get(int i) const { return v[i]; } };
+
+template <int kKit, int kLW, bool kPacked>
 struct SlotCounts {
   static constexpr int kNP = (kKit + 1) / 2;
-  static constexpr int kSide = 2 * kNP + kSRows * kLW;   // loads ahead of the weights of a row block
-  static constexpr int kLoads = kSide + kSRows * kKit;   // loads per row block
+  static constexpr int kDwords = kNP + kSRows * kLW;
+  static constexpr int kFull = kDwords / 4, kTail = kDwords % 4;
+  static constexpr int kSide = kPacked ? kFull + (kTail ? 1 : 0) : 2 * kNP + kSRows * kLW;  // loads ahead of the weights
+  static constexpr int kLoads = kSide + kSRows * kKit;                                     // loads per row block
+};
+template <int kKit, int kLW, bool kPacked>
+struct Slot {
+  using C = SlotCounts<kKit, kLW, kPacked>;
+  u32x4 w[kKit][kSRows];
+  // canonical buffers
+  uint32_t sc[kPacked ? 1 : C::kNP], zw[kPacked ? 1 : C::kNP];
+  uint32_t l[kSRows][(!kPacked && kLW > 0) ? kLW : 1];
+  // side stream
+  SideChunk<4> q[(kPacked && C::kFull > 0) ? C::kFull : 1];
+  SideChunk<(C::kTail ? C::kTail : 1)> tail;
+  __device__ __forceinline__ uint32_t side(int d) const { return d < 4 * C::kFull ? q[d >> 2].get(d & 3) : tail.get(d & 3); }
 };
 
 // Heavy instantiations (more than four steps in flight per wave) run with at most 8 waves per workgroup, which leaves
@@ -123,12 +164,12 @@ __host__ __device__ constexpr int stream_xw(int kit, int db) { return stream_hea
 // Registers: a row block in flight is 8 kKit + 2 kNP + 2 kLW VGPRs that must never be spilled (a spill would store them
 // before their loads have returned); the build checks that no instantiation uses scratch.  Light instantiations are
 // held to 128 VGPRs (4 waves per SIMD), heavy ones get 256.
-template <int kKit, int kLW, int kDB>
+template <int kKit, int kLW, int kDB, bool kPacked>
 __global__ __launch_bounds__(stream_heavy(kKit, kDB) ? 512 : 1024)
 __attribute__((amdgpu_waves_per_eu((stream_heavy(kKit, kDB) ? 1 : 2), (stream_heavy(kKit, kDB) ? 2 : 4))))
 void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__ r, const int K, const int rank,
                         const int group_size, const float alpha, const GroupDev g) {
-  using C = SlotCounts<kKit, kLW>;
+  using C = SlotCounts<kKit, kLW, kPacked>;
   constexpr int kNP = C::kNP;
   constexpr int kXW = stream_xw(kKit, kDB);
   static_assert(kDB * C::kLoads + 1 <= 63, "the wait for the activations counts every load behind them");
@@ -189,7 +230,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
   for (int j = 0; j < kLW; ++j) loff[j] = (uint32_t)min(lane + kWave * j, ldw_half - 1) * 4u;
 
   // ---- every load of every row block of this wave
-  Slot<kKit, kLW> slot[kDB];
+  Slot<kKit, kLW, kPacked> slot[kDB];
   bool valid[kDB];
 #pragma unroll
   for (int d = 0; d < kDB; ++d) {
@@ -205,12 +246,21 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
     const char* sc0 = reinterpret_cast<const char*>(mem.scales + (size_t)n0 * mem.lds);
     const char* zw0 = reinterpret_cast<const char*>(mem.qzeros + (size_t)n0 * mem.ldz);
     const uint32_t sc_row = two ? (uint32_t)mem.lds * 2u : 0u, zw_row = two ? (uint32_t)mem.ldz * 4u : 0u;
+    if constexpr (kPacked) {
+      const char* sb = reinterpret_cast<const char*>(mem.side) + (size_t)blk * (256 * C::kDwords);
+#pragma unroll
+      for (int c = 0; c < C::kFull; ++c) slot[d].q[c].v = ld_b128_nt(sb + 1024 * c, voff & live);
+      if constexpr (C::kTail == 1) slot[d].tail.v = ld_b32_nt(sb + 1024 * C::kFull, ((uint32_t)lane * 4u) & live);
+      if constexpr (C::kTail == 2) slot[d].tail.v = ld_b64_nt(sb + 1024 * C::kFull, ((uint32_t)lane * 8u) & live);
+      if constexpr (C::kTail == 3) slot[d].tail.v = ld_b96_nt(sb + 1024 * C::kFull, ((uint32_t)lane * 12u) & live);
+    } else {
 #pragma unroll
     for (int p = 0; p < kNP; ++p) {
       slot[d].sc[p] = ld_u16_nt(sc0, (rsel * sc_row + goff[p]) & live);
       slot[d].zw[p] = ld_b32_nt(zw0, (rsel * zw_row + zoff[p]) & live);
     }
-    if constexpr (kLW > 0) {
+    }
+    if constexpr (kLW > 0 && !kPacked) {
       // a member without L reads r itself (valid memory) and is weighted by zero
       const char* l0 = mem.L ? reinterpret_cast<const char*>(mem.L + (size_t)n0 * rank) : reinterpret_cast<const char*>(r);
       const char* l1 = (mem.L && two) ? l0 + (size_t)rank * 2 : l0;
@@ -262,7 +312,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
   static_for<kDB>([&](auto D) {
     constexpr int d = decltype(D)::value;
     if (!valid[d]) return;  // uniform; the waits of a later row block cover this one's loads as well
-    Slot<kKit, kLW>& b = slot[d];
+    Slot<kKit, kLW, kPacked>& b = slot[d];
     const int blk = first + d * stride;
     float tot[kSRows] = {0.f, 0.f};
     uint32_t rec = 0;
@@ -276,15 +326,21 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
       int u = active ? uraw : U - 1;
       if constexpr (it == 0) {
         // the side loads of a row block sit ahead of its weights: the same count covers them
+        if constexpr (kPacked) {
 #pragma unroll
-        for (int q = 0; q < kNP; ++q) {
-          wait_vm<kBehind>(b.sc[q]);
-          wait_vm<kBehind>(b.zw[q]);
-        }
+          for (int c = 0; c < C::kFull; ++c) wait_vm<kBehind>(b.q[c].v);
+          if constexpr (C::kTail > 0) wait_vm<kBehind>(b.tail.v);
+        } else {
 #pragma unroll
-        for (int j = 0; j < kLW; ++j) {
-          wait_vm<kBehind>(b.l[0][j]);
-          wait_vm<kBehind>(b.l[1][j]);
+          for (int q = 0; q < kNP; ++q) {
+            wait_vm<kBehind>(b.sc[q]);
+            wait_vm<kBehind>(b.zw[q]);
+          }
+#pragma unroll
+          for (int j = 0; j < kLW; ++j) {
+            wait_vm<kBehind>(b.l[0][j]);
+            wait_vm<kBehind>(b.l[1][j]);
+          }
         }
       }
       wait_vm<kBehind>(b.w[it][0], b.w[it][1], u);
@@ -293,7 +349,10 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
 #pragma unroll
       for (int j = 0; j < 4; ++j) xq[j] = xs[(size_t)j * U + u];
       const float sg = sig[u];
-      if constexpr ((it & 1) == 0) rec = (b.sc[p] & 0xFFFFu) | (nibble(b.zw[p], (int)(sgrp[p] & 7u)) << 16);
+      if constexpr ((it & 1) == 0) {
+        if constexpr (kPacked) rec = b.side(p);
+        else rec = (b.sc[p] & 0xFFFFu) | (nibble(b.zw[p], (int)(sgrp[p] & 7u)) << 16);
+      }
       float sc[kSRows], zp[kSRows];
       const int grel = grp - ((128 * p) >> upg_shift);
 #pragma unroll
@@ -321,7 +380,8 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
           const h2 rv = reinterpret_cast<const h2*>(rs)[min(idx, ldw_half - 1)];
 #pragma unroll
           for (int rr = 0; rr < kSRows; ++rr)
-            tot[rr] = __builtin_fmaf(a, __builtin_amdgcn_fdot2(bitcast_u32<h2>(b.l[rr][j]), rv, 0.f, false), tot[rr]);
+            tot[rr] = __builtin_fmaf(a, __builtin_amdgcn_fdot2(bitcast_u32<h2>(kPacked ? b.side(kNP + kSRows * j + rr) : b.l[rr][j]),
+                                                               rv, 0.f, false), tot[rr]);
         }
       }
     });
@@ -378,12 +438,12 @@ bool stream_supported(const GroupDev& g) {
 
 namespace {
 
-template <int kKit, int kLW, int kDB>
-hipError_t launch_stream_t(GroupDev& g, int waves, hipStream_t stream) {
-  if constexpr (kDB * SlotCounts<kKit, kLW>::kLoads + 1 > 63 || (kKit == 9 && kLW > 0)) {
+template <int kKit, int kLW, int kDB, bool kPacked>
+hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
+  if constexpr (kDB * SlotCounts<kKit, kLW, kPacked>::kLoads + 1 > 63 || (kKit == 9 && kLW > 0)) {
     return hipErrorInvalidValue;  // (nine steps with a correction do not fit the register file without spilling)
   } else {
-    auto kern = gemv_stream_kernel<kKit, kLW, kDB>;
+    auto kern = gemv_stream_kernel<kKit, kLW, kDB, kPacked>;
     const size_t lds = wave_dot_lds_bytes(1, g.K, g.rank, g.r != nullptr);
     static LdsLimit lds_limit;
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
@@ -399,6 +459,14 @@ hipError_t launch_stream_t(GroupDev& g, int waves, hipStream_t stream) {
                        g.alpha, g);
     return hipGetLastError();
   }
+}
+
+template <int kKit, int kLW, int kDB>
+hipError_t launch_stream_t(GroupDev& g, int waves, hipStream_t stream) {
+  bool packed = true;
+  for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr;
+  if (packed) return launch_stream_p<kKit, kLW, kDB, true>(g, waves, stream);
+  return launch_stream_p<kKit, kLW, kDB, false>(g, waves, stream);
 }
 
 template <int kKit, int kLW>

@@ -3,6 +3,7 @@
 #include <cstdlib>
 
 #include "common.hpp"
+#include "side_stream.hpp"
 
 namespace glowq {
 
@@ -42,6 +43,33 @@ __global__ __launch_bounds__(256) void unpack_kernel(const int32_t* __restrict__
     const int rrow = (int)(idx / total_vals);
     const int k = (int)(idx - (long)rrow * total_vals);
     codes[idx] = (uint8_t)nibble((uint32_t)packed[(size_t)rrow * ld + (k >> 3)], k & 7);
+  }
+}
+
+// Writes a member's side stream (side_stream.hpp) from its canonical buffers: one thread per (row block, lane, dword).
+__global__ __launch_bounds__(256) void pack_side_kernel(const half_t* __restrict__ scales, const int32_t* __restrict__ qzeros,
+                                                        const uint32_t* __restrict__ L, unsigned char* __restrict__ out,
+                                                        int N, int rank, int lds, int ldz, SideLayout lay) {
+  const int blocks = (N + 1) >> 1;
+  const long total = (long)blocks * 64 * lay.dwords;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int d = (int)(idx % lay.dwords);
+    const int lane = (int)((idx / lay.dwords) & 63);
+    const int b = (int)(idx / ((long)lay.dwords * 64));
+    uint32_t val = 0;
+    if (d < lay.np) {
+      const int row = 2 * b + (lane >> 5);
+      int g = side_gbase(lay, d) + (lane & 31);
+      g = g < lay.groups ? g : lay.groups - 1;
+      if (row < N)
+        val = (uint32_t)__builtin_bit_cast(uint16_t, scales[(size_t)row * lds + g]) |
+              (nibble((uint32_t)qzeros[(size_t)row * ldz + (g >> 3)], g & 7) << 16);
+    } else {
+      const int j = (d - lay.np) >> 1, row = 2 * b + ((d - lay.np) & 1);
+      const int i = lane + 64 * j;
+      if (L != nullptr && row < N && i < (rank >> 1)) val = L[(size_t)row * (rank >> 1) + i];
+    }
+    *reinterpret_cast<uint32_t*>(out + (size_t)b * side_block_bytes(lay) + side_dword_offset(lay, d, lane)) = val;
   }
 }
 
@@ -169,6 +197,19 @@ hipError_t launch_unpack(const int32_t* packed, uint8_t* codes, int rows, int to
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, packed, codes, rows, total_vals, ld);
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_side(const half_t* scales, const int32_t* qzeros, const half_t* L, void* out, int N, int K,
+                            int group_size, int rank, int lds, int ldz, int num_cus, hipStream_t stream) {
+  SideLayout lay;
+  if (!side_layout(K, group_size, rank, lay)) return hipErrorInvalidValue;
+  const long total = (long)((N + 1) >> 1) * 64 * lay.dwords;
+  long blocks = (total + 255) / 256;
+  if (blocks > (long)num_cus * 16) blocks = (long)num_cus * 16;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(pack_side_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, scales, qzeros,
+                     reinterpret_cast<const uint32_t*>(L), static_cast<unsigned char*>(out), N, rank, lds, ldz, lay);
   return hipGetLastError();
 }
 

@@ -28,7 +28,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .correction import AddSVDCorrection, patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
-from .kernels import load_w4a16_extension
+from .kernels import PreparedGroup, load_w4a16_extension
 from .linear import CudaW4A16Linear, convert_to_cuda_w4a16
 
 
@@ -285,14 +285,20 @@ class FusedStep:
         R, alpha = (corrected[0] if corrected else (None, 1.0))
         shared = all(a == alpha and (B.data_ptr() == R.data_ptr() or (B.shape == R.shape and bool(torch.equal(B, R))))
                      for B, a in corrected)
+        ext = load_w4a16_extension()
+        K = mods[0].inner.in_features if isinstance(mods[0], AddSVDCorrection) else mods[0].in_features
+
+        def single(mem, Ri, ai, out):
+            return {"members": [mem], "R": Ri, "r": torch.zeros(1, Ri.size(0), **f16) if Ri is not None else None,
+                    "alpha": ai, "gs": gs, "outs": [out], "per_member": None,
+                    "call": PreparedGroup(ext, [mem], K, gs, ai if Ri is not None else 0.0, R=Ri)}
+
+        # the no-sharing comparator and artifacts with a factor pair per module: one projection and one launch per module
+        per_member = [single(mem, *(f if f is not None else (None, 1.0)), out) for mem, f, out in zip(members, factors, outs)]
         if shared:
             r = torch.zeros(1, R.size(0), **f16) if R is not None else None
-            return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs, "per_member": None}
-        per_member = []
-        for mem, f, out in zip(members, factors, outs):
-            Ri, ai = f if f is not None else (None, 1.0)
-            per_member.append({"members": [mem], "R": Ri, "r": torch.zeros(1, Ri.size(0), **f16) if Ri is not None else None,
-                               "alpha": ai, "gs": gs, "outs": [out], "per_member": None})
+            return {"members": members, "R": R, "r": r, "alpha": alpha, "gs": gs, "outs": outs, "per_member": None,
+                    "alone": per_member, "call": PreparedGroup(ext, members, K, gs, alpha if R is not None else 0.0, R=R)}
         return {"members": members, "R": None, "r": None, "alpha": 1.0, "gs": gs, "outs": outs, "per_member": per_member}
 
     def _norm(self, x, delta, ln, grp):
@@ -308,17 +314,14 @@ class FusedStep:
     def _linear(self, x, grp, r_ready=False):
         if grp["per_member"] is not None:
             for sub in grp["per_member"]:
-                self.ext.group_forward(x, sub["r"], sub["members"], sub["gs"], sub["alpha"], outs=sub["outs"], R=sub["R"])
+                sub["call"].run(x, r=sub["r"], outs=sub["outs"])
             return
         if self.share:
-            self.ext.group_forward(x, grp["r"], grp["members"], grp["gs"], grp["alpha"], outs=grp["outs"],
-                                   R=None if r_ready else grp["R"])
+            grp["call"].run(x, r=grp["r"], outs=grp["outs"], project=not r_ready)
             return
         # layer-wise correction without sharing (test/step3_1_layerwise.py:133-153): one projection and one launch per module
-        for mem, out in zip(grp["members"], grp["outs"]):
-            corrected = mem["L"] is not None
-            self.ext.group_forward(x, grp["r"] if corrected else None, [mem], grp["gs"], grp["alpha"], outs=[out],
-                                   R=grp["R"] if corrected else None)
+        for sub in grp["alone"]:
+            sub["call"].run(x, r=sub["r"], outs=sub["outs"])
 
     @torch.no_grad()
     def run(self):

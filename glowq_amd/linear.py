@@ -49,9 +49,37 @@ def _env_number(*names: str, default: int) -> int:
 
 
 def _get_kernel_out_dtype() -> torch.dtype:
-    """`W4A16_KERNEL_OUT_DTYPE` (legacy `MIXED_KERNEL_OUT_DTYPE`): fp16 or fp32, default fp32 (linear.py:29-39)."""
+    """`W4A16_KERNEL_OUT_DTYPE` (legacy `MIXED_KERNEL_OUT_DTYPE`) as the environment has it now: fp16 or fp32, default
+    fp32 (linear.py:29-39)."""
     v = os.environ.get("W4A16_KERNEL_OUT_DTYPE", os.environ.get("MIXED_KERNEL_OUT_DTYPE", "fp32")).lower()
     return torch.float16 if v in ("fp16", "float16", "half") else torch.float32
+
+
+class _Knobs:
+    """The `W4A16_*` switches a forward depends on, read from the environment ONCE (at import, and again by
+    `refresh_env_knobs()`), not on every call as the reference does (linear.py:172-177).  `_configure_cuda_w4a16_env`
+    refreshes them itself; code that edits `os.environ` by hand afterwards calls `refresh_env_knobs()`."""
+
+    __slots__ = ("out_dtype", "force_gemm", "force_gemv", "use_gemv", "split_k_iters")
+
+    def __init__(self):
+        self.read()
+
+    def read(self) -> None:
+        self.out_dtype = _get_kernel_out_dtype()
+        self.force_gemm = _env_flag("W4A16_FORCE_GEMM", "CUDA_MIXED_FORCE_GEMM")
+        self.force_gemv = _env_flag("W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV")
+        self.use_gemv = _env_flag("W4A16_USE_GEMV")
+        self.split_k_iters = _env_number("W4A16_SPLIT_K_ITERS", default=1)
+
+
+KNOBS = _Knobs()
+
+
+def refresh_env_knobs() -> None:
+    """Re-reads the `W4A16_*` environment switches (output dtype, forced routes, split-K iterations) for every module.
+    The row threshold `W4A16_GEMV_M_MAX` is read when a module is constructed, as in the reference (linear.py:120)."""
+    KNOBS.read()
 
 
 # ----------------------------------------------------------------------------------------------
@@ -127,6 +155,7 @@ class CudaW4A16Linear(nn.Module):
 
         self._ext = None
         self._gemv_threshold = _env_number("W4A16_GEMV_M_MAX", "CUDA_MIXED_GEMV_M_MAX", default=DEFAULT_GEMV_M_MAX)
+        self._prepared = None  # descriptors of the bare module for single-call forwards (kernels.PreparedGroup)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
@@ -151,11 +180,31 @@ class CudaW4A16Linear(nn.Module):
         return {"qweight": self.qweight_i32, "scales": self.scales_f16, "qzeros": self.qzeros_i32, "L": L,
                 "bias": None}
 
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() / .half() move the buffers: descriptors built from their addresses go with them
+        from .kernels import bump_generation
+
+        self._prepared = None
+        bump_generation()
+        return super()._apply(fn, *args, **kwargs)
+
+    def _bare_group(self):
+        """The module alone as a prepared group (validated once, side stream packed once); rebuilt when a buffer has
+        been replaced since."""
+        key = (self.qweight_i32.data_ptr(), self.scales_f16.data_ptr(), self.qzeros_i32.data_ptr(),
+               self.bias.data_ptr() if self.bias is not None else 0)
+        if self._prepared is None or self._prepared[0] != key:
+            from .kernels import PreparedGroup
+
+            member = self._member()
+            member["bias"] = self.bias.data if self.bias is not None else None
+            self._prepared = (key, PreparedGroup(self._get_ext(), [member], self.in_features, self.group_size, 0.0))
+        return self._prepared[1]
+
     def _prefer_gemv(self, m: int) -> bool:
-        if _env_flag("W4A16_FORCE_GEMM", "CUDA_MIXED_FORCE_GEMM"):
+        if KNOBS.force_gemm:
             return False
-        return (_env_flag("W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV") or _env_flag("W4A16_USE_GEMV")
-                or m <= self._gemv_threshold)
+        return KNOBS.force_gemv or KNOBS.use_gemv or m <= self._gemv_threshold
 
     def _require_gpu(self, x: torch.Tensor) -> None:
         if not x.is_cuda or not self.qweight_i32.is_cuda:
@@ -163,11 +212,10 @@ class CudaW4A16Linear(nn.Module):
                 "CudaW4A16Linear.forward runs only on the GPU through the glowq HIP library; "
                 "move the module and its input to the device (there is no CPU route)")
 
-    def _finish(self, out: torch.Tensor, lead_shape) -> torch.Tensor:
-        out_dtype = _get_kernel_out_dtype()
-        if out.dtype != out_dtype:
-            out = out.to(out_dtype)
-        if self.bias is not None:
+    def _finish(self, out: torch.Tensor, lead_shape, bias_applied: bool = False) -> torch.Tensor:
+        if out.dtype != KNOBS.out_dtype:
+            out = out.to(KNOBS.out_dtype)
+        if self.bias is not None and not bias_applied:
             out = out + self.bias.to(out.dtype)
         return out.reshape(*lead_shape, self.out_features)
 
@@ -175,13 +223,12 @@ class CudaW4A16Linear(nn.Module):
         lead = x.shape[:-1]
         x2d = self._as_rows(x)
         self._require_gpu(x2d)
-        ext = self._get_ext()
-        if self._prefer_gemv(x2d.size(0)):
-            out = ext.w4a16_gemv_forward_cuda(x2d, self.qweight_i32, self.scales_f16, self.qzeros_i32, self.group_size)
-        else:
-            out = ext.w4a16_gemm_forward_cuda(x2d, self.qweight_i32, self.scales_f16, self.qzeros_i32, self.group_size,
-                                              _env_number("W4A16_SPLIT_K_ITERS", default=1))
-        return self._finish(out, lead)
+        if KNOBS.force_gemm or (not self._prefer_gemv(x2d.size(0))):
+            out = self._get_ext().w4a16_gemm_forward_cuda(x2d, self.qweight_i32, self.scales_f16, self.qzeros_i32,
+                                                          self.group_size, KNOBS.split_k_iters)
+            return self._finish(out, lead)
+        # the decode kernels through descriptors validated once (the bias rides in the kernel's epilogue)
+        return self._finish(self._bare_group().run(x2d)[0], lead, bias_applied=True)
 
     def dequantize(self) -> torch.Tensor:
         """fp16 [out_features, in_features] weight, fp16((code - zero) * scale); the device twin of the
@@ -223,4 +270,4 @@ def convert_to_cuda_w4a16(model: nn.Module, group_size: int = 128) -> nn.Module:
     return model
 
 
-__all__ = ["CudaW4A16Linear", "convert_to_cuda_w4a16", "DEFAULT_GEMV_M_MAX"]
+__all__ = ["CudaW4A16Linear", "convert_to_cuda_w4a16", "refresh_env_knobs", "DEFAULT_GEMV_M_MAX"]

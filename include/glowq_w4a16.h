@@ -50,7 +50,8 @@ typedef struct glowq_member {
   int32_t lds;
   int32_t ldz_i32;
   int32_t ldy;
-  int32_t reserved;
+  int32_t side_rank;      /* the rank `side` was packed for (0: packed without a left factor) */
+  const void* side;       /* the member's side stream written by glowq_pack_side for this K and group_size, or NULL */
 } glowq_member_t;
 
 /* Library / device information. */
@@ -118,6 +119,22 @@ int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int r
 int glowq_shared_proj_ws(const void* x, const void* R, void* r, int M, int K, int rank, void* workspace,
                          size_t workspace_bytes, void* stream);
 size_t glowq_proj_workspace_bytes(int M, int K, int rank);
+
+/*
+ * Side stream of a member: its scales, zero-points and left-factor rows (L may be NULL) repacked, two output rows at a
+ * time, into the order the single-token decode GEMV consumes them in, so that a wave fetches them with one to three
+ * coalesced loads per row block instead of a small request per array and row.  A deterministic function of the
+ * canonical buffers, which stay what every other kernel reads (the reference has no counterpart: its GEMV reads
+ * scale and zero-point per thread and row, src/cuda_w4a16/csrc/gemv_w4a16.cu:96-104).  glowq_side_bytes gives the
+ * size of `side` (16-byte aligned device memory), 0 for shapes the layout does not cover (K a multiple of 32 up to
+ * 18432, power-of-two groups of 128 columns and more, even ranks up to 256).  A member whose `side` is set must have
+ * been packed for the K and group_size of the call and with the same L, and states the rank it was packed for in
+ * `side_rank`; single-token calls read it instead of scales / qzeros / L when every member of the group brings one
+ * whose rank is the rank the call applies (0 for a call without correction), and ignore it otherwise.
+ */
+size_t glowq_side_bytes(int N, int K, int group_size, int rank);
+int glowq_pack_side(const void* scales, const int32_t* qzeros, const void* L, void* side, int N, int K, int group_size,
+                    int rank, int lds, int ldz_i32, void* stream);
 
 /*
  * One launch for a whole group: for every member i

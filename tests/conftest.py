@@ -38,3 +38,14 @@ def small_m_route(request, ext):
     ext.set_tuning("quad_max_m", old)
     ext.set_tuning("quad_min_m", old_min)
     ext.set_tuning("small_group_mb", old_small)
+
+
+@pytest.fixture(autouse=True)
+def _fresh_env_knobs():
+    """The modules read the W4A16_* switches from a cache: every test starts and ends with the cache in step with the
+    environment, and a test that edits the environment re-reads it with `refresh_env_knobs()`."""
+    from glowq_amd.linear import refresh_env_knobs
+
+    refresh_env_knobs()
+    yield
+    refresh_env_knobs()

@@ -12,7 +12,7 @@ import torch.nn as nn
 import glowq_oracle as oracle
 from glowq_amd import correction as corr
 from glowq_amd import decode
-from glowq_amd.linear import CudaW4A16Linear
+from glowq_amd.linear import CudaW4A16Linear, refresh_env_knobs
 
 pytestmark = pytest.mark.gpu
 
@@ -23,6 +23,7 @@ TINY = dict(hidden=256, layers=2, heads=4, kv_heads=2, head_dim=64, intermediate
 @pytest.fixture()
 def fp16_out(monkeypatch):
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    refresh_env_knobs()
     with torch.no_grad():
         yield
 

@@ -117,3 +117,86 @@ def test_selective_members_skip_correction(ext, small_m_route):
     outs0 = ext.group_forward(dev(x), r, mem, 128, 0.0)
     plain0 = _run_single(ext, x, members[0])
     np.testing.assert_array_equal(outs0[0].cpu().numpy().view(np.uint16), plain0.view(np.uint16))
+
+
+# ---------------------------------------------------------------- side streams of the single-token GEMV
+def _unpack_side(side, N, K, gs, rank):
+    """Host reading of a side stream following its layout description (csrc/side_stream.hpp): per row block of two rows
+    and lane, np scale/zero-point dwords then 2 lw dwords of L, in lane-major chunks of four dwords."""
+    U = K // 32
+    kit = -(-U // 64)
+    np_, lw = (kit + 1) // 2, (rank + 127) // 128
+    D = np_ + 2 * lw
+    upg = (gs // 32).bit_length() - 1
+    G = -(-U // (1 << upg))
+    blocks = (N + 1) // 2
+    raw = side.cpu().numpy().view(np.uint32).reshape(blocks, 64 * D)
+    dw = np.zeros((blocks, 64, D), dtype=np.uint32)
+    for d in range(D):
+        c = d // 4
+        size = min(4, D - 4 * c)
+        for lane in range(64):
+            dw[:, lane, d] = raw[:, (1024 * c + lane * 4 * size + 4 * (d % 4)) // 4]
+    return dw, np_, lw, upg, G
+
+
+@pytest.mark.parametrize("N,K,gs,rank,with_L", [(64, 4096, 128, 128, True), (33, 4096, 128, 128, True), (40, 14336, 128, 128, True),
+                                                (24, 5120, 128, 256, True), (16, 8192, 256, 64, True), (10, 4096, 128, 0, False),
+                                                (12, 2048, 128, 128, False), (8, 17408, 128, 0, False)])
+def test_side_stream_holds_exactly_the_canonical_values(ext, N, K, gs, rank, with_L):
+    _, (m,), _ = make_group(N + K, 1, K, [N], rank if with_L else 0, group_size=gs)
+    L = dev(m["L"]) if with_L else None
+    side = ext.pack_side(dev(m["scales"]), dev(m["qzeros"]), L, K, gs, rank)
+    assert side is not None and side.numel() == ext.lib.glowq_side_bytes(N, K, gs, rank)
+    dw, np_, lw, upg, G = _unpack_side(side, N, K, gs, rank)
+    _, zeros, scales, _ = oracle.codes_and_params(m["qweight"], m["qzeros"], m["scales"], K, gs)
+    for b in range((N + 1) // 2):
+        for lane in range(64):
+            row = 2 * b + lane // 32
+            for p in range(np_):
+                g = min(((128 * p) >> upg) + lane % 32, G - 1)
+                want = (int(scales[row, g].view(np.uint16)) | (int(zeros[row, g]) << 16)) if row < N else 0
+                assert int(dw[b, lane, p]) == want, (b, lane, p)
+            for j in range(lw):
+                for rr in range(2):
+                    row, i = 2 * b + rr, lane + 64 * j
+                    want = 0
+                    if with_L and row < N and i < rank // 2:
+                        want = int(m["L"][row, 2 * i:2 * i + 2].view(np.uint32)[0])
+                    assert int(dw[b, lane, np_ + 2 * j + rr]) == want, (b, lane, j, rr)
+
+
+@pytest.mark.parametrize("K,Ns,rank", [(4096, [256, 64, 33], 128), (14336, [96], 128), (5120, [64, 64], 256), (2048, [40], 64),
+                                       (8192, [48], 0), (17408, [32], 0)])
+def test_single_token_launch_reads_the_same_values_through_side_streams(ext, K, Ns, rank):
+    print(f"case K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(3 + K + rank, 1, K, Ns, rank, with_bias=True)
+    base = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]),
+             "L": dev(m["L"]) if rank else None, "bias": dev(m["bias"])} for m in members]
+    if rank:
+        base[-1]["L"] = None                      # one member of the corrected group without its own L
+    xd = dev(x)
+    r = ext.shared_proj(xd, dev(R)) if rank else None
+    plain = ext.group_forward(xd, r, base, 128, 0.5)
+    packed = [dict(m, side=(ext.pack_side(m["scales"], m["qzeros"], m["L"], K, 128, rank), rank)) for m in base]
+    assert all(m["side"][0] is not None for m in packed)
+    with_side = ext.group_forward(xd, r, packed, 128, 0.5)
+    torch.cuda.synchronize()
+    for a, b, m in zip(plain, with_side, members):
+        assert torch.equal(a, b)
+    # and both are right
+    for y, m, bm in zip(with_side, members, base):
+        want = (oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 0.5) if bm["L"] is not None
+                else oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)) + m["bias"].astype(np.float64)[None, :]
+        assert_close(y.cpu().numpy(), want, f"side stream K={K}")
+    # a stream packed for another rank than the launch applies is ignored, not misread
+    other = rank + 2                              # neither the rank of this launch nor 0
+    wrong = [dict(m, side=(torch.full_like(p["side"][0], 0x5A), other)) for m, p in zip(base, packed)]
+    for a, b in zip(plain, ext.group_forward(xd, r, wrong, 128, 0.5)):
+        assert torch.equal(a, b)
+    # the prepared group builds its own streams and gives the same bits
+    from glowq_amd.kernels import PreparedGroup
+    pg = PreparedGroup(ext, base, K, 128, 0.5, R=dev(R) if rank else None, side_streams=True)
+    assert all(k[5] is not None for k in pg.keep)
+    for a, b in zip(plain, pg.run(xd)):
+        assert torch.equal(a, b)

@@ -28,6 +28,7 @@ def _ref(x, mod, L=None, R=None, alpha=1.0):
 @pytest.fixture()
 def fp16_out(monkeypatch):
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    linear.refresh_env_knobs()
     with torch.no_grad():  # inference path: the reference evaluates under no_grad as well
         yield
 
@@ -44,14 +45,19 @@ def test_converted_linear_forward(fp16_out, monkeypatch):
         assert_close(y.cpu().numpy().reshape(-1, 96), _ref(x.numpy().reshape(-1, 512), mod), f"linear {shape}")
     # fp32 inputs are cast; fp32 output is the reference's module default
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp32")
+    assert mod(torch.randn(4, 512).cuda()).dtype == torch.float16      # the switches are cached: not honoured yet ...
+    linear.refresh_env_knobs()
     y32 = mod(torch.randn(4, 512).cuda())
-    assert y32.dtype == torch.float32
+    assert y32.dtype == torch.float32                                   # ... but after a refresh
     # forced routes agree with each other within tolerance
     x = torch.randn(3, 512).half()
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp16")
     monkeypatch.setenv("W4A16_FORCE_GEMM", "1")
+    linear.refresh_env_knobs()
+    assert linear.KNOBS.force_gemm and not mod._prefer_gemv(1)
     yg = mod(x.cuda()).cpu().numpy()
     monkeypatch.delenv("W4A16_FORCE_GEMM")
+    linear.refresh_env_knobs()
     assert_close(yg, _ref(x.numpy(), mod), "forced gemm route")
     w = mod.dequantize().cpu().numpy()
     np.testing.assert_array_equal(w.view(np.uint16), oracle.dequant(mod.qweight_i32.cpu().numpy(), mod.qzeros_i32.cpu().numpy(),

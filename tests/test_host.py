@@ -97,9 +97,15 @@ def test_env_knobs(monkeypatch):
     m = linear.CudaW4A16Linear(64, 8, 32)
     assert m._gemv_threshold == 7 and m._prefer_gemv(7) and not m._prefer_gemv(8)
     monkeypatch.setenv("W4A16_FORCE_GEMV", "1")
+    assert not m._prefer_gemv(1000)            # forced routes are read once and again on refresh, not per call
+    linear.refresh_env_knobs()
     assert m._prefer_gemv(1000)
     monkeypatch.setenv("W4A16_FORCE_GEMM", "true")
+    linear.refresh_env_knobs()
     assert not m._prefer_gemv(1)
+    monkeypatch.setenv("W4A16_SPLIT_K_ITERS", "4")
+    linear.refresh_env_knobs()
+    assert linear.KNOBS.split_k_iters == 4 and linear.KNOBS.out_dtype == torch.float16
     monkeypatch.delenv("W4A16_GEMV_M_MAX")
     monkeypatch.setenv("CUDA_MIXED_GEMV_M_MAX", "3")  # legacy alias
     assert linear.CudaW4A16Linear(64, 8, 32)._gemv_threshold == 3
@@ -275,7 +281,8 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert set(kernels._SIGNATURES) == declared
-    assert ctypes.sizeof(kernels._Member) == 6 * 8 + 6 * 4  # matches glowq_member_t
+    assert ctypes.sizeof(kernels._Member) == 6 * 8 + 6 * 4 + 8  # matches glowq_member_t
+    assert kernels._Member.side.offset == 72 and kernels._Member.side_rank.offset == 68
 
 
 def test_abi_rejects_bad_arguments_without_a_gpu():
