@@ -103,7 +103,7 @@ int num_cus() {
 
 namespace {
 
-constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4;
+constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4, kRouteStream = 5;
 constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
 
 // Route limits, settable at run time (glowq_set_tuning) and initialised from the environment:
@@ -198,9 +198,32 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
   d.ldy = s.ldy;
 }
 
+//   stream_max_m    token rows up to which the stream GEMV (every request of a wave in flight up front) is used where it
+//                   applies; 0 switches it off (GLOWQ_STREAM_M)
+std::atomic<int> g_stream_max_m{clampi(env_or("GLOWQ_STREAM_M", 4), 0, 4)};
+//   stream_shape_rule  1: with more than one token row the stream GEMV is used only for the shapes it was measured
+//                   faster on (its dot products repeat per token row on the vector ALUs, the 4x4x4 kernel's do not);
+//                   0: for every shape up to stream_max_m rows (GLOWQ_STREAM_SHAPE_RULE)
+std::atomic<int> g_stream_shape_rule{clampi(env_or("GLOWQ_STREAM_SHAPE_RULE", 1), 0, 1)};
+
+// 8B-shape groups, group launch alone, us (stream / others): two rows q|k|v 5.9 / 7.6, o_proj 4.9 / 5.4, gate|up 15.5 /
+// 16.7, down_proj (K = 14336) 11.1 / 10.5; three rows 7.1 / 7.6, 5.6 / 7.4, 19.9 / 19.0, 13.4 / 14.3; four rows 8.1 / 7.7,
+// 6.6 / 7.4, 24.2 / 18.8, 15.7 / 14.6.
+bool stream_pays(const GroupDev& g) {
+  if (g.M <= 1 || g_stream_shape_rule.load(std::memory_order_relaxed) == 0) return true;
+  long rows = 0;
+  for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
+  const bool short_k = g.K <= 4 * 2048;
+  if (g.M == 2) return short_k;
+  if (g.M == 3) return (short_k && rows <= 8192) || (!short_k && rows <= 4096);
+  return short_k && rows <= 4096;
+}
+
 int pick_route(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
+  if (force < 0 && g.M <= g_stream_max_m.load(std::memory_order_relaxed) && stream_supported(g) && stream_pays(g))
+    return kRouteStream;
   const bool quad_rows = quad_wanted(g.M) ||
                          (g.M > 1 && g.M <= 16 && g_quad_max_m.load(std::memory_order_relaxed) > 0 && !(skinny_supported(g) && skinny_group_form(g)));
   if (force < 0 && small_group_prefers_wave_dot(g)) {
@@ -241,13 +264,12 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     g.r = g.r_out;
     g.R = nullptr;
   }
-  static const int use_stream = env_or("GLOWQ_STREAM", 1);
   // side streams are used only where every member brings one packed for the rank this launch applies
   bool packed = true;
   for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr && g.mem[i].side_rank == (g.r ? g.rank : 0);
   if (!packed)
     for (int i = 0; i < g.n_members; ++i) g.mem[i].side = nullptr;
-  if (route == kRouteWaveDot && g.M == 1 && use_stream != 0 && stream_supported(g)) {
+  if (route == kRouteStream) {
     e = launch_stream(g, cus, stream);
   } else if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
@@ -536,6 +558,8 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "quad_min_m") == 0) { slot = &g_quad_min_m; lo = 1; }
   else if (strcmp(key, "skinny_max_m") == 0) { slot = &g_skinny_max_m; hi = 64; }
   else if (strcmp(key, "small_group_mb") == 0) { slot = &g_small_group_mb; hi = 4096; }
+  else if (strcmp(key, "stream_max_m") == 0) { slot = &g_stream_max_m; hi = 4; }
+  else if (strcmp(key, "stream_shape_rule") == 0) { slot = &g_stream_shape_rule; hi = 1; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from .correction import AddSVDCorrection, patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
 from .kernels import PreparedGroup, load_w4a16_extension
-from .linear import CudaW4A16Linear, convert_to_cuda_w4a16
+from .linear import CudaW4A16Linear, convert_to_cuda_w4a16, refresh_env_knobs
 
 
 @dataclass
@@ -459,6 +459,7 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
     import os
 
     os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    refresh_env_knobs()
     cfg = DecoderConfig(layers=layers, vocab=vocab, max_len=max(1024, prompt_tokens + new_tokens + 8))
     t0 = time.perf_counter()
     model, _, _ = build_decoder(cfg, with_correction=correction)

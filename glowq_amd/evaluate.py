@@ -21,6 +21,7 @@ import torch
 import torch.nn.functional as F
 
 from .decode import Decoder, DecoderConfig, GreedyDecoder, build_decoder
+from .linear import refresh_env_knobs
 
 
 def load_local_tokens(path: str, vocab: int) -> torch.Tensor:
@@ -75,6 +76,7 @@ def main():
     ap.add_argument("--vocab", type=int, default=128256)
     args = ap.parse_args()
     os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
+    refresh_env_knobs()
     cfg = DecoderConfig(layers=args.layers, vocab=args.vocab, max_len=args.seq_len)
     model, _, _ = build_decoder(cfg)
     if args.tokens:

@@ -190,7 +190,8 @@ size_t glowq_static_scratch_bytes(void);
 
 /*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
- * 2 = tiled MFMA GEMM, 3 = generic (odd shapes), 4 = 4x4x4 matrix-core GEMV.
+ * 2 = tiled MFMA GEMM, 3 = generic (odd shapes), 4 = 4x4x4 matrix-core GEMV, 5 = stream GEMV (every request of a
+ * wave in flight up front; the default at one token row).
  */
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
 
@@ -202,8 +203,11 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * "small_group_mb": at 3..4 token rows a group whose int4 weights are smaller than this many MB goes to the
  * skinny MFMA kernel (or stays on the wave-dot GEMV) instead of the 4x4x4 GEMV, which starts up more slowly; at 2
  * rows it stays on the wave-dot GEMV and the limit is 40/17 of it; 0 = never.
+ * "stream_max_m" (0..4): token rows up to which the stream GEMV is used where its layout applies, ahead of the
+ * others; 0 switches it off.  "stream_shape_rule" (0 / 1): with more than one token row, only for the shapes it was
+ * measured faster on (1, the default) or for every shape (0).
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
- * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M and GLOWQ_SMALL_GROUP_MB.
+ * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M and GLOWQ_STREAM_SHAPE_RULE.
  */
 int glowq_set_tuning(const char* key, int value);
 

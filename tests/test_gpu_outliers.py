@@ -4,7 +4,7 @@
 On such inputs the reference's two routes differ from each other by more than the tolerance (shown on the CPU in
 tests/test_oracle.py::test_two_reference_semantics_part_on_outlier_activations), so each kernel is judged against the
 semantics it implements:
-  * wave-dot and 4x4x4 GEMV keep the dequantised weight unrounded, like the reference's GEMV kernel
+  * the stream, wave-dot and 4x4x4 GEMV keep the dequantised weight unrounded, like the reference's GEMV kernel
     (src/cuda_w4a16/csrc/gemv_w4a16.cu:96-112): yardstick `corrected_linear_exact`;
   * the skinny and the tiled MFMA kernels round the dequantised weight to fp16 once, like the reference's
     dequantise-then-matmul route (src/cuda_w4a16/csrc/gemm_w4a16.cu:46-49,132): yardstick
@@ -20,12 +20,13 @@ from helpers import ABS_TOL, REL_TOL, dev, make_group, outlier_activations
 
 pytestmark = pytest.mark.gpu
 
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv"}
 
 # (token rows, K, member widths, rank, route mode); the default limits send 1 row to the wave-dot GEMV, 2..4 rows to the
 # wave-dot GEMV, the 4x4x4 GEMV or the skinny kernel by group size, 5..64 to the skinny kernel, more to the tiled GEMM
 CASES = [
-    (1, 4096, [512, 128], 128, "default"), (1, 14336, [128], 128, "default"),
+    (1, 4096, [512, 128], 128, "default"), (1, 14336, [128], 128, "default"), (1, 4096, [512, 128], 128, "classic"),
+    (2, 4096, [4096], 128, "stream"), (3, 2048, [300], 64, "stream"), (4, 14336, [2048, 2048], 128, "stream"),
     (2, 4096, [4096], 128, "default"), (2, 14336, [8192], 128, "default"),
     (3, 2048, [300], 64, "default"), (4, 4096, [2048, 2048], 64, "default"),
     (4, 4096, [2048, 2048], 64, "quad"), (4, 4096, [2048, 2048], 64, "classic"),
@@ -42,7 +43,12 @@ def tuned(ext):
     def apply(mode):
         if mode == "default":
             return
-        for key, value in (("quad_max_m", 16 if mode == "quad" else 0), ("quad_min_m", 1), ("small_group_mb", 0)):
+        if mode == "stream":
+            saved["stream_max_m"] = ext.set_tuning("stream_max_m", 4)
+            saved["stream_shape_rule"] = ext.set_tuning("stream_shape_rule", 0)
+            return
+        for key, value in (("quad_max_m", 16 if mode == "quad" else 0), ("quad_min_m", 1), ("small_group_mb", 0),
+                           ("stream_max_m", 0)):
             saved[key] = ext.set_tuning(key, value)
 
     yield apply

@@ -301,6 +301,17 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.glowq_shared_proj(one, one, one, 0, 64, 8, None) == -1
     assert lib.glowq_w4a16_dequant(one, one, one, one, 4, 64, 32, 8, 2, 0, None) == -2
     assert ext.route(2048, 3584, 3584) == "tiled_mfma_gemm"
+    # the stream GEMV: one token row always, more rows by the measured shape rule (short K; fewer rows of output the more
+    # token rows), never past four
+    assert ext.route(1, 4096, 4096) == "stream_gemv" and ext.route(1, 14336, 4096) == "stream_gemv" and ext.route(1, 17408, 5120) == "stream_gemv"
+    assert ext.route(2, 4096, 28672) == "stream_gemv" and ext.route(2, 14336, 4096) != "stream_gemv"
+    assert ext.route(3, 4096, 6144) == "stream_gemv" and ext.route(3, 4096, 28672) != "stream_gemv"
+    assert ext.route(4, 4096, 4096) == "stream_gemv" and ext.route(4, 4096, 6144) != "stream_gemv" and ext.route(5, 4096, 4096) != "stream_gemv"
+    assert ext.route(1, 4096, 4096, group_size=64) != "stream_gemv"          # groups below 128 columns stay on the others
+    rule = ext.set_tuning("stream_shape_rule", 0)
+    assert ext.route(4, 4096, 28672) == "stream_gemv"
+    ext.set_tuning("stream_shape_rule", rule)
+    stream = ext.set_tuning("stream_max_m", 0)                                  # the routes behind it
     old = ext.set_tuning("quad_max_m", 0)
     assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096) == "skinny_mfma"
     ext.set_tuning("quad_max_m", 16)
@@ -312,6 +323,7 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     old = ext.set_tuning("small_group_mb", 0)
     assert ext.route(2, 4096, 4096) == "quad_mfma_gemv"
     ext.set_tuning("small_group_mb", old)
+    ext.set_tuning("stream_max_m", stream)
     with pytest.raises(ValueError):
         ext.set_tuning("no_such_key", 1)
     assert ext.route(1, 100, 8) == "generic"
