@@ -301,28 +301,30 @@ def summarize_pmc(fetch_csv, write_csv):
     scaled by what it reads for the 256 MiB device copies of the same run."""
     import csv
 
-    def averages(path, counter):
+    def per_kernel(path, counter):
         per = {}
         with open(path, newline="") as f:
             for row in csv.DictReader(f):
-                if row.get("Counter_Name") != counter:
-                    continue
-                per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
-        return {k: sum(v) / len(v) for k, v in per.items()}
+                if row.get("Counter_Name") == counter:
+                    per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return per
 
     out = {"kernel": None, "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py "
                                       "--dominant-only --calibrate-copy", "copy_bytes_each_way": 256 << 20}
     total = 0.0
     for path, counter in ((fetch_csv, "FETCH_SIZE"), (write_csv, "WRITE_SIZE")):
-        avg = averages(path, counter)
-        copy = [k for k in avg if "copy" in k.lower()]
-        dom = [k for k in avg if "gemv_stream_kernel" in k or "gemv_wave_dot_kernel" in k]
-        if not copy or not dom:
-            raise SystemExit(f"{path}: need the copy kernel and the GEMV kernel in the counter file, found {sorted(avg)}")
-        factor = (256 << 20) / 1024.0 / avg[copy[0]]          # KiB per count
-        kib = avg[dom[0]] * factor
+        per = per_kernel(path, counter)
+        # the 256 MiB copies are the largest dispatches of any copy kernel in the run (smaller ones move parameters)
+        copies = [v for k, vs in per.items() if "copy" in k.lower() for v in vs]
+        dom = [k for k in per if "gemv_stream_kernel" in k or "gemv_wave_dot_kernel" in k]
+        if not copies or not dom:
+            raise SystemExit(f"{path}: need the copy kernel and the GEMV kernel in the counter file, found {sorted(per)}")
+        big = [v for v in copies if v >= 0.5 * max(copies)]
+        per_copy, per_launch = sum(big) / len(big), sum(per[dom[0]]) / len(per[dom[0]])
+        factor = (256 << 20) / 1024.0 / per_copy          # KiB per count
+        kib = per_launch * factor
         out["kernel"] = dom[0][:120]
-        out[counter] = {"count_per_launch": round(avg[dom[0]], 1), "count_per_copy": round(avg[copy[0]], 1),
+        out[counter] = {"count_per_launch": round(per_launch, 1), "count_per_copy": round(per_copy, 1),
                         "KiB_per_count": round(factor, 4), "KiB_per_launch": round(kib, 1)}
         total += kib * 1024.0
     out["traffic_bytes_per_launch"] = int(round(total))
