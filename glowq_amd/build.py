@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libglowq_w4a16.so")
-SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_quad.hip", "skinny.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
+SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_chain.hip", "gemv_quad.hip", "skinny.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
 ARCH = "gfx950"
 
 HIPCC_FLAGS = [
@@ -42,8 +42,9 @@ def _hipcc() -> str:
 
 
 # Sources whose kernels keep loads in flight that the compiler does not track (inline assembly with hand-placed waits):
-# a register spilled there would be stored before its load has returned, so these must compile without scratch memory.
-NO_SCRATCH = {"gemv_stream.hip": "gemv_stream_kernel"}
+# a register spilled there would be stored before its load has returned, so these must compile without scratch memory,
+# and their assembly must not touch a register of a load that is still outstanding (isa_lint.py).
+NO_SCRATCH = {"gemv_stream.hip": "gemv_stream_kernel", "gemv_chain.hip": "gemv_stream_kernel"}
 
 
 def _check_no_scratch(src: str, kernel: str, remarks: str) -> None:
@@ -58,22 +59,40 @@ def _check_no_scratch(src: str, kernel: str, remarks: str) -> None:
                                    "must stay in registers")
 
 
+def _check_in_flight_registers(src: str, kernel: str, asm_dir: str) -> None:
+    """The device assembly the compile left in `asm_dir` through the lint of isa_lint.py."""
+    from .isa_lint import lint
+
+    stem = os.path.splitext(src)[0]
+    listings = [f for f in os.listdir(asm_dir) if f.startswith(stem + "-hip-amdgcn") and f.endswith(".s")]
+    if not listings:
+        raise RuntimeError(f"{src}: the compile left no device assembly to check")
+    for f in listings:
+        with open(os.path.join(asm_dir, f)) as fh:
+            found = lint(fh.read(), kernel)
+        if found:
+            raise RuntimeError(f"{src}: registers of loads in flight are touched before their wait "
+                               f"({len(found)} places), first:\n  " + "\n  ".join(found[:3]))
+
+
 def _compile(src: str, obj_dir: str, extra) -> str:
     obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     if src in NO_SCRATCH:
         cmd.insert(1, "-Rpass-analysis=kernel-resource-usage")
+        cmd.insert(1, "-save-temps=obj")  # keeps the device assembly beside the object
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     if src in NO_SCRATCH and res.returncode == 0:
         _check_no_scratch(src, NO_SCRATCH[src], res.stderr)
+        _check_in_flight_registers(src, NO_SCRATCH[src], obj_dir)
         kept, skip = [], 0
         for l in res.stderr.splitlines():  # a remark is its own line plus the source line and the caret under it
             if "-Rpass-analysis=kernel-resource-usage" in l:
                 skip = 2
             elif skip:
                 skip -= 1
-            elif "remarks generated" not in l:
+            elif "remarks generated" not in l and not l.startswith("In file included from"):
                 kept.append(l)
         res.stderr = "\n".join(kept)
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)

@@ -19,6 +19,8 @@ bool wave_dot_supported(int M, int K, int rank, bool has_r);
 // gemv_stream.hip
 bool stream_supported(const GroupDev& g);
 hipError_t launch_stream(GroupDev& g, int num_cus, hipStream_t stream);
+bool chain_combination_supported(int pro, int epi);
+hipError_t launch_stream_chained(GroupDev& g, const streamk::ChainDev& ch, int pro, int epi, hipStream_t stream);
 // gemv_quad.hip
 int quad_capacity(int M, int K, int rank, bool has_r);
 hipError_t launch_quad(GroupDev& g, int num_cus, hipStream_t stream);
@@ -331,7 +333,7 @@ int forward_single(const void* x, const int32_t* qweight, const void* scales, co
 
 extern "C" {
 
-int glowq_version(void) { return 101; }
+int glowq_version(void) { return 102; }
 
 const char* glowq_last_error(void) { return g_err; }
 
@@ -360,6 +362,68 @@ int glowq_w4a16_dequant(const int32_t* qweight, const void* scales, const int32_
   hipError_t e = launch_dequant(qweight, static_cast<const half_t*>(scales), qzeros, static_cast<half_t*>(out), N, K,
                                 group_size, ldw_i32, lds, ldz_i32, num_cus(), static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "dequant launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int glowq_w4a16_group_forward_chained(const void* x, const void* r, const glowq_member_t* members, int n_members, int K,
+                                      int group_size, int rank, float alpha, const glowq_chain_t* chain, void* stream) {
+  int rc = check_common(x, 1, K, group_size);
+  if (rc) return rc;
+  if (chain == nullptr || members == nullptr) return fail(GLOWQ_EINVAL, "chained: members and chain must not be NULL");
+  if (n_members < 1 || n_members > GLOWQ_MAX_MEMBERS) return fail(GLOWQ_EINVAL, "n_members must be 1..%d", GLOWQ_MAX_MEMBERS);
+  const int pro = chain->prologue, epi = chain->epilogue;
+  if (!chain_combination_supported(pro, epi))
+    return fail(GLOWQ_EUNSUPPORTED, "chained: prologue %d with epilogue %d is not served", pro, epi);
+  if (rank <= 0) return fail(GLOWQ_EUNSUPPORTED, "chained: needs a correction (rank > 0)");
+  if (pro == GLOWQ_CHAIN_PRO_PLAIN && r == nullptr) return fail(GLOWQ_EINVAL, "chained: the plain prologue needs r");
+  if (pro != GLOWQ_CHAIN_PRO_PLAIN && (chain->acc_in == nullptr || (reinterpret_cast<uintptr_t>(chain->acc_in) & 7u)))
+    return fail(GLOWQ_EINVAL, "chained: acc_in must be an 8-byte aligned device pointer");
+  if (pro == GLOWQ_CHAIN_PRO_NORM_ACC && (chain->norm_weight == nullptr || !aligned16(chain->norm_weight)))
+    return fail(GLOWQ_EINVAL, "chained: norm_weight must be a 16-byte aligned device pointer");
+  if (epi == GLOWQ_CHAIN_EPI_RESIDUAL && (n_members != 1 || chain->resid == nullptr || !aligned4(chain->resid)))
+    return fail(GLOWQ_EINVAL, "chained: the residual epilogue takes one member and a 4-byte aligned resid");
+  if (epi == GLOWQ_CHAIN_EPI_SWIGLU && (n_members != 2 || members[0].N != members[1].N || chain->act == nullptr))
+    return fail(GLOWQ_EINVAL, "chained: the SwiGLU epilogue takes two members of equal N and act");
+  if (chain->next_Rt != nullptr && (chain->acc_out == nullptr || (reinterpret_cast<uintptr_t>(chain->acc_out) & 7u) || !aligned4(chain->next_Rt)))
+    return fail(GLOWQ_EINVAL, "chained: next_Rt needs an 8-byte aligned acc_out and 4-byte alignment itself");
+  GroupDev g;
+  memset(&g, 0, sizeof(g));
+  g.x = static_cast<const half_t*>(x);
+  g.r = static_cast<const half_t*>(r);
+  g.n_members = n_members;
+  g.M = 1;
+  g.K = K;
+  g.group_size = group_size;
+  g.rank = rank;
+  g.alpha = alpha;
+  for (int i = 0; i < n_members; ++i) {
+    glowq_member_t m = members[i];
+    const bool y_optional = epi != GLOWQ_CHAIN_EPI_NONE && m.y == nullptr;
+    if (y_optional) m.y = const_cast<void*>(x);  // (passes the pointer check; restored below)
+    if (m.ldy == 0) m.ldy = m.N;
+    rc = check_member(m, K, group_size, i);
+    if (rc) return rc;
+    if (m.L == nullptr) return fail(GLOWQ_EUNSUPPORTED, "chained: member %d has no L", i);
+    if (y_optional) m.y = nullptr;
+    to_dev(m, g.mem[i]);
+    g.mem[i].side = nullptr;
+  }
+  if (g.r == nullptr) g.r = g.x;  // (the layout check wants an r for a corrected group; chained prologues do not read it)
+  const bool ok = fast_layout(g) && stream_supported(g);
+  if (pro != GLOWQ_CHAIN_PRO_PLAIN) g.r = nullptr;
+  if (!ok) return fail(GLOWQ_EUNSUPPORTED, "chained: shape outside the stream GEMV (K=%d, group_size=%d, rank=%d)", K, group_size, rank);
+  streamk::ChainDev ch;
+  memset(&ch, 0, sizeof(ch));
+  ch.norm_w = static_cast<const half_t*>(chain->norm_weight);
+  ch.acc_in = static_cast<const long long*>(chain->acc_in);
+  ch.resid = static_cast<half_t*>(chain->resid);
+  ch.next_w = static_cast<const half_t*>(chain->next_norm_weight);
+  ch.next_rt = static_cast<const half_t*>(chain->next_Rt);
+  ch.acc_out = static_cast<long long*>(chain->acc_out);
+  ch.act = static_cast<half_t*>(chain->act);
+  ch.eps = chain->eps;
+  hipError_t e = launch_stream_chained(g, ch, pro, epi, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "chained launch failed: %s", hipGetErrorString(e));
   return GLOWQ_OK;
 }
 

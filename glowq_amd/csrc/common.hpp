@@ -50,6 +50,26 @@ struct GroupDev {
   float alpha;
 };
 
+// Arguments of the chained single-token forms of the stream GEMV (stream_kernel.hpp).
+namespace streamk {
+constexpr int kAccCopies = GLOWQ_CHAIN_ACC_COPIES;
+constexpr int kAccStride = GLOWQ_CHAIN_ACC_STRIDE;
+constexpr int kProPlain = 0, kProAcc = 1, kProNormAcc = 2;
+constexpr int kEpiNone = 0, kEpiResidual = 1, kEpiSwiglu = 2;
+
+struct ChainDev {
+  const half_t* norm_w;     // kProNormAcc: weight of the norm in front of this group [K]
+  const long long* acc_in;  // kProAcc, kProNormAcc: accumulator the producer in front filled
+  half_t* resid;            // kEpiResidual: residual stream rows of this group's output [N], read then written
+  const half_t* next_w;     // kEpiResidual: weight of the norm that follows [N], or nullptr (all ones)
+  const half_t* next_rt;    // epilogues: right factor of the group that follows, transposed [N, rank]; nullptr: no P
+  long long* acc_out;       // with next_rt
+  half_t* act;              // kEpiSwiglu: gated activations [N]
+  float eps;                // kProNormAcc
+  float part_limit;         // epilogues: see above
+};
+}  // namespace streamk
+
 // Records the calling thread's error message (returned by glowq_last_error) and hands back `code`.
 int fail(int code, const char* fmt, ...);
 // Compute units of the current device (cached).
@@ -110,5 +130,9 @@ __device__ __forceinline__ float quad_sum(float v) {
   v += __builtin_bit_cast(float, t);
   return v;
 }
+
+// x * sigmoid(x) in fp32: one exponential and one reciprocal (the hardware approximations, about 1 ulp each: far inside
+// the fp16 rounding that follows); a full-precision division costs ten instructions more per element.
+__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 
 }  // namespace glowq

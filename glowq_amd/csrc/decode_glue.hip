@@ -21,10 +21,6 @@ __device__ __forceinline__ float block_sum(float v, float* red, int nwaves) {
   return t;
 }
 
-// x * sigmoid(x) in fp32: one exponential and one reciprocal (the hardware approximations, about 1 ulp each: far inside
-// the fp16 rounding that follows); a full-precision division costs ten instructions more per element.
-__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
-
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));

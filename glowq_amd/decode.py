@@ -28,7 +28,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .correction import AddSVDCorrection, patch_svd_correction_wrappers, patch_svd_correction_wrappers_cumulative
-from .kernels import PreparedGroup, load_w4a16_extension
+from .kernels import (CHAIN_ACC_BYTES, CHAIN_EPI_NONE, CHAIN_EPI_RESIDUAL, CHAIN_EPI_SWIGLU, CHAIN_PRO_ACC, CHAIN_PRO_NORM_ACC,
+                      CHAIN_PRO_PLAIN, PreparedGroup, load_w4a16_extension)
 from .linear import CudaW4A16Linear, convert_to_cuda_w4a16, refresh_env_knobs
 
 
@@ -218,11 +219,16 @@ def load_glowq_artifacts(shared_path: str, bmap_path: str, device="cuda"):
 
 
 class FusedStep:
-    """One decode token as a fixed chain of launches on static buffers (10 per layer), ready for HIP-graph capture.
-    Reads the quantised buffers and low-rank factors straight out of the model's modules; q|k|v and gate|up go through
-    the one-call projection + group entry point, o_proj and down_proj as solo groups."""
+    """One decode token as a fixed chain of launches on static buffers, ready for HIP-graph capture.  Reads the
+    quantised buffers and low-rank factors straight out of the model's modules.
+    With `chain` (and a model whose four groups per layer all carry a shared correction of one rank) a layer is six
+    launches -- q|k|v, attention, merge of its splits, o_proj, gate|up, down_proj -- with the norms, the residual adds,
+    the gate and every projection r = x R^T done inside the group launches on either side of them
+    (glowq_w4a16_group_forward_chained).  Otherwise nine: the same with two norm launches and a gate launch that also
+    produce the projections."""
 
-    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 4):
+    def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 4,
+                 chain: bool = True):
         cfg = model.cfg
         self.share = share  # False: every module projects x on R by itself and launches alone (the no-sharing comparator)
         self.model, self.cfg = model, cfg
@@ -261,6 +267,36 @@ class FusedStep:
                 "down": self._group([mlp.down_proj], [self.dn], f16),
             })
         self.q_view, self.k_view, self.v_view = self.qkv[0, :qd], self.qkv[0, qd:qd + kd], self.qkv[0, qd + kd:]
+        self.chained = bool(chain) and share and attention_splits > 1 and self._chainable()
+        if self.chained:
+            # the next group's right factor transposed (rows = the producing group's output rows), and one accumulator
+            # per hand-over, all cleared by one fill at the head of the step
+            n = len(self.plan)
+            self.acc = torch.zeros(n, 3, CHAIN_ACC_BYTES, dtype=torch.uint8, device=dev)
+            for i, lay in enumerate(self.plan):
+                lay["Rt_gu"] = lay["gu"]["R"].t().contiguous()
+                lay["Rt_down"] = lay["down"]["R"].t().contiguous()
+                lay["Rt_next"] = self.plan[i + 1]["qkv"]["R"].t().contiguous() if i + 1 < n else None
+                lay["ln1_next"] = self.plan[i + 1]["ln1"] if i + 1 < n else None
+
+    def _chainable(self) -> bool:
+        """Every group of every layer: one launch with a shared right factor, one rank throughout, shapes the chained
+        launch takes; o_proj and down_proj alone in their groups, gate and up of equal width."""
+        ranks = set()
+        for lay in self.plan:
+            for name in ("qkv", "o", "gu", "down"):
+                grp = lay[name]
+                if grp["per_member"] is not None or grp["R"] is None or any(m["L"] is None for m in grp["members"]):
+                    return False
+                K, gs, rank = grp["call"].K, grp["gs"], grp["R"].size(0)
+                ranks.add(rank)
+                if K % 32 or K > 9 * 2048 or gs < 128 or gs & (gs - 1) or rank % 2 or not 2 <= rank <= 256:
+                    return False
+            if len(lay["o"]["members"]) != 1 or len(lay["down"]["members"]) != 1 or len(lay["gu"]["members"]) != 2:
+                return False
+            if lay["gu"]["members"][0]["qweight"].size(0) != lay["gu"]["members"][1]["qweight"].size(0):
+                return False
+        return len(ranks) == 1
 
     @staticmethod
     def _group(mods, outs, f16):
@@ -324,7 +360,40 @@ class FusedStep:
             sub["call"].run(x, r=sub["r"], outs=sub["outs"])
 
     @torch.no_grad()
+    def _run_chained(self):
+        ext, cfg = self.ext, self.cfg
+        x = self.x  # the residual stream, updated in place by the o_proj and down_proj launches
+        self.acc.zero_()
+        for i, (lay, (ck, cv)) in enumerate(zip(self.plan, self.caches)):
+            qkv, o, gu, down = lay["qkv"], lay["o"], lay["gu"], lay["down"]
+            outs = [self.q_view, self.k_view, self.v_view]
+            if i == 0:
+                torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=self.x_alt)
+                ext.add_rmsnorm_proj(self.x_alt, None, lay["ln1"].weight, x, self.h, qkv["R"], qkv["r"], lay["ln1"].eps)
+                qkv["call"].run(self.h, r=qkv["r"], outs=qkv["outs"], project=False)
+            else:
+                qkv["call"].run_chained(x[0], CHAIN_PRO_NORM_ACC, CHAIN_EPI_NONE, outs=outs, norm_weight=lay["ln1"].weight,
+                                        eps=lay["ln1"].eps, acc_in=self.acc[i - 1, 2])
+            ext.rope_attend_split(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.partials, self.scale)
+            ext.attend_combine_proj(self.partials, self.attn, o["R"], o["r"])
+            o["call"].run_chained(self.attn[0], CHAIN_PRO_PLAIN, CHAIN_EPI_RESIDUAL, r=o["r"][0], outs=[None], resid=x[0],
+                                  next_norm_weight=lay["ln2"].weight, next_Rt=lay["Rt_gu"], acc_out=self.acc[i, 0])
+            gu["call"].run_chained(x[0], CHAIN_PRO_NORM_ACC, CHAIN_EPI_SWIGLU, outs=[None, None], norm_weight=lay["ln2"].weight,
+                                   eps=lay["ln2"].eps, acc_in=self.acc[i, 0], act=self.act[0], next_Rt=lay["Rt_down"],
+                                   acc_out=self.acc[i, 1])
+            nxt = lay["ln1_next"]
+            down["call"].run_chained(self.act[0], CHAIN_PRO_ACC, CHAIN_EPI_RESIDUAL, acc_in=self.acc[i, 1], outs=[None], resid=x[0],
+                                     next_norm_weight=nxt.weight if nxt is not None else None, next_Rt=lay["Rt_next"],
+                                     acc_out=self.acc[i, 2] if nxt is not None else None)
+        norm = self.model.model.norm
+        ext.add_rmsnorm(x, None, norm.weight, self.h, norm.eps)
+        torch.mm(self.h, self.model.lm_head.weight.t(), out=self.logits)
+        ext.argmax_advance(self.logits, self.next_tok, self.tok, self.pos)
+
+    @torch.no_grad()
     def run(self):
+        if self.chained:
+            return self._run_chained()
         ext, cfg = self.ext, self.cfg
         x = self.x
         torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=x)
@@ -362,7 +431,7 @@ class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
     def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True,
-                 attention_splits: int = 0):
+                 attention_splits: int = 0, chain: bool = True):
         self.model = model
         cfg = model.cfg
         if attention_splits <= 0:
@@ -382,7 +451,7 @@ class GreedyDecoder:
         self.use_graph = use_graph
         self.graph = None
         self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok, share,
-                               attention_splits) if fused else None
+                               attention_splits, chain) if fused else None
 
     @torch.no_grad()
     def _step(self):
@@ -453,7 +522,8 @@ class GreedyDecoder:
 
 
 def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
-            fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0) -> dict:
+            fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0,
+            chain: bool = True) -> dict:
     """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
     second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798)."""
     import os
@@ -465,7 +535,8 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
     model, _, _ = build_decoder(cfg, with_correction=correction)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits)
+    dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits, chain=chain)
+    chained = dec.fused is not None and dec.fused.chained
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (prompt_tokens,), generator=g)
     dec.generate(prompt, 4)  # warm-up (also captures the graph)
@@ -474,6 +545,8 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
         "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
                     f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + (f" + GlowQ r={cfg.rank}" if correction else ""),
         "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "graph": graph, "fused_step": fused, "group_sharing": share,
+        "chained_launches": chained,
+        "launches_per_token": (6 * cfg.layers + 6 if chained else 9 * cfg.layers + 5) if (fused and share and correction) else None,
         "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((new_tokens - 1) / decode_s, 1),
         "ms_per_token": round(decode_s * 1e3 / (new_tokens - 1), 3), "build_s": round(build_s, 1)}
 
@@ -487,13 +560,15 @@ def main():
     ap.add_argument("--no-sharing", action="store_true", help="fused step with one projection and one launch per module")
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="fused step with separate norm / gate launches (nine per layer) instead of the chained group launches (six)")
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--attention-splits", type=int, default=0,
                     help="workgroups per head in the fused step's attention (0: by the cache length)")
     args = ap.parse_args()
     print(json.dumps(measure(args.layers, args.prompt, args.new, vocab=args.vocab, graph=not args.no_graph,
                              fused=not args.module_path, share=not args.no_sharing, correction=not args.no_correction,
-                             attention_splits=args.attention_splits)))
+                             attention_splits=args.attention_splits, chain=not args.no_chain)))
 
 
 if __name__ == "__main__":

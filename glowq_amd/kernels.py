@@ -40,6 +40,18 @@ class _Member(ctypes.Structure):
     ]
 
 
+class _Chain(ctypes.Structure):
+    _fields_ = [
+        ("prologue", ctypes.c_int), ("epilogue", ctypes.c_int), ("norm_weight", _P), ("eps", ctypes.c_float),
+        ("acc_in", _P), ("resid", _P), ("next_norm_weight", _P), ("next_Rt", _P), ("acc_out", _P), ("act", _P),
+    ]
+
+
+# prologues and epilogues of the chained single-token group launch, and the size of one accumulator
+CHAIN_PRO_PLAIN, CHAIN_PRO_ACC, CHAIN_PRO_NORM_ACC = 0, 1, 2
+CHAIN_EPI_NONE, CHAIN_EPI_RESIDUAL, CHAIN_EPI_SWIGLU = 0, 1, 2
+CHAIN_ACC_BYTES = (16 * 256 + 8) * 8
+
 _SIGNATURES = {
     "glowq_version": (ctypes.c_int, []),
     "glowq_last_error": (ctypes.c_char_p, []),
@@ -60,6 +72,8 @@ _SIGNATURES = {
     "glowq_pack_side": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_w4a16_group_forward_fused": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
+    "glowq_w4a16_group_forward_chained": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, ctypes.c_float,
+                                               ctypes.POINTER(_Chain), _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
     "glowq_set_tuning": (_I, [ctypes.c_char_p, _I]),
     "glowq_add_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
@@ -559,6 +573,59 @@ class PreparedGroup:
         if rc:
             ext._raise(rc, "w4a16_group_forward")
         return outs
+
+
+    def run_chained(self, x: torch.Tensor, prologue: int, epilogue: int, *, r: Optional[torch.Tensor] = None,
+                    outs: Optional[List[Optional[torch.Tensor]]] = None, norm_weight=None, eps: float = 0.0, acc_in=None,
+                    resid=None, next_norm_weight=None, next_Rt=None, acc_out=None, act=None) -> None:
+        """One token through the chained form of the group launch (`glowq_w4a16_group_forward_chained`): `prologue` says
+        where the activations and r come from (as given / r from the accumulator `acc_in` / RMSNorm of the residual stream
+        `x` with `norm_weight`, `eps` and r from `acc_in`), `epilogue` where the outputs go (the members' `outs` / added
+        into the residual stream `resid` / gated into `act`) and, with `next_Rt` ([N, rank], the next group's right
+        factor transposed), that the projection of the result on it is added into the accumulator `acc_out`.
+        Accumulators are uint8 tensors of CHAIN_ACC_BYTES, zero before the producer runs.  `outs` may hold None for
+        members whose own output nobody reads (epilogues other than CHAIN_EPI_NONE)."""
+        _check(x.is_cuda and x.dtype == torch.float16 and x.numel() == self.K and x.is_contiguous(),
+               "inputs must be one contiguous CUDA fp16 token row [IC]")
+        _check(self.corrected, "chained: the group needs a correction")
+        keep = [x, r, norm_weight, acc_in, resid, next_norm_weight, next_Rt, acc_out, act]
+        for e, N, y in zip(self.arr, self.Ns, outs if outs is not None else [None] * len(self.Ns)):
+            if y is None:
+                _check(epilogue != CHAIN_EPI_NONE, "chained: without an epilogue every member needs an output")
+                e.y, e.ldy = None, N
+            else:
+                _check(y.dtype == torch.float16 and y.numel() == N and y.is_contiguous(), "output must be CUDA fp16 [OC]")
+                e.y, e.ldy = y.data_ptr(), N
+        for t, what in ((norm_weight, "norm_weight"), (resid, "resid"), (next_norm_weight, "next_norm_weight"), (act, "act")):
+            if t is not None:
+                ext_f16 = t.is_cuda and t.dtype == torch.float16 and t.is_contiguous()
+                _check(ext_f16, f"chained: {what} must be a contiguous CUDA fp16 tensor")
+        for t, what in ((acc_in, "acc_in"), (acc_out, "acc_out")):
+            if t is not None:
+                _check(t.is_cuda and t.is_contiguous() and t.numel() * t.element_size() >= CHAIN_ACC_BYTES,
+                       f"chained: {what} must hold CHAIN_ACC_BYTES")
+        n_total = sum(self.Ns) if epilogue != CHAIN_EPI_SWIGLU else self.Ns[0]
+        if next_Rt is not None:
+            _check(next_Rt.is_cuda and next_Rt.dtype == torch.float16 and next_Rt.is_contiguous()
+                   and tuple(next_Rt.shape) == (n_total, self.rank), "chained: next_Rt must be fp16 [N, rank] of this group's rank")
+        if resid is not None:
+            _check(resid.numel() == n_total, "chained: resid must have one entry per output row")
+        if act is not None:
+            _check(act.numel() == n_total, "chained: act must have one entry per gate row")
+        if norm_weight is not None:
+            _check(norm_weight.numel() == self.K, "chained: norm_weight must have IC entries")
+        if r is not None:
+            _check(r.dtype == torch.float16 and r.numel() == self.rank and r.is_contiguous(), "r must be fp16 [rank]")
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        ch = _Chain(int(prologue), int(epilogue), ptr(norm_weight), float(eps), ptr(acc_in), ptr(resid),
+                    ptr(next_norm_weight), ptr(next_Rt), ptr(acc_out), ptr(act))
+        with torch.cuda.device(x.device):
+            rc = self.lib.glowq_w4a16_group_forward_chained(
+                x.data_ptr(), ptr(r), self.arr, len(self.Ns), self.K, self.group_size, self.rank, self.alpha,
+                ctypes.byref(ch), self.ext._stream(x.device))
+        del keep
+        if rc:
+            self.ext._raise(rc, "w4a16_group_forward_chained")
 
 
 def library_path() -> str:

@@ -256,6 +256,56 @@ int glowq_rope_attend_split(const void* q, const void* k_new, const void* v_new,
 int glowq_attend_combine_proj(const float* partials, void* out, const void* R, void* r, int heads, int head_dim, int splits,
                               int rank, void* stream);
 
+/*
+ * ---- chained group launches (single token) --------------------------------------------------------------
+ * The work between two linears of a decoder layer -- residual add, RMSNorm or SwiGLU gate, and the projection of the
+ * result on the next group's right factor -- done inside the two group launches on either side of it, so that a
+ * layer is q|k|v, attention, merge, o_proj, gate|up, down_proj: six launches, none of them a norm, a gate or a
+ * projection.  The modules the reference runs there are Hugging Face's LlamaRMSNorm, the residual adds and LlamaMLP's
+ * act_fn(gate) * up around the wrappers' forward (src/step3_eval_dataset.py:470-511, generate loop :705-798); results
+ * agree with the separate launches above within fp16 rounding of r (the projection is taken of the unrounded norm).
+ *
+ * prologue  GLOWQ_CHAIN_PRO_PLAIN     x [K] and r [rank] as in glowq_w4a16_group_forward (r may be NULL with rank 0)
+ *           GLOWQ_CHAIN_PRO_ACC       x [K] as given, r = fp16(P) with P read from acc_in
+ *           GLOWQ_CHAIN_PRO_NORM_ACC  x is the residual stream [K]: the launch applies RMSNorm(norm_weight, eps) to it
+ *                                     itself and takes r = fp16(f P), f the norm's scalar factor
+ * epilogue  GLOWQ_CHAIN_EPI_NONE      outputs to the members' y
+ *           GLOWQ_CHAIN_EPI_RESIDUAL  one member: resid[n] = fp16(resid[n] + y[n]) in place (y itself is written only
+ *                                     if the member's y is not NULL); with next_Rt: P = next_R (next_norm_weight (.) resid)
+ *                                     added into acc_out (next_norm_weight NULL: all ones)
+ *           GLOWQ_CHAIN_EPI_SWIGLU    two members of equal N (gate, up): act[n] = fp16(fp16(silu(gate[n])) * up[n]);
+ *                                     with next_Rt: P = next_R act added into acc_out
+ * next_Rt is the next group's right factor transposed, [N_total, rank] fp16 row-major, of the same rank as this launch.
+ * An accumulator is GLOWQ_CHAIN_ACC_BYTES of device memory, 8-byte aligned, all zero when the producer starts (the
+ * caller clears it once per token, e.g. with a fill kernel; 64-bit fixed-point sums, so results do not depend on the
+ * order in which workgroups finish).  A partial sum too large for the fixed point (|.| >= 2^31 / workgroups) or NaN
+ * makes the consumer's r NaN rather than wrong.  Chained prologues and epilogues need rank > 0, L on every member and
+ * a shape the stream GEMV takes (K % 32 == 0, K <= 18432, group_size a power of two >= 128, rank even <= 256);
+ * otherwise GLOWQ_EUNSUPPORTED.
+ */
+#define GLOWQ_CHAIN_ACC_COPIES 16
+#define GLOWQ_CHAIN_ACC_STRIDE 256
+#define GLOWQ_CHAIN_ACC_BYTES ((GLOWQ_CHAIN_ACC_COPIES * GLOWQ_CHAIN_ACC_STRIDE + 8) * 8)
+#define GLOWQ_CHAIN_PRO_PLAIN 0
+#define GLOWQ_CHAIN_PRO_ACC 1
+#define GLOWQ_CHAIN_PRO_NORM_ACC 2
+#define GLOWQ_CHAIN_EPI_NONE 0
+#define GLOWQ_CHAIN_EPI_RESIDUAL 1
+#define GLOWQ_CHAIN_EPI_SWIGLU 2
+typedef struct glowq_chain_t {
+  int prologue, epilogue;
+  const void* norm_weight; /* PRO_NORM_ACC: [K] fp16 */
+  float eps;
+  const void* acc_in;      /* PRO_ACC, PRO_NORM_ACC */
+  void* resid;             /* EPI_RESIDUAL: [N] fp16, read and written */
+  const void* next_norm_weight; /* EPI_RESIDUAL: [N] fp16 or NULL */
+  const void* next_Rt;     /* epilogues: [N, rank] fp16 or NULL (no projection wanted) */
+  void* acc_out;           /* with next_Rt */
+  void* act;               /* EPI_SWIGLU: [N] fp16 */
+} glowq_chain_t;
+int glowq_w4a16_group_forward_chained(const void* x, const void* r, const glowq_member_t* members, int n_members, int K,
+                                      int group_size, int rank, float alpha, const glowq_chain_t* chain, void* stream);
+
 /* *next_token = index of the first maximum of logits[0..n); then *token = *next_token and *pos += 1 (each if non-NULL). */
 int glowq_argmax_advance(const void* logits, int n, int64_t* next_token, int64_t* token, int64_t* pos, void* stream);
 

@@ -15,6 +15,11 @@ reference checkout):
   gemm_ref             src/cuda_w4a16/csrc/gemm_w4a16.cu:76-135   (dequant to fp16, then matmul)
   shared_proj / correction / group_forward   src/step3_eval_dataset.py:470-511
   MiniGroupCacheModel  src/step3_eval_dataset.py:417-444
+  rmsnorm / swiglu / residual_add   the decoder-layer modules around the wrappers' forward.  The reference runs them
+                       through Hugging Face transformers' LlamaRMSNorm and LlamaMLP (transformers is a pip dependency
+                       of the reference, requirements.txt, not vendored); restated from their published definitions:
+                       fp32 variance, x * rsqrt(var + eps) rounded to the input dtype, then times the weight;
+                       act_fn(gate) * up with SiLU; hidden = residual + hidden in fp16.
 
 How each function is pinned (tests/test_oracle_*.py):
   * pack / unpack / quantize / dequant / the CPU forward: bit-exact against golden vectors that
@@ -25,6 +30,9 @@ How each function is pinned (tests/test_oracle_*.py):
     linear_rounded_exact rounded to fp16 is gemm_ref.
   * correction / group_forward: closed form ``z + alpha * (x R^T) L^T`` against a float64 library
     matmul; alpha = 0 identity; linearity in alpha; group == independent solo results.
+  * rmsnorm / swiglu / residual_add: against torch's own fp32 formulas (torch.nn.functional.silu, the variance written
+    out) on seeded inputs, the norm's scale invariance rmsnorm(c x) = rmsnorm(x) for eps = 0, and hand-computed
+    vectors (tests/test_oracle.py).
   * quantize on constant groups (scale underflows to 0 in fp16 -> NaN zero-point) is UNDEFINED in
     the reference; it is excluded from parity and documented as such.
 """
@@ -208,6 +216,32 @@ def corrected_linear_rounded_exact(x, qweight, qzeros, scales, group_size, R, L,
     z = linear_rounded_exact(x, qweight, qzeros, scales, group_size)
     r = _h(x).astype(np.float64) @ _h(R).astype(np.float64).T
     return z + float(alpha) * (r @ _h(L).astype(np.float64).T)
+
+
+def rmsnorm(x, weight, eps: float) -> np.ndarray:
+    """fp16(fp16(x * rsqrt(mean(x^2) + eps)) * weight) over the last axis, statistics in fp32 (LlamaRMSNorm)."""
+    x32 = _h(x).astype(np.float32)
+    var = np.mean(x32.astype(np.float64) ** 2, axis=-1, keepdims=True).astype(np.float32)
+    n = _h(x32 * (np.float32(1.0) / np.sqrt(var + np.float32(eps))))
+    return _h(n.astype(np.float32) * _h(weight).astype(np.float32))
+
+
+def rmsnorm_factor(x, eps: float) -> np.ndarray:
+    """rsqrt(mean(x^2) + eps) in float64: the one scalar per row that keeps RMSNorm from being linear."""
+    x64 = _h(x).astype(np.float64)
+    return 1.0 / np.sqrt(np.mean(x64 ** 2, axis=-1, keepdims=True) + float(eps))
+
+
+def swiglu(gate, up) -> np.ndarray:
+    """fp16(fp16(silu(gate)) * up): act_fn(gate_proj(x)) * up_proj(x) of LlamaMLP on fp16 tensors."""
+    g = _h(gate).astype(np.float64)
+    a = _h(g / (1.0 + np.exp(-g)))
+    return _h(a.astype(np.float32) * _h(up).astype(np.float32))
+
+
+def residual_add(residual, hidden) -> np.ndarray:
+    """fp16(residual + hidden): the decoder layer's residual connection on fp16 tensors."""
+    return _h(_h(residual).astype(np.float32) + _h(hidden).astype(np.float32))
 
 
 def group_forward(x, members, R, alpha: float, semantics: str = "gemv"):

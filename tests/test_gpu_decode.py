@@ -308,12 +308,14 @@ def test_split_attention_and_merge_match_single_workgroup(ext, fp16_out, pos, sp
     assert torch.equal(plain, got)
 
 
-def test_fused_step_matches_module_path(fp16_out):
+@pytest.mark.parametrize("chain", [True, False], ids=["chained", "separate_glue"])
+def test_fused_step_matches_module_path(fp16_out, chain):
     cfg = decode.DecoderConfig(**TINY)
     model, _, _ = decode.build_decoder(cfg, seed=8)
     prompt = torch.randint(0, cfg.vocab, (11,), generator=torch.Generator().manual_seed(4))
     ref = decode.GreedyDecoder(model, use_graph=False)
-    fus = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    fus = decode.GreedyDecoder(model, use_graph=False, fused=True, chain=chain)
+    assert fus.fused.chained == chain
     first = ref.prefill(prompt)
     fus.prefill(prompt)
     tok = first.clone()
@@ -328,7 +330,7 @@ def test_fused_step_matches_module_path(fp16_out):
         tok = want.argmax(-1)
     # without sharing (one projection and one launch per module) the step computes the same tokens
     alone, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True, share=False).generate(prompt, 10)
-    assert torch.equal(alone, decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)[0])
+    assert torch.equal(alone, decode.GreedyDecoder(model, use_graph=False, fused=True, chain=chain).generate(prompt, 10)[0])
     # the context split over 3 workgroups per head merges to the same logits within tolerance
     spl = decode.GreedyDecoder(model, use_graph=False, fused=True)
     spl.fused = decode.FusedStep(model, spl.caches, spl.cos, spl.sin, spl.tok, spl.pos, spl.next_tok, attention_splits=3)
@@ -341,8 +343,8 @@ def test_fused_step_matches_module_path(fp16_out):
     one.fused.run()
     assert (spl.fused.logits.float() - one.fused.logits.float()).abs().max() <= 1e-2
     # the captured fused step replays to the same tokens as the eager fused step
-    eager, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True).generate(prompt, 10)
-    graphed = decode.GreedyDecoder(model, use_graph=True, fused=True)
+    eager, _, _ = decode.GreedyDecoder(model, use_graph=False, fused=True, chain=chain).generate(prompt, 10)
+    graphed = decode.GreedyDecoder(model, use_graph=True, fused=True, chain=chain)
     for _ in range(3):
         got, _, _ = graphed.generate(prompt, 10)
         assert torch.equal(got, eager)
@@ -352,7 +354,8 @@ GEOM_8B = dict(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128, interm
                group_size=128, rank=128)
 
 
-def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out):
+@pytest.mark.parametrize("chain", [True, False], ids=["chained", "separate_glue"])
+def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out, chain):
     """Two layers of the Llama-3.1-8B geometry (hidden 4096, 32 query / 8 KV heads of 128, SwiGLU 14336, W4A16 g = 128,
     rank 128) with 512 cached positions: the fused single-token step (group launches, attention split over 4 workgroups
     per head, glue kernels that carry the projections) against the same network with every quantised module replaced
@@ -363,7 +366,8 @@ def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out):
     prompt = torch.randint(0, cfg.vocab, (512,), generator=torch.Generator().manual_seed(6))
     deq = {}
     ref = decode.GreedyDecoder(model, use_graph=False)
-    fus = decode.GreedyDecoder(model, use_graph=False, fused=True)     # reads the quantised buffers of the modules
+    fus = decode.GreedyDecoder(model, use_graph=False, fused=True, chain=chain)     # reads the quantised buffers of the modules
+    assert fus.fused.chained == chain
     bare = decode.GreedyDecoder(model, use_graph=False)
     saved = _swap_in_reference(model, with_correction=False, deq_cache=deq)
     bare.prefill(prompt)
@@ -395,7 +399,7 @@ def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out):
     pos = torch.tensor([prompt.numel()], device="cuda")
     without = model.forward_tokens(first, pos, bare.caches, bare.cos, bare.sin).float()
     _restore(saved)
-    fus2 = decode.GreedyDecoder(model, use_graph=False, fused=True)
+    fus2 = decode.GreedyDecoder(model, use_graph=False, fused=True, chain=chain)
     saved = _swap_in_reference(model, deq_cache=deq)
     fus2.prefill(prompt)
     _restore(saved)
@@ -421,6 +425,7 @@ def test_fused_step_with_a_factor_pair_per_module(fp16_out):
     ref = decode.GreedyDecoder(model, use_graph=False)
     fus = decode.GreedyDecoder(model, use_graph=False, fused=True)
     assert fus.fused.plan[0]["qkv"]["per_member"] is not None and fus.fused.plan[0]["o"]["per_member"] is None
+    assert not fus.fused.chained  # the chained launches need one shared factor per group
     first = ref.prefill(prompt)
     fus.prefill(prompt)
     pos = torch.tensor([prompt.numel()], device="cuda")

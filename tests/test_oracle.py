@@ -261,3 +261,34 @@ def test_fp16_conversions_of_c_oracle():
     vals = np.concatenate([rng.standard_normal(4000) * 10 ** rng.uniform(-8, 5, 4000), [65519.9, 65520.0, 2.0 ** -25, 2.0 ** -25 * 1.0001, 0.0]]).astype(np.float32)
     for v in vals:
         assert lib.oracle_f2h(float(v)) == int(np.array([v], dtype=np.float32).astype(np.float16).view(np.uint16)[0])
+
+
+# ---------------------------------------------------------------- decoder-layer glue restated in the oracle
+def test_rmsnorm_swiglu_residual_against_torch_and_by_hand():
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(3, 512, generator=g) * 3).half()
+    w = (1 + 0.1 * torch.randn(512, generator=g)).half()
+    # LlamaRMSNorm written out in torch: fp32 statistics, rounding to fp16 before the weight
+    x32 = x.float()
+    want = w * (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + 1e-5)).half()
+    np.testing.assert_array_equal(oracle.rmsnorm(x.numpy(), w.numpy(), 1e-5).view(np.uint16), want.numpy().view(np.uint16))
+    # by hand: (3, 4) has mean square 12.5; with weight 2 the norm is 2 * (3, 4) / sqrt(12.5)
+    got = oracle.rmsnorm(np.array([[3.0, 4.0]], np.float16), np.array([2.0, 2.0], np.float16), 0.0)
+    np.testing.assert_allclose(got.astype(np.float64), [[6 / 12.5 ** 0.5, 8 / 12.5 ** 0.5]], rtol=2e-3)
+    # scale invariance without eps, and the factor that carries the scale
+    a = oracle.rmsnorm(x.numpy(), w.numpy(), 0.0).astype(np.float64)
+    b = oracle.rmsnorm((x * 4).numpy(), w.numpy(), 0.0).astype(np.float64)
+    np.testing.assert_allclose(a, b, rtol=0, atol=0)  # a power of two scales exactly
+    f = oracle.rmsnorm_factor(x.numpy(), 1e-5)
+    np.testing.assert_allclose((x.double().numpy() * f) ** 2 @ np.ones(512) / 512, np.ones(3), rtol=1e-4)
+    # SwiGLU against torch's silu in fp32 with the fp16 rounding between the two factors
+    gate = (torch.randn(4, 256, generator=g) * 2).half()
+    up = torch.randn(4, 256, generator=g).half()
+    want = torch.nn.functional.silu(gate.float()).half() * up
+    np.testing.assert_array_equal(oracle.swiglu(gate.numpy(), up.numpy()).view(np.uint16), want.numpy().view(np.uint16))
+    assert oracle.swiglu(np.array([0.0], np.float16), np.array([7.0], np.float16))[0] == 0.0
+    np.testing.assert_allclose(float(oracle.swiglu(np.array([1.0], np.float16), np.array([1.0], np.float16))[0]), 1 / (1 + np.exp(-1.0)), rtol=1e-3)
+    # residual add: one rounding of the wide sum
+    r = torch.randn(64, generator=g).half()
+    h = torch.randn(64, generator=g).half()
+    np.testing.assert_array_equal(oracle.residual_add(r.numpy(), h.numpy()).view(np.uint16), (r + h).numpy().view(np.uint16))
