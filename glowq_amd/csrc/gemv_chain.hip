@@ -43,11 +43,12 @@ hipError_t launch_chain_i(GroupDev& g, const ChainDev& ch, int waves, hipStream_
 
 template <int kKit, int kLW>
 hipError_t launch_chain_pe(GroupDev& g, const ChainDev& ch, int pro, int epi, int waves, hipStream_t stream) {
-  // the four combinations a decoder layer uses: q|k|v, o_proj, gate|up, down_proj
+  // the combinations a decoder layer uses: q|k|v, o_proj, gate|up (behind a norm of its own or a norm launch), down_proj
   if (pro == kProNormAcc && epi == kEpiNone) return launch_chain_i<kKit, kLW, kProNormAcc, kEpiNone>(g, ch, waves, stream);
   if (pro == kProPlain && epi == kEpiResidual) return launch_chain_i<kKit, kLW, kProPlain, kEpiResidual>(g, ch, waves, stream);
   if (pro == kProNormAcc && epi == kEpiSwiglu) return launch_chain_i<kKit, kLW, kProNormAcc, kEpiSwiglu>(g, ch, waves, stream);
   if (pro == kProAcc && epi == kEpiResidual) return launch_chain_i<kKit, kLW, kProAcc, kEpiResidual>(g, ch, waves, stream);
+  if (pro == kProPlain && epi == kEpiSwiglu) return launch_chain_i<kKit, kLW, kProPlain, kEpiSwiglu>(g, ch, waves, stream);
   return hipErrorInvalidValue;
 }
 
@@ -60,9 +61,10 @@ hipError_t launch_chain_lw(GroupDev& g, const ChainDev& ch, int pro, int epi, in
 }  // namespace
 
 // The combinations served: (norm + accumulator, none), (plain, residual), (norm + accumulator, SwiGLU),
-// (accumulator, residual).
+// (plain, SwiGLU), (accumulator, residual).
 bool chain_combination_supported(int pro, int epi) {
-  return (pro == kProNormAcc && (epi == kEpiNone || epi == kEpiSwiglu)) || (epi == kEpiResidual && (pro == kProPlain || pro == kProAcc));
+  return (pro == kProNormAcc && (epi == kEpiNone || epi == kEpiSwiglu)) || (epi == kEpiResidual && (pro == kProPlain || pro == kProAcc)) ||
+         (pro == kProPlain && epi == kEpiSwiglu);
 }
 
 hipError_t launch_stream_chained(GroupDev& g, const ChainDev& ch, int pro, int epi, hipStream_t stream) {

@@ -218,17 +218,22 @@ def load_glowq_artifacts(shared_path: str, bmap_path: str, device="cuda"):
     return shared, bmap
 
 
+# How much of the work between the linears the fused step folds into the group launches by default (FusedStep).
+DEFAULT_CHAIN = "mlp"
+
+
 class FusedStep:
     """One decode token as a fixed chain of launches on static buffers, ready for HIP-graph capture.  Reads the
     quantised buffers and low-rank factors straight out of the model's modules.
-    With `chain` (and a model whose four groups per layer all carry a shared correction of one rank) a layer is six
-    launches -- q|k|v, attention, merge of its splits, o_proj, gate|up, down_proj -- with the norms, the residual adds,
-    the gate and every projection r = x R^T done inside the group launches on either side of them
-    (glowq_w4a16_group_forward_chained).  Otherwise nine: the same with two norm launches and a gate launch that also
-    produce the projections."""
+    Without `chain` a layer is nine launches: q|k|v, attention, merge of its splits, o_proj, gate|up, down_proj and,
+    between them, two norm launches and a gate launch that also produce the projections r = x R^T.
+    `chain` (for a model whose four groups per layer all carry a shared correction of one rank) moves that work into
+    the group launches on either side of it (glowq_w4a16_group_forward_chained): "mlp" folds the gate into gate|up and
+    the residual add, the next layer's norm and its projection into down_proj and q|k|v (seven launches per layer);
+    "full" also folds the norm in front of gate|up into o_proj and gate|up (six)."""
 
     def __init__(self, model: Decoder, caches, cos, sin, tok, pos, next_tok, share: bool = True, attention_splits: int = 4,
-                 chain: bool = True):
+                 chain=DEFAULT_CHAIN):
         cfg = model.cfg
         self.share = share  # False: every module projects x on R by itself and launches alone (the no-sharing comparator)
         self.model, self.cfg = model, cfg
@@ -267,7 +272,11 @@ class FusedStep:
                 "down": self._group([mlp.down_proj], [self.dn], f16),
             })
         self.q_view, self.k_view, self.v_view = self.qkv[0, :qd], self.qkv[0, qd:qd + kd], self.qkv[0, qd + kd:]
-        self.chained = bool(chain) and share and attention_splits > 1 and self._chainable()
+        if chain is True:
+            chain = "full"
+        if chain not in (False, None, "full", "mlp"):
+            raise ValueError("chain must be False, 'mlp' or 'full'")
+        self.chained = chain if (chain and share and attention_splits > 1 and self._chainable()) else False
         if self.chained:
             # the next group's right factor transposed (rows = the producing group's output rows), and one accumulator
             # per hand-over, all cleared by one fill at the head of the step
@@ -391,9 +400,45 @@ class FusedStep:
         ext.argmax_advance(self.logits, self.next_tok, self.tok, self.pos)
 
     @torch.no_grad()
+    def _run_chained_mlp(self):
+        """Seven launches per layer: the norm in front of gate|up stays a launch of its own (it also adds o_proj's output
+        to the residual stream and projects on gate|up's right factor); the residual stream moves to the other of the
+        two buffers there."""
+        ext = self.ext
+        cur = self.x
+        self.acc.zero_()
+        for i, (lay, (ck, cv)) in enumerate(zip(self.plan, self.caches)):
+            qkv, o, gu, down = lay["qkv"], lay["o"], lay["gu"], lay["down"]
+            if i == 0:
+                torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=self.x_alt)
+                ext.add_rmsnorm_proj(self.x_alt, None, lay["ln1"].weight, cur, self.h, qkv["R"], qkv["r"], lay["ln1"].eps)
+                qkv["call"].run(self.h, r=qkv["r"], outs=qkv["outs"], project=False)
+            else:
+                qkv["call"].run_chained(cur[0], CHAIN_PRO_NORM_ACC, CHAIN_EPI_NONE, outs=[self.q_view, self.k_view, self.v_view],
+                                        norm_weight=lay["ln1"].weight, eps=lay["ln1"].eps, acc_in=self.acc[i - 1, 2])
+            ext.rope_attend_split(self.q_view, self.k_view, self.v_view, self.cos, self.sin, self.pos, ck, cv, self.partials, self.scale)
+            ext.attend_combine_proj(self.partials, self.attn, o["R"], o["r"])
+            o["call"].run(self.attn, r=o["r"], outs=o["outs"], project=False)
+            nxt_buf = self.x_alt if cur is self.x else self.x
+            ext.add_rmsnorm_proj(cur, self.o, lay["ln2"].weight, nxt_buf, self.h, gu["R"], gu["r"], lay["ln2"].eps)
+            cur = nxt_buf
+            gu["call"].run_chained(self.h[0], CHAIN_PRO_PLAIN, CHAIN_EPI_SWIGLU, r=gu["r"][0], outs=[None, None], act=self.act[0],
+                                   next_Rt=lay["Rt_down"], acc_out=self.acc[i, 1])
+            nxt = lay["ln1_next"]
+            down["call"].run_chained(self.act[0], CHAIN_PRO_ACC, CHAIN_EPI_RESIDUAL, acc_in=self.acc[i, 1], outs=[None], resid=cur[0],
+                                     next_norm_weight=nxt.weight if nxt is not None else None, next_Rt=lay["Rt_next"],
+                                     acc_out=self.acc[i, 2] if nxt is not None else None)
+        norm = self.model.model.norm
+        ext.add_rmsnorm(cur, None, norm.weight, self.h, norm.eps)
+        torch.mm(self.h, self.model.lm_head.weight.t(), out=self.logits)
+        ext.argmax_advance(self.logits, self.next_tok, self.tok, self.pos)
+
+    @torch.no_grad()
     def run(self):
-        if self.chained:
+        if self.chained == "full":
             return self._run_chained()
+        if self.chained == "mlp":
+            return self._run_chained_mlp()
         ext, cfg = self.ext, self.cfg
         x = self.x
         torch.index_select(self.model.model.embed_tokens.weight, 0, self.tok, out=x)
@@ -431,7 +476,7 @@ class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
     def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True,
-                 attention_splits: int = 0, chain: bool = True):
+                 attention_splits: int = 0, chain=DEFAULT_CHAIN):
         self.model = model
         cfg = model.cfg
         if attention_splits <= 0:
@@ -523,7 +568,7 @@ class GreedyDecoder:
 
 def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
             fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0,
-            chain: bool = True) -> dict:
+            chain=DEFAULT_CHAIN) -> dict:
     """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
     second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798)."""
     import os
@@ -536,7 +581,7 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
     dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits, chain=chain)
-    chained = dec.fused is not None and dec.fused.chained
+    chained = dec.fused.chained if dec.fused is not None else False
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (prompt_tokens,), generator=g)
     dec.generate(prompt, 4)  # warm-up (also captures the graph)
@@ -546,7 +591,8 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
                     f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + (f" + GlowQ r={cfg.rank}" if correction else ""),
         "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "graph": graph, "fused_step": fused, "group_sharing": share,
         "chained_launches": chained,
-        "launches_per_token": (6 * cfg.layers + 6 if chained else 9 * cfg.layers + 5) if (fused and share and correction) else None,
+        "launches_per_token": ({"full": 6 * cfg.layers + 6, "mlp": 7 * cfg.layers + 6, False: 9 * cfg.layers + 5}[chained]
+                               if (fused and share and correction) else None),
         "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((new_tokens - 1) / decode_s, 1),
         "ms_per_token": round(decode_s * 1e3 / (new_tokens - 1), 3), "build_s": round(build_s, 1)}
 
@@ -560,15 +606,16 @@ def main():
     ap.add_argument("--no-sharing", action="store_true", help="fused step with one projection and one launch per module")
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
     ap.add_argument("--no-correction", action="store_true")
-    ap.add_argument("--no-chain", action="store_true",
-                    help="fused step with separate norm / gate launches (nine per layer) instead of the chained group launches (six)")
+    ap.add_argument("--chain", choices=["off", "mlp", "full"], default=None,
+                    help="fused step: how much of the work between the linears the group launches take over (9 / 7 / 6 launches per layer)")
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--attention-splits", type=int, default=0,
                     help="workgroups per head in the fused step's attention (0: by the cache length)")
     args = ap.parse_args()
     print(json.dumps(measure(args.layers, args.prompt, args.new, vocab=args.vocab, graph=not args.no_graph,
                              fused=not args.module_path, share=not args.no_sharing, correction=not args.no_correction,
-                             attention_splits=args.attention_splits, chain=not args.no_chain)))
+                             attention_splits=args.attention_splits,
+                             chain={None: DEFAULT_CHAIN, "off": False, "mlp": "mlp", "full": "full"}[args.chain])))
 
 
 if __name__ == "__main__":

@@ -265,7 +265,7 @@ int glowq_attend_combine_proj(const float* partials, void* out, const void* R, v
  * act_fn(gate) * up around the wrappers' forward (src/step3_eval_dataset.py:470-511, generate loop :705-798); results
  * agree with the separate launches above within fp16 rounding of r (the projection is taken of the unrounded norm).
  *
- * prologue  GLOWQ_CHAIN_PRO_PLAIN     x [K] and r [rank] as in glowq_w4a16_group_forward (r may be NULL with rank 0)
+ * prologue  GLOWQ_CHAIN_PRO_PLAIN     x [K] and r [rank] as in glowq_w4a16_group_forward
  *           GLOWQ_CHAIN_PRO_ACC       x [K] as given, r = fp16(P) with P read from acc_in
  *           GLOWQ_CHAIN_PRO_NORM_ACC  x is the residual stream [K]: the launch applies RMSNorm(norm_weight, eps) to it
  *                                     itself and takes r = fp16(f P), f the norm's scalar factor
@@ -275,6 +275,7 @@ int glowq_attend_combine_proj(const float* partials, void* out, const void* R, v
  *                                     added into acc_out (next_norm_weight NULL: all ones)
  *           GLOWQ_CHAIN_EPI_SWIGLU    two members of equal N (gate, up): act[n] = fp16(fp16(silu(gate[n])) * up[n]);
  *                                     with next_Rt: P = next_R act added into acc_out
+ * Served combinations: (NORM_ACC, NONE), (NORM_ACC, SWIGLU), (PLAIN, SWIGLU), (PLAIN, RESIDUAL), (ACC, RESIDUAL).
  * next_Rt is the next group's right factor transposed, [N_total, rank] fp16 row-major, of the same rank as this launch.
  * An accumulator is GLOWQ_CHAIN_ACC_BYTES of device memory, 8-byte aligned, all zero when the producer starts (the
  * caller clears it once per token, e.g. with a fill kernel; 64-bit fixed-point sums, so results do not depend on the

@@ -156,6 +156,31 @@ def test_norm_prologue_with_swiglu_epilogue(ext, K, N, rank, gs, bias):
     assert torch.equal(act2, act) and torch.equal(acc2, acc_out)
 
 
+@pytest.mark.parametrize("K,N,rank,gs", [(4096, 2048, 128, 128), (1536, 333, 64, 128)])
+def test_swiglu_epilogue_with_r_given(ext, K, N, rank, gs):
+    """h and r come from a norm launch of their own; the launch gates its two members and projects the result."""
+    print(f"case K={K} N={N} rank={rank}", flush=True)
+    x, members, R = make_group(1700 + N, 1, K, [N, N], rank, group_size=gs)
+    next_R = (torch.randn(rank, N, generator=torch.Generator().manual_seed(N)) * N ** -0.5).half().numpy()
+    pg = prepared(ext, members, K, gs, 1.0)
+    r64 = x[0].astype(np.float64) @ R.astype(np.float64).T
+    act, acc_out = torch.zeros(N, dtype=torch.float16, device="cuda"), new_acc()
+    gate_y, up_y = (torch.zeros(N, dtype=torch.float16, device="cuda") for _ in range(2))
+    pg.run_chained(dev(x[0]), CHAIN_PRO_PLAIN, CHAIN_EPI_SWIGLU, r=dev(r64.astype(np.float16)), outs=[gate_y, up_y], act=act,
+                   next_Rt=dev(np.ascontiguousarray(next_R.T)), acc_out=acc_out)
+    torch.cuda.synchronize()
+    want = [oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], gs, R, m["L"], 1.0)[0] for m in members]
+    assert_close(gate_y.cpu().numpy(), want[0], "gate")
+    assert_close(up_y.cpu().numpy(), want[1], "up")
+    ref_act = oracle.swiglu(gate_y.cpu().numpy(), up_y.cpu().numpy()).astype(np.float64)
+    got_act = act.cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got_act - ref_act) <= 2.0 ** -10 * np.abs(ref_act) + 1e-7)
+    P, flag = acc_values(acc_out, rank)
+    assert flag == 0
+    np.testing.assert_allclose(P, next_R.astype(np.float64) @ got_act, rtol=0,
+                               atol=2e-6 * (np.abs(next_R.astype(np.float64)) @ np.abs(got_act)).max() + 1e-6)
+
+
 def test_overflow_raises_the_flag_and_poisons_r(ext):
     """A partial sum beyond the fixed point's range must not wrap silently: the producer sets the flag, the consumer's
     outputs come out NaN."""

@@ -308,7 +308,7 @@ def test_split_attention_and_merge_match_single_workgroup(ext, fp16_out, pos, sp
     assert torch.equal(plain, got)
 
 
-@pytest.mark.parametrize("chain", [True, False], ids=["chained", "separate_glue"])
+@pytest.mark.parametrize("chain", ["full", "mlp", False], ids=["chained", "chained_mlp", "separate_glue"])
 def test_fused_step_matches_module_path(fp16_out, chain):
     cfg = decode.DecoderConfig(**TINY)
     model, _, _ = decode.build_decoder(cfg, seed=8)
@@ -354,7 +354,7 @@ GEOM_8B = dict(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128, interm
                group_size=128, rank=128)
 
 
-@pytest.mark.parametrize("chain", [True, False], ids=["chained", "separate_glue"])
+@pytest.mark.parametrize("chain", ["full", "mlp", False], ids=["chained", "chained_mlp", "separate_glue"])
 def test_fused_step_at_8b_geometry_matches_effective_weight_network(fp16_out, chain):
     """Two layers of the Llama-3.1-8B geometry (hidden 4096, 32 query / 8 KV heads of 128, SwiGLU 14336, W4A16 g = 128,
     rank 128) with 512 cached positions: the fused single-token step (group launches, attention split over 4 workgroups
