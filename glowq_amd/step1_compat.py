@@ -14,9 +14,12 @@ reports.
 
     python -m glowq_amd.step1_compat --weights original_weights.pt [--group-size 128]
 
-Parity of `quantize_step1`: pinned through its agreement with the golden-pinned W4A16 quantiser on in-range groups and
-by reading for the packing; its behaviour on out-of-range zero-points (a float -> uint8 conversion of a negative or
-large value) is implementation-defined in the reference and is flagged here, not reproduced.
+Parity of `quantize_step1` / `dequant_step1`: bit for bit against vectors the reference's own layer wrote on CPU
+tensors (tests/golden/step1_golden.npz) for weights whose zero-points are in range.  On out-of-range zero-points the
+reference stores whatever its float -> uint8 conversion yields (implementation-defined; on CPU the value modulo 256,
+whose upper bits then overwrite the neighbouring group's nibble): flagged here, not reproduced.  The reference's layer
+raises for in_features that are not a multiple of the group size and for an odd number of groups (its buffers are sized
+in_features / 2 and groups // 2); this module pads both, which only a caller outside the reference's domain can see.
 """
 from __future__ import annotations
 

@@ -8,6 +8,8 @@ Covers the functions whose bit-exact behaviour depends on per-op fp16 rounding o
 and so cannot be fixed by mathematics alone:
   _pack_int4_to_int32, _unpack_int4_i32, _quantize_per_group_w4, CudaW4A16Linear._dequant_chunk and
   the CPU chunked forward (src/cuda_w4a16/linear.py:42-88,229-253).
+and the quantiser of step 1's layer, TritonTrue4BitLinear.from_float with dequantize_from_triton_layer
+(src/step1_quantize.py:215-290), on CPU tensors (its Triton kernel is never launched).
 Outputs are plain ``.npz`` arrays (inputs and expected outputs only).
 """
 import os
@@ -96,5 +98,44 @@ def main(ref_root: str) -> None:
     print("wrote", os.path.join(here, "w4a16_golden.npz"), len(out), "arrays")
 
 
+def step1(ref_root: str) -> None:
+    """Step 1's quantiser: in-range groups, one-sided groups (zero-point outside [0, 15]), two group sizes."""
+    sys.path.insert(0, os.path.join(ref_root, "src"))
+    import step1_quantize as ref  # noqa: E402  (imports transformers / datasets / triton; runs nothing of them)
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    out = {}
+    cases = {
+        # name: (N, K, group_size, std, seed, one-sided rows)
+        "in_range": (8, 512, 128, 0.02, 20, False),
+        "many_groups": (6, 1024, 128, 0.05, 21, False),   # (an odd number of groups raises in the reference: its
+                                                           #  zero-point buffer holds G // 2 bytes, from_float packs ceil)
+        "small_groups": (4, 256, 64, 1.0, 22, False),      # (K not a multiple of the group size raises as well: the code
+                                                           #  buffer holds K // 2 bytes, from_float packs the padded row)
+        "one_sided": (8, 256, 128, 0.02, 23, True),
+    }
+    for name, (n, k, gs, std, seed, one_sided) in cases.items():
+        g = torch.Generator().manual_seed(seed)
+        w = (torch.randn(n, k, generator=g) * std).half()
+        if one_sided:
+            w[0, :128] = w[0, :128].abs() + 0.05          # all positive, far from zero: zero-point below 0
+            w[1, 128:] = -w[1, 128:].abs() - 0.05         # all negative: zero-point above 15
+            w[2, :128] = w[2, :128].abs() + 0.001         # all positive, touching zero: zero-point 0 or -1
+        lin = torch.nn.Linear(k, n, bias=False).half()
+        with torch.no_grad():
+            lin.weight.copy_(w)
+        layer = ref.TritonTrue4BitLinear.from_float(lin, gs)
+        out[f"{name}_w"] = w.numpy()
+        out[f"{name}_gs"] = np.array([gs], dtype=np.int64)
+        out[f"{name}_qweight"] = layer.qweight.numpy()
+        out[f"{name}_qzeros"] = layer.qzeros.numpy()
+        out[f"{name}_scales"] = layer.scales.numpy()
+        out[f"{name}_deq"] = ref.dequantize_from_triton_layer(layer).numpy()
+    np.savez_compressed(os.path.join(here, "step1_golden.npz"), **out)
+    print("wrote", os.path.join(here, "step1_golden.npz"), len(out), "arrays")
+
+
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference")
+    root = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+    main(root)
+    step1(root)
