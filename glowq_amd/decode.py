@@ -49,13 +49,30 @@ class DecoderConfig:
     rank: int = 128
 
 
+class _Glue:
+    """What the modules need to run a single token through the library's glue kernels instead of torch expressions
+    (`Decoder.use_single_token_glue`): the extension, the rotary tables [max_len, head_dim] fp32 and the device tensor
+    holding the token's position."""
+
+    def __init__(self, ext, cos_t, sin_t, pos):
+        self.ext, self.cos_t, self.sin_t, self.pos = ext, cos_t, sin_t, pos
+
+
 class RMSNorm(nn.Module):
     def __init__(self, dim: int, eps: float):
         super().__init__()
         self.weight = nn.Parameter(torch.ones(dim, dtype=torch.float16))
         self.eps = eps
+        self.glue: Optional[_Glue] = None
 
-    def forward(self, x):
+    def forward(self, x, delta=None):
+        """rmsnorm(x) * weight; with `delta` (single-token glue only) x += delta first, in place."""
+        if self.glue is not None and x.dim() == 2 and x.size(0) == 1 and x.dtype == torch.float16:
+            h = torch.empty_like(x)
+            self.glue.ext.add_rmsnorm(x, delta, self.weight, h, self.eps)
+            return h
+        if delta is not None:
+            x.add_(delta)
         return F.rms_norm(x, (x.size(-1),), self.weight, self.eps)
 
 
@@ -68,6 +85,7 @@ class Attention(nn.Module):
         self.k_proj = nn.Linear(h, cfg.kv_heads * d, bias=False)
         self.v_proj = nn.Linear(h, cfg.kv_heads * d, bias=False)
         self.o_proj = nn.Linear(cfg.heads * d, h, bias=False)
+        self.glue: Optional[_Glue] = None
 
     def forward(self, x, cos, sin, cache_k, cache_v, pos_idx, mask):
         """x [T, hidden]; cos/sin [T, head_dim]; caches [kv_heads, max_len, head_dim]; pos_idx [T] (device,
@@ -75,6 +93,14 @@ class Attention(nn.Module):
         empty cache (prefill): attention then runs causally over the new keys alone."""
         cfg = self.cfg
         T = x.size(0)
+        if self.glue is not None and T == 1 and mask is not None and pos_idx is self.glue.pos:
+            # one launch: rotary embedding, cache append and attention of the one query over the cache
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+            if q.dtype == k.dtype == v.dtype == torch.float16:
+                out = torch.empty_like(q)
+                self.glue.ext.rope_attend(q[0], k[0], v[0], self.glue.cos_t, self.glue.sin_t, pos_idx, cache_k, cache_v, out[0],
+                                          cfg.head_dim ** -0.5)
+                return self.o_proj(out)
         q = self.q_proj(x).view(T, cfg.heads, cfg.head_dim).transpose(0, 1)      # [H, T, d]
         k = self.k_proj(x).view(T, cfg.kv_heads, cfg.head_dim).transpose(0, 1)   # [KV, T, d]
         v = self.v_proj(x).view(T, cfg.kv_heads, cfg.head_dim).transpose(0, 1)
@@ -102,9 +128,15 @@ class MLP(nn.Module):
         self.gate_proj = nn.Linear(cfg.hidden, cfg.intermediate, bias=False)
         self.up_proj = nn.Linear(cfg.hidden, cfg.intermediate, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate, cfg.hidden, bias=False)
+        self.glue: Optional[_Glue] = None
 
     def forward(self, x):
-        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+        gate, up = self.gate_proj(x), self.up_proj(x)
+        if self.glue is not None and x.size(0) == 1 and gate.dtype == up.dtype == torch.float16:
+            act = torch.empty_like(gate)
+            self.glue.ext.silu_mul(gate, up, act)
+            return self.down_proj(act)
+        return self.down_proj(F.silu(gate) * up)
 
 
 class DecoderLayer(nn.Module):
@@ -116,6 +148,11 @@ class DecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(cfg.hidden, cfg.rms_eps)
 
     def forward(self, x, cos, sin, cache_k, cache_v, pos_idx, mask):
+        if self.input_layernorm.glue is not None and x.size(0) == 1 and x.dtype == torch.float16:
+            # single-token glue: the residual add rides on the norm launch that follows it (x is updated in place)
+            attn = self.self_attn(self.input_layernorm(x), cos, sin, cache_k, cache_v, pos_idx, mask)
+            h = self.post_attention_layernorm(x, delta=attn.to(x.dtype))
+            return x.add_(self.mlp(h).to(x.dtype))
         x = x + self.self_attn(self.input_layernorm(x), cos, sin, cache_k, cache_v, pos_idx, mask)
         return x + self.mlp(self.post_attention_layernorm(x))
 
@@ -136,6 +173,16 @@ class Decoder(nn.Module):
         self.model.layers = nn.ModuleList()
         self.model.norm = RMSNorm(cfg.hidden, cfg.rms_eps)
         self.lm_head = nn.Linear(cfg.hidden, cfg.vocab, bias=False)
+
+    def use_single_token_glue(self, cos_t=None, sin_t=None, pos=None) -> None:
+        """Switches the modules' single-token path to the library's glue kernels (one launch each for norm + residual
+        add, rotary + cache append + attention, and the gate), or back to torch expressions when called without
+        arguments.  `cos_t` / `sin_t` are the tables of `rope_tables`, `pos` the int64 device tensor the decode loop
+        passes as `pos_idx` for its one token (the attention kernel reads the position from it on the device)."""
+        glue = _Glue(load_w4a16_extension(), cos_t, sin_t, pos) if cos_t is not None else None
+        for mod in self.modules():
+            if isinstance(mod, (RMSNorm, Attention, MLP)):
+                mod.glue = glue
 
     def rope_tables(self, device):
         cfg = self.cfg
@@ -476,7 +523,7 @@ class GreedyDecoder:
     """Prefill + greedy decode at batch 1 with a static KV cache; the one-token step is captured as a HIP graph."""
 
     def __init__(self, model: Decoder, use_graph: bool = True, fused: bool = False, share: bool = True,
-                 attention_splits: int = 0, chain=DEFAULT_CHAIN):
+                 attention_splits: int = 0, chain=DEFAULT_CHAIN, module_glue: bool = False):
         self.model = model
         cfg = model.cfg
         if attention_splits <= 0:
@@ -497,6 +544,9 @@ class GreedyDecoder:
         self.graph = None
         self.fused = FusedStep(model, self.caches, self.cos, self.sin, self.tok, self.pos, self.next_tok, share,
                                attention_splits, chain) if fused else None
+        # module path: torch expressions between the linears (the default, what an unmodified model does) or the
+        # library's single-token glue kernels
+        self.module_glue = bool(module_glue) and not fused
 
     @torch.no_grad()
     def _step(self):
@@ -505,7 +555,13 @@ class GreedyDecoder:
         if self.fused is not None:
             self.fused.run()
             return
-        logits = self.model.forward_tokens(self.tok, self.pos, self.caches, self.cos, self.sin)
+        if self.module_glue:
+            self.model.use_single_token_glue(self.cos, self.sin, self.pos)
+        try:
+            logits = self.model.forward_tokens(self.tok, self.pos, self.caches, self.cos, self.sin)
+        finally:
+            if self.module_glue:
+                self.model.use_single_token_glue()
         self.next_tok.copy_(logits.argmax(-1))
         self.tok.copy_(self.next_tok)
         self.pos.add_(1)
@@ -568,9 +624,11 @@ class GreedyDecoder:
 
 def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
             fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0,
-            chain=DEFAULT_CHAIN) -> dict:
+            chain=DEFAULT_CHAIN, module_glue: bool = True) -> dict:
     """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
-    second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798)."""
+    second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798).
+    `fused=False` decodes through the torch modules (CudaW4A16Linear / AddSVDCorrection inside the decoder's layers),
+    with the library's single-token glue kernels between them (`module_glue`) or torch expressions."""
     import os
 
     os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
@@ -580,7 +638,8 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
     model, _, _ = build_decoder(cfg, with_correction=correction)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
-    dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits, chain=chain)
+    dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits, chain=chain,
+                        module_glue=module_glue)
     chained = dec.fused.chained if dec.fused is not None else False
     g = torch.Generator().manual_seed(3)
     prompt = torch.randint(0, cfg.vocab, (prompt_tokens,), generator=g)
@@ -590,7 +649,7 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
         "workload": f"random-init Llama-style decoder, {cfg.layers} layers, hidden {cfg.hidden}, GQA {cfg.heads}/{cfg.kv_heads}x{cfg.head_dim}, "
                     f"SwiGLU {cfg.intermediate}, W4A16 g={cfg.group_size}" + (f" + GlowQ r={cfg.rank}" if correction else ""),
         "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "graph": graph, "fused_step": fused, "group_sharing": share,
-        "chained_launches": chained,
+        "chained_launches": chained, "module_glue": dec.module_glue,
         "launches_per_token": ({"full": 6 * cfg.layers + 6, "mlp": 7 * cfg.layers + 6, False: 9 * cfg.layers + 5}[chained]
                                if (fused and share and correction) else None),
         "ttfb_ms": round(ttfb * 1e3, 2), "decode_tok_per_s": round((new_tokens - 1) / decode_s, 1),
@@ -605,6 +664,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-sharing", action="store_true", help="fused step with one projection and one launch per module")
     ap.add_argument("--module-path", action="store_true", help="decode through the torch modules instead of the fused step")
+    ap.add_argument("--torch-glue", action="store_true",
+                    help="with --module-path: torch expressions between the linears instead of the library's single-token glue kernels")
     ap.add_argument("--no-correction", action="store_true")
     ap.add_argument("--chain", choices=["off", "mlp", "full"], default=None,
                     help="fused step: how much of the work between the linears the group launches take over (9 / 7 / 6 launches per layer)")
@@ -615,7 +676,8 @@ def main():
     print(json.dumps(measure(args.layers, args.prompt, args.new, vocab=args.vocab, graph=not args.no_graph,
                              fused=not args.module_path, share=not args.no_sharing, correction=not args.no_correction,
                              attention_splits=args.attention_splits,
-                             chain={None: DEFAULT_CHAIN, "off": False, "mlp": "mlp", "full": "full"}[args.chain])))
+                             chain={None: DEFAULT_CHAIN, "off": False, "mlp": "mlp", "full": "full"}[args.chain],
+                             module_glue=not args.torch_glue)))
 
 
 if __name__ == "__main__":

@@ -350,6 +350,41 @@ def test_fused_step_matches_module_path(fp16_out, chain):
         assert torch.equal(got, eager)
 
 
+def test_module_path_with_single_token_glue_matches_torch_expressions(fp16_out):
+    """The decoder's modules with the library's glue kernels between the linears (norm + residual add, rotary + cache
+    append + attention, gate) against the same modules with torch expressions, teacher forced, and under a graph."""
+    cfg = decode.DecoderConfig(**TINY)
+    model, _, _ = decode.build_decoder(cfg, seed=8)
+    prompt = torch.randint(0, cfg.vocab, (11,), generator=torch.Generator().manual_seed(4))
+    ref = decode.GreedyDecoder(model, use_graph=False)
+    fast = decode.GreedyDecoder(model, use_graph=False, module_glue=True)
+    first = ref.prefill(prompt)
+    fast.prefill(prompt)
+    tok = first.clone()
+    for step in range(5):
+        pos = torch.tensor([prompt.numel() + step], device="cuda")
+        want = model.forward_tokens(tok, pos, ref.caches, ref.cos, ref.sin).float()
+        fast.tok.copy_(tok), fast.pos.copy_(pos)
+        fast._step()
+        assert all(m.glue is None for m in model.modules() if hasattr(m, "glue"))   # switched back after the step
+        assert int(fast.pos) == int(pos) + 1
+        for (ka, va), (kb, vb) in zip(ref.caches, fast.caches):
+            assert (ka[:, int(pos)].float() - kb[:, int(pos)].float()).abs().max() <= 2e-2
+            assert (va[:, int(pos)].float() - vb[:, int(pos)].float()).abs().max() <= 2e-2
+        # the step's own logits are not kept: compare the pick, and the logits of a second pass through the glue path
+        model.use_single_token_glue(fast.cos, fast.sin, fast.pos)
+        fast.pos.copy_(pos)
+        got = model.forward_tokens(tok, fast.pos, fast.caches, fast.cos, fast.sin).float()
+        model.use_single_token_glue()
+        fast.pos.copy_(pos + 1)
+        assert (got - want).abs().max() <= 1e-2 + 1e-2 * want.abs().max(), step
+        tok = want.argmax(-1)
+    eager, _, _ = decode.GreedyDecoder(model, use_graph=False, module_glue=True).generate(prompt, 8)
+    graphed = decode.GreedyDecoder(model, use_graph=True, module_glue=True)
+    for _ in range(2):
+        assert torch.equal(graphed.generate(prompt, 8)[0], eager)
+
+
 GEOM_8B = dict(hidden=4096, layers=2, heads=32, kv_heads=8, head_dim=128, intermediate=14336, vocab=4096, max_len=640,
                group_size=128, rank=128)
 
