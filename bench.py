@@ -192,7 +192,7 @@ def prefill_leg(torch, ext, dev):
     prefill = {"workload": f"Qwen2.5-7B-shaped layer, M={PREFILL_TOKENS}, int4 g=128 asym, shared rank-{RANK} correction",
                "per_group": {}}
     pl = make_layer(torch, dev, 7, PREFILL_GROUPS)
-    tot_us, tot_fl = 0.0, 0.0
+    tot_us, tot_fl, tot_vus, tot_vfl = 0.0, 0.0, 0.0, 0.0
     for name, (K, Ns) in PREFILL_GROUPS.items():
         members, R = pl[name]
         xp = torch.randn(PREFILL_TOKENS, K, device=dev, generator=g).half()
@@ -214,14 +214,39 @@ def prefill_leg(torch, ext, dev):
         us = sorted(ts)[len(ts) // 2]
         N = sum(Ns)
         fl = 2.0 * PREFILL_TOKENS * (N * K + RANK * K + N * RANK)
+        # yardstick: the vendor library's plain fp16 GEMM of the same M x N x K on weights that are already fp16 (no
+        # dequantisation, no correction): what the matrix cores sustain on this shape under their power limit
+        wd = torch.randn(N, K, device=dev, generator=g).half().mul_(0.02)
+        yd = torch.empty(PREFILL_TOKENS, N, dtype=torch.float16, device=dev)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.03:
+            torch.mm(xp, wd.t(), out=yd)
+            torch.cuda.synchronize()
+        tv = []
+        for _ in range(5):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(4):
+                torch.mm(xp, wd.t(), out=yd)
+            b.record()
+            torch.cuda.synchronize()
+            tv.append(a.elapsed_time(b) * 1e3 / 4)
+        vus = sorted(tv)[len(tv) // 2]
+        vfl = 2.0 * PREFILL_TOKENS * N * K
         prefill["per_group"][name] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
-                                      "frac_mfma_peak": round(fl / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+                                      "frac_mfma_peak": round(fl / us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
+                                      "vendor_fp16_gemm_us": round(vus, 1),
+                                      "vendor_fp16_gemm_frac_mfma_peak": round(vfl / vus / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
         tot_us += us
         tot_fl += fl
-        del xp, rp, op
+        tot_vus += vus
+        tot_vfl += vfl
+        del xp, rp, op, wd, yd
     prefill["us_per_layer"] = round(tot_us, 1)
     prefill["TFLOPs"] = round(tot_fl / tot_us / 1e6, 1)
     prefill["frac_mfma_peak"] = round(tot_fl / tot_us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)
+    prefill["vendor_fp16_gemm_us_per_layer"] = round(tot_vus, 1)
+    prefill["vendor_fp16_gemm_frac_mfma_peak"] = round(tot_vfl / tot_vus / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)
     return prefill
 
 
@@ -503,7 +528,14 @@ def main():
         import contextlib
         from glowq_amd import decode as decode_loop
         with contextlib.redirect_stdout(sys.stderr):  # the patcher reports what it wrapped; stdout carries the JSON line only
-            decode = decode_loop.measure(32, 512, 256)
+            cfg = decode_loop.DecoderConfig(layers=32, max_len=1024)
+            model, _, _ = decode_loop.build_decoder(cfg)
+            decode = decode_loop.measure(32, 512, 256, model=model)
+            # the same model through its torch modules (CudaW4A16Linear / AddSVDCorrection), single-token glue kernels
+            # between them, under a graph
+            mod = decode_loop.measure(32, 512, 64, fused=False, model=model)
+            decode["module_path"] = {k: mod[k] for k in ("new_tokens", "graph", "module_glue", "decode_tok_per_s", "ms_per_token")}
+            del model
 
     traffic, traffic_source = read_traffic_sidecar()
     result = {

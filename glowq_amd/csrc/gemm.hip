@@ -50,6 +50,11 @@ struct GemmGroup {
   // `partials` ([slice][tile][BM * BN] in accumulator-register order) and gemm_reduce_kernel adds them in slice order
   int slices;
   float* partials;
+  // tail split (super-block form, slices == 1): workgroups [0, full) are whole tiles; behind them every tail tile comes
+  // as tail_slices workgroups, slice t % tail_slices of tile full + t / tail_slices for t = blockIdx.x - full, which
+  // leave partials ([slice][tail tile][BM * BN]) for gemm_reduce_kernel.  The last, partly filled round of workgroups
+  // of a launch then costs its share of a round instead of a whole one.  tail_slices <= 1: off.
+  int full, tail_slices;
 };
 
 __device__ __forceinline__ h8 permute_for_nibble_order(const h8& v) {
@@ -92,10 +97,23 @@ template <int kMT, int kNT, bool kQuant, bool kSuper = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
 void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   // member of this workgroup, picked with scalar selects from fixed kernel-argument offsets
+  // which tile and which slice of its K range this workgroup serves
+  int wg = (int)blockIdx.x, slice = (int)blockIdx.y, nslices = gg.slices, part_tile = (int)blockIdx.x, part_tiles = (int)gridDim.x;
+  if (kQuant && kSuper && gg.tail_slices > 1) {
+    nslices = 1;
+    if (wg >= gg.full) {
+      const int t = wg - gg.full;
+      part_tile = t / gg.tail_slices;
+      slice = t - part_tile * gg.tail_slices;
+      wg = gg.full + part_tile;
+      nslices = gg.tail_slices;
+      part_tiles = ((int)gridDim.x - gg.full) / gg.tail_slices;
+    }
+  }
   GemmArgs a = gg.m[0];
   int blk_base = 0;
 #define GLOWQ_PICK(i)                                         \
-  if (gg.n > i && (int)blockIdx.x >= gg.blk_end[i - 1]) {    \
+  if (gg.n > i && wg >= gg.blk_end[i - 1]) {                 \
     a = gg.m[i];                                              \
     blk_base = gg.blk_end[i - 1];                             \
   }
@@ -111,7 +129,7 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int blk = (int)blockIdx.x - blk_base;
+  const int blk = wg - blk_base;
   const int bm = blk % m_blocks;  // row blocks vary fastest: neighbouring workgroups share weight columns
   const int bn = blk / m_blocks;
   const int m0 = bm * BM;
@@ -181,7 +199,7 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   int stage = 0;
 
   // ---- phase 1: the correction as a K-extension, acc = r . L^T, fp16 B operand ----------------------
-  if (kQuant && a.r != nullptr && blockIdx.y == 0) {
+  if (kQuant && a.r != nullptr && slice == 0) {
     // ranks are multiples of 8: in a partial last block the octets of r past the rank count as zero and L is read
     // from the row's last octet (finite values)
     const int steps = (a.rank + kBK - 1) / kBK;
@@ -358,10 +376,10 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
       __syncthreads();
       stage ^= 1;
     };
-    // this workgroup's super-blocks: all of them, or slice blockIdx.y of gg.slices
+    // this workgroup's super-blocks: all of them, or slice `slice` of `nslices`
     const int sb_total = steps >> 2;  // steps is a multiple of 4 here
-    const int sb_per = (sb_total + gg.slices - 1) / gg.slices;
-    const int ks0 = min((int)blockIdx.y * sb_per, sb_total) * 4;
+    const int sb_per = (sb_total + nslices - 1) / nslices;
+    const int ks0 = min(slice * sb_per, sb_total) * 4;
     const int ks1 = min(ks0 + sb_per * 4, steps);
     load_a_sub(areg, ks0);
     issue_b(ks0 >> 2, bl);
@@ -475,8 +493,8 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
 
   // ---- epilogue: accumulator register i of a 32x32 tile is row 8*(i/4) + 4*lh + i%4, column ln ---------
   if constexpr (kQuant && kSuper) {
-    if (gg.slices > 1) {
-      float* part = gg.partials + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (BM * BN);
+    if (nslices > 1) {
+      float* part = gg.partials + ((size_t)slice * part_tiles + part_tile) * (BM * BN);
 #pragma unroll
       for (int tm = 0; tm < kMT; ++tm)
 #pragma unroll
@@ -506,16 +524,20 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
 // in x, same workgroup -> (member, row block, column block) map and accumulator-register order as the producer.
 template <int kMT, int kNT>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, const int m_blocks) {
+  // uniform split: one workgroup per tile of the producer; tail split: one per tail tile (tiles full, full + 1, ...)
+  const bool tail = gg.tail_slices > 1;
+  const int wg = (tail ? gg.full : 0) + (int)blockIdx.x;
+  const int nslices = tail ? gg.tail_slices : gg.slices;
   GemmArgs a = gg.m[0];
   int blk_base = 0;
   for (int i = 1; i < gg.n; ++i)
-    if ((int)blockIdx.x >= gg.blk_end[i - 1]) {
+    if (wg >= gg.blk_end[i - 1]) {
       a = gg.m[i];
       blk_base = gg.blk_end[i - 1];
     }
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, lh = lane >> 5;
-  const int blk = (int)blockIdx.x - blk_base;
+  const int blk = wg - blk_base;
   const int m0 = (blk % m_blocks) * BM, bn = blk / m_blocks;
   const size_t slice_stride = (size_t)gridDim.x * (BM * BN);
   const float* part = gg.partials + (size_t)blockIdx.x * (BM * BN) + tid;
@@ -528,7 +550,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, co
       float v[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) v[i] = 0.f;
-      for (int z = 0; z < gg.slices; ++z) {
+      for (int z = 0; z < nslices; ++z) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) v[i] += part[(size_t)z * slice_stride + ((tm * kNT + tn) * 16 + i) * 256];
       }
@@ -556,13 +578,21 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
     gg.blk_end[i] = total;
   }
   if (!(kQuant && kSuper)) gg.slices = 1;
+  if (!(kQuant && kSuper) || gg.slices > 1 || gg.tail_slices < 2 || gg.full < 0 || gg.full >= total) gg.tail_slices = 0;
+  if (gg.tail_slices > 1) {
+    const int tail_tiles = total - gg.full;
+    hipLaunchKernelGGL(kern, dim3(gg.full + tail_tiles * gg.tail_slices, 1), dim3(256), lds, stream, gg, m_blocks);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(tail_tiles), dim3(256), 0, stream, gg, m_blocks);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(kern, dim3(total, gg.slices), dim3(256), lds, stream, gg, m_blocks);
   if (hipError_t e = hipGetLastError(); e != hipSuccess || gg.slices == 1) return e;
   hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(total), dim3(256), 0, stream, gg, m_blocks);
   return hipGetLastError();
 }
 
-static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stream) {
+static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, size_t ws_bytes, hipStream_t stream) {
   // Tile choice: the largest tile (most reuse of both operands) whose workgroup count still fills the chip; when
   // none does, the one with the most workgroups.  Row tiles are capped by M (and at 4: 8 spills), column tiles at
   // 2 per wave unless every member is narrow.
@@ -631,6 +661,34 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, hipStream_t stre
       gg.slices = (int)want;
     }
   }
+  // Tail split: the tiles beyond the last multiple of the CU count are cut along K so that the work they add is spread
+  // over the whole chip (2368 tiles on 256 CUs: 9.25 tiles' worth of time instead of 10; 288 tiles: 1.125 instead of 2).
+  // Only where that tail is at most 0.6 of a round, K leaves every slice two super-blocks or more, and the workspace
+  // holds the partial tiles.
+  static const int env_tail = getenv("GLOWQ_GEMM_TAIL") ? atoi(getenv("GLOWQ_GEMM_TAIL")) : 1;
+  gg.full = 0;
+  gg.tail_slices = 0;
+  if (super && env_tail != 0 && gg.slices == 1 && ws_bytes > 0) {
+    long tiles = 0;
+    for (int i = 0; i < gg.n; ++i) tiles += (long)((M + 32 * mt - 1) / (32 * mt)) * ((gg.m[i].N + 128 * nt - 1) / (128 * nt));
+    const long tail = tiles % num_cus;
+    const int sb_total = gg.m[0].K >> 8;
+    // (measured at 2048 rows: 2368 tiles 600 -> 596 us; 288 tiles 120 -> 128 us, and 112 with 64-row tiles: with about one
+    // tile per CU a second workgroup on a CU costs little, so there the split only adds its partials)
+    if (tiles >= 4L * num_cus && tail > 0 && tail * 10 <= (long)num_cus * 6) {
+      long s_want = num_cus / tail;
+      if (s_want > 8) s_want = 8;
+      if (s_want > sb_total / 2) s_want = sb_total / 2;
+      const size_t tile_bytes = (size_t)(32 * mt) * (128 * nt) * sizeof(float);
+      while (s_want >= 2 && (size_t)tail * s_want * tile_bytes > ws_bytes) --s_want;
+      if (s_want >= 2) {
+        // (slices of equal depth: no more of them than leave none empty)
+        const int per = (sb_total + (int)s_want - 1) / (int)s_want;
+        gg.tail_slices = (sb_total + per - 1) / per;
+        gg.full = (int)(tiles - tail);
+      }
+    }
+  }
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
   if (mt == MT && nt == NT)                                                                \
     return super ? launch_gemm_t<MT, NT, true, true>(gg, stream) : launch_gemm_t<MT, NT, true>(gg, stream);
@@ -690,7 +748,7 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
   const bool ws_ok = g.ws != nullptr && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0;
   gg.slices = ws_ok ? (int)std::min<size_t>(g.ws_bytes / (padded * sizeof(float)), 64) : 0;
   gg.partials = static_cast<float*>(g.ws);
-  return launch_gemm_group(gg, num_cus, stream);
+  return launch_gemm_group(gg, num_cus, ws_ok ? g.ws_bytes : 0, stream);
 }
 
 // ---- shared projection for many rows: r[M, rank] = fp16(x[M, K] . R[rank, K]^T) ---------------------------

@@ -624,7 +624,7 @@ class GreedyDecoder:
 
 def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, vocab: int = 128256, graph: bool = True,
             fused: bool = True, share: bool = True, correction: bool = True, attention_splits: int = 0,
-            chain=DEFAULT_CHAIN, module_glue: bool = True) -> dict:
+            chain=DEFAULT_CHAIN, module_glue: bool = True, model: Optional[Decoder] = None) -> dict:
     """Greedy decode of a random-init Llama-3.1-8B-shaped model at batch 1: time to the first token and tokens per
     second over the decode phase, the counterpart of `measure_generation_metrics` (src/step3_eval_dataset.py:705-798).
     `fused=False` decodes through the torch modules (CudaW4A16Linear / AddSVDCorrection inside the decoder's layers),
@@ -633,10 +633,12 @@ def measure(layers: int = 32, prompt_tokens: int = 512, new_tokens: int = 256, v
 
     os.environ.setdefault("W4A16_KERNEL_OUT_DTYPE", "fp16")
     refresh_env_knobs()
-    cfg = DecoderConfig(layers=layers, vocab=vocab, max_len=max(1024, prompt_tokens + new_tokens + 8))
     t0 = time.perf_counter()
-    model, _, _ = build_decoder(cfg, with_correction=correction)
-    torch.cuda.synchronize()
+    if model is None:  # (a caller that measures several paths builds the model once and hands it in)
+        cfg = DecoderConfig(layers=layers, vocab=vocab, max_len=max(1024, prompt_tokens + new_tokens + 8))
+        model, _, _ = build_decoder(cfg, with_correction=correction)
+        torch.cuda.synchronize()
+    cfg = model.cfg
     build_s = time.perf_counter() - t0
     dec = GreedyDecoder(model, use_graph=graph, fused=fused, share=share, attention_splits=attention_splits, chain=chain,
                         module_glue=module_glue)
