@@ -634,21 +634,35 @@ def library_path() -> str:
 
 def load_w4a16_extension(verbose: Optional[bool] = None) -> W4A16Extension:
     """Loads the prebuilt in-tree library (python -m glowq_amd.build).  Raises RuntimeError when it is
-    missing or does not load; nothing is compiled at run time and nothing falls back to torch."""
+    missing or does not load; nothing falls back to torch.  With W4A16_ALLOW_JIT=1 -- the reference's switch for
+    compiling its extension at run time when the prebuilt one is missing (src/cuda_w4a16/kernels.py:24-59) -- a
+    library that does not load is built once with hipcc (`glowq_amd.build.build`, about a minute) and loaded again."""
     global _ext
     if _ext is not None:
         return _ext
-    want_verbose = bool(verbose) or os.environ.get("W4A16_VERBOSE", os.environ.get("CUDA_MIXED_VERBOSE", "")).lower() in {
-        "1", "true", "yes", "y", "on"}
+    truthy = {"1", "true", "yes", "y", "on"}
+    want_verbose = bool(verbose) or os.environ.get("W4A16_VERBOSE", os.environ.get("CUDA_MIXED_VERBOSE", "")).lower() in truthy
+
+    def load():
+        return W4A16Extension(ctypes.CDLL(LIB_PATH))
+
     try:
-        lib = ctypes.CDLL(LIB_PATH)
-        ext = W4A16Extension(lib)
+        ext = load()
     except (OSError, AttributeError) as exc:
-        raise RuntimeError(
-            "Failed to load the prebuilt glowq W4A16 HIP library "
-            f"({LIB_PATH}). Build it first with:\n  python -m glowq_amd.build\n"
-            "There is no CPU or torch fallback for this path."
-        ) from exc
+        if os.environ.get("W4A16_ALLOW_JIT", "").lower() not in truthy:
+            raise RuntimeError(
+                "Failed to load the prebuilt glowq W4A16 HIP library "
+                f"({LIB_PATH}). Build it first with:\n  python -m glowq_amd.build\n"
+                "If you intentionally want it built at run time, set W4A16_ALLOW_JIT=1.\n"
+                "There is no CPU or torch fallback for this path."
+            ) from exc
+        from . import build as _build
+
+        _build.build(verbose=want_verbose)
+        try:
+            ext = load()
+        except (OSError, AttributeError) as exc2:
+            raise RuntimeError(f"Built the glowq W4A16 HIP library at run time, but it still does not load ({LIB_PATH})") from exc2
     if want_verbose:
         print(f"[glowq_amd] loaded {LIB_PATH} (version {ext.version})")
     _ext = ext

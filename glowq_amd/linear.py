@@ -236,6 +236,15 @@ class CudaW4A16Linear(nn.Module):
         self._require_gpu(self.qweight_i32)
         return self._get_ext().dequant(self.qweight_i32, self.scales_f16, self.qzeros_i32, self.in_features, self.group_size)
 
+    def _dequant_chunk(self, start: int, end: int) -> torch.Tensor:
+        """fp16 rows [start, end) of the dequantised weight, [end - start, in_features] (linear.py:248-253)."""
+        self._require_gpu(self.qweight_i32)
+        start, end = max(0, int(start)), min(self.out_features, int(end))
+        if end <= start:
+            return torch.empty((0, self.in_features), dtype=torch.float16, device=self.qweight_i32.device)
+        return self._get_ext().dequant(self.qweight_i32[start:end], self.scales_f16[start:end], self.qzeros_i32[start:end],
+                                       self.in_features, self.group_size)
+
     @classmethod
     def from_float(cls, linear_layer: nn.Linear, group_size: int):
         src = linear_layer.weight

@@ -158,3 +158,20 @@ def test_state_dict_round_trip_on_device(fp16_out):
     b.load_state_dict(a.state_dict())
     x = torch.randn(2, 256).half().cuda()
     assert torch.equal(a(x), b(x))
+
+
+def test_dequant_chunk_rows_match_the_reference_vectors(golden):
+    """`_dequant_chunk(start, end)` (src/cuda_w4a16/linear.py:248-253): rows of the dequantised weight, bit for bit
+    against what the reference's own method returned for the whole matrix."""
+    from glowq_amd.linear import CudaW4A16Linear
+
+    gs = int(golden["m2_gs"][0])
+    n, k = golden["m2_w"].shape
+    mod = CudaW4A16Linear(k, n, gs, bias=False).cuda()
+    mod.qweight_i32.copy_(torch.from_numpy(golden["m2_qweight"]))
+    mod.scales_f16.copy_(torch.from_numpy(golden["m2_scales"]))
+    mod.qzeros_i32.copy_(torch.from_numpy(golden["m2_qzeros"]))
+    want = golden["m2_deq"]
+    for start, end in ((0, n), (3, 17), (n - 1, n), (5, 5), (30, n + 10)):
+        got = mod._dequant_chunk(start, end).cpu().numpy()
+        np.testing.assert_array_equal(got.view(np.uint16), want[start:min(end, n)].view(np.uint16))

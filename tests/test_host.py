@@ -343,5 +343,32 @@ def test_tensor_front_end_checks():
 def test_missing_library_raises(monkeypatch):
     monkeypatch.setattr(kernels, "_ext", None)
     monkeypatch.setattr(kernels, "LIB_PATH", "/nonexistent/libglowq_w4a16.so")
+    monkeypatch.delenv("W4A16_ALLOW_JIT", raising=False)
     with pytest.raises(RuntimeError, match="python -m glowq_amd.build"):
         kernels.load_w4a16_extension()
+
+
+def test_allow_jit_builds_a_missing_library_once(monkeypatch):
+    """W4A16_ALLOW_JIT=1 (src/cuda_w4a16/kernels.py:24-59): a library that does not load is built and loaded again; the
+    build itself is stubbed here (it takes a minute), once leaving the library missing and once putting it in place."""
+    from glowq_amd import build as build_mod
+
+    real = kernels.LIB_PATH
+    calls = []
+    monkeypatch.setattr(kernels, "_ext", None)
+    monkeypatch.setattr(kernels, "LIB_PATH", "/nonexistent/libglowq_w4a16.so")
+    monkeypatch.setenv("W4A16_ALLOW_JIT", "1")
+    monkeypatch.setattr(build_mod, "build", lambda verbose=False, extra_flags=(): calls.append("build"))
+    with pytest.raises(RuntimeError, match="still does not load"):
+        kernels.load_w4a16_extension()
+    assert calls == ["build"]
+
+    def fake_build(verbose=False, extra_flags=()):
+        calls.append("build")
+        monkeypatch.setattr(kernels, "LIB_PATH", real)
+
+    monkeypatch.setattr(build_mod, "build", fake_build)
+    monkeypatch.setattr(kernels, "LIB_PATH", "/nonexistent/libglowq_w4a16.so")
+    ext = kernels.load_w4a16_extension()
+    assert calls == ["build", "build"] and ext.version >= 100
+    monkeypatch.setattr(kernels, "_ext", None)
