@@ -522,6 +522,8 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
 
 // y = fp16(sum over the slices, in slice order, of the partial tiles of gemm_mfma_kernel<kMT, kNT> + bias); same grid
 // in x, same workgroup -> (member, row block, column block) map and accumulator-register order as the producer.
+// gridDim.y = kMT * kNT: workgroup y of a tile sums one 32 x 32 accumulator tile of each wave (a tile per workgroup
+// left the sum of 64 tail tiles to 64 workgroups: 20 us for 34 MB).
 template <int kMT, int kNT>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, const int m_blocks) {
   // uniform split: one workgroup per tile of the producer; tail split: one per tail tile (tiles full, full + 1, ...)
@@ -541,12 +543,11 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, co
   const int m0 = (blk % m_blocks) * BM, bn = blk / m_blocks;
   const size_t slice_stride = (size_t)gridDim.x * (BM * BN);
   const float* part = gg.partials + (size_t)blockIdx.x * (BM * BN) + tid;
-#pragma unroll
-  for (int tn = 0; tn < kNT; ++tn) {
+  const int tn = (int)blockIdx.y % kNT, tm = (int)blockIdx.y / kNT;
+  {
     const int n = bn * BN + wave * (32 * kNT) + tn * 32 + ln;
     const float b = (n < a.N && a.bias) ? (float)a.bias[n] : 0.f;
-#pragma unroll
-    for (int tm = 0; tm < kMT; ++tm) {
+    {
       float v[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) v[i] = 0.f;
@@ -583,12 +584,12 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
     const int tail_tiles = total - gg.full;
     hipLaunchKernelGGL(kern, dim3(gg.full + tail_tiles * gg.tail_slices, 1), dim3(256), lds, stream, gg, m_blocks);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-    hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(tail_tiles), dim3(256), 0, stream, gg, m_blocks);
+    hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(tail_tiles, kMT * kNT), dim3(256), 0, stream, gg, m_blocks);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(kern, dim3(total, gg.slices), dim3(256), lds, stream, gg, m_blocks);
   if (hipError_t e = hipGetLastError(); e != hipSuccess || gg.slices == 1) return e;
-  hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(total), dim3(256), 0, stream, gg, m_blocks);
+  hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(total, kMT * kNT), dim3(256), 0, stream, gg, m_blocks);
   return hipGetLastError();
 }
 
@@ -673,9 +674,8 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, size_t ws_bytes,
     for (int i = 0; i < gg.n; ++i) tiles += (long)((M + 32 * mt - 1) / (32 * mt)) * ((gg.m[i].N + 128 * nt - 1) / (128 * nt));
     const long tail = tiles % num_cus;
     const int sb_total = gg.m[0].K >> 8;
-    // (measured at 2048 rows: 2368 tiles 600 -> 596 us; 288 tiles 120 -> 128 us, and 112 with 64-row tiles: with about one
-    // tile per CU a second workgroup on a CU costs little, so there the split only adds its partials)
-    if (tiles >= 4L * num_cus && tail > 0 && tail * 10 <= (long)num_cus * 6) {
+    // (measured at 2048 rows, projection launch included: 2368 tiles 590 -> 573 us, 288 tiles 119 -> 107 us)
+    if (tiles > num_cus && tail > 0 && tail * 10 <= (long)num_cus * 6) {
       long s_want = num_cus / tail;
       if (s_want > 8) s_want = 8;
       if (s_want > sb_total / 2) s_want = sb_total / 2;

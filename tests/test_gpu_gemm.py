@@ -243,3 +243,50 @@ def test_gemm_split_k_through_workspace(ext, M, K, Ns, rank):
         seen[nbytes] = [o.clone() for o in outs]
     ext.WORKSPACE_BYTES = 64 << 20
     ext._workspaces.clear()
+
+
+@pytest.mark.parametrize("M,K,Ns,rank", [(384, 2048, [16384, 5120, 1024], 64), (200, 1024, [40000], 0), (2048, 3584, [3584, 512, 512], 128)])
+def test_gemm_tail_tiles_split_along_k(ext, M, K, Ns, rank):
+    """More output tiles than CUs, with a partly filled last round: the tiles of that round are cut along K (partials in
+    the workspace, summed by a second launch).  Sampled rows and the columns of the first and of the last tiles of every
+    member against the oracle; the same bits on a second call; and the unsplit launch (no workspace) within tolerance."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).half().numpy()
+    R = (torch.randn(rank, K, generator=g) * K ** -0.5).half().numpy() if rank else None
+    rows = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(M).integers(0, M, 6)]))
+    mem, checks = [], []
+    for N in Ns:
+        w = (torch.randn(N, K, generator=g) * 0.02).half().numpy()
+        qw, qz, sc, _ = oracle.quantize_per_group_w4(w, 128)
+        L = (torch.randn(N, rank, generator=g) * 0.01).half().numpy() if rank else None
+        bias = (torch.randn(N, generator=g) * 0.1).half().numpy()
+        mem.append({"qweight": dev(qw), "scales": dev(sc), "qzeros": dev(qz), "L": dev(L) if rank else None, "bias": dev(bias)})
+        cols = np.unique(np.concatenate([np.arange(0, min(N, 300)), np.arange(max(0, N - 600), N)]))
+        xs = x[rows]
+        if rank:
+            want = oracle.corrected_linear_exact(xs, qw[cols], qz[cols], sc[cols], 128, R, L[cols], 1.0)
+        else:
+            want = oracle.linear_exact(xs, qw[cols], qz[cols], sc[cols], 128)
+        checks.append((cols, want + bias[cols].astype(np.float64)[None, :]))
+    xd = dev(x)
+    r = ext.shared_proj(xd, dev(R)) if rank else None
+    outs = ext.group_forward(xd, r, mem, 128, 1.0)
+    torch.cuda.synchronize()
+    for i, (y, (cols, want)) in enumerate(zip(outs, checks)):
+        assert_close(y.cpu().numpy()[np.ix_(rows, cols)], want, f"member {i}")
+    again = ext.group_forward(xd, r, mem, 128, 1.0)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(outs, again))
+    saved = ext.WORKSPACE_BYTES, dict(ext._workspaces)
+    try:
+        ext.WORKSPACE_BYTES = 16
+        ext._workspaces.clear()
+        plain = ext.group_forward(xd, r, mem, 128, 1.0)
+        torch.cuda.synchronize()
+        for i, (y, (cols, want)) in enumerate(zip(plain, checks)):
+            assert_close(y.cpu().numpy()[np.ix_(rows, cols)], want, f"member {i} without a workspace")
+    finally:
+        ext.WORKSPACE_BYTES = saved[0]
+        ext._workspaces.clear()
+        ext._workspaces.update(saved[1])
