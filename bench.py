@@ -301,6 +301,11 @@ def selective_leg(torch, ext, dev):
                     else:
                         plain(n, li)
 
+        # fraction of the HBM peak per group: algorithmic bytes of the call (with R, L and r where corrected) over its time
+        entry["corrected_pct_hbm_peak"] = {n: round(100.0 * algorithmic_bytes(rows, K, sum(Ns), SELECTIVE_RANK) / entry["corrected_us"][n] / 1e6 / (HBM_PEAK_GBPS / 1e3), 1)
+                                           for n, (K, Ns) in SELECTIVE_GROUPS.items()}
+        entry["plain_pct_hbm_peak"] = {n: round(100.0 * algorithmic_bytes(rows, K, sum(Ns), 0) / entry["plain_us"][n] / 1e6 / (HBM_PEAK_GBPS / 1e3), 1)
+                                       for n, (K, Ns) in SELECTIVE_GROUPS.items()}
         entry["all_corrected_us_per_layer"] = round(sum(entry["corrected_us"].values()), 2)
         entry["none_corrected_us_per_layer"] = round(sum(entry["plain_us"].values()), 2)
         entry["half_selected_us_per_layer"] = round(timed(half) / SELECTIVE_LAYERS, 2)

@@ -223,3 +223,92 @@ def test_opt13b_qkv_group_through_the_modules(monkeypatch):
 
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp16")    # smoke() sets it; restored when the test ends
     __graft_entry__.smoke()
+
+
+@pytest.mark.parametrize("model", ["llama8b", "qwen14b"])
+def test_chained_layer_at_full_size(ext, model):
+    """o_proj -> (norm launch) -> gate|up -> down_proj -> next q|k|v through the chained single-token launches at the
+    layer's own shapes (Llama-3.1-8B: rank 128, K = 4096 / 14336; Qwen3-14B: rank 256, K = 5120 / 17408), both chain
+    modes: sampled output rows of every launch against the oracle on the launch's own inputs, the residual stream and
+    the gated activations against the oracle's residual add and SwiGLU of the launch's own outputs, the accumulators
+    against the projection of the launch's own outputs."""
+    from glowq_amd.kernels import (CHAIN_ACC_BYTES, CHAIN_EPI_NONE, CHAIN_EPI_RESIDUAL, CHAIN_EPI_SWIGLU, CHAIN_PRO_ACC,
+                                   CHAIN_PRO_NORM_ACC, CHAIN_PRO_PLAIN, PreparedGroup)
+
+    rank, shapes = MODELS[model]
+    H, I = shapes["o"][0], shapes["down"][0]
+    eps = 1e-6
+    g = torch.Generator(device="cuda").manual_seed(99)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    layers = {n: _layer(model, n, 1, 700 + i) for i, n in enumerate(GROUPS)}
+    pg = {n: PreparedGroup(ext, layers[n][2], shapes[n][0], GS, 1.0) for n in GROUPS}
+    R = {n: layers[n][1] for n in GROUPS}
+    Rt = {n: R[n].t().contiguous() for n in GROUPS}
+    ln2 = (1 + 0.1 * torch.randn(H, device="cuda", generator=g)).half()
+    ln1n = (1 + 0.1 * torch.randn(H, device="cuda", generator=g)).half()
+    attn = layers["o"][0][0].contiguous()
+    x_res0 = (torch.randn(H, device="cuda", generator=g) * 2).half()
+
+    def acc_p(acc):
+        words = acc.cpu().numpy().view(np.int64)
+        assert words[16 * 256] == 0
+        return words[:16 * 256].reshape(16, 256)[:, :rank].sum(axis=0).astype(np.float64) * 2.0 ** -32
+
+    def check_rows(name, x, outs_or_none, r64=None):
+        """Sampled rows of a launch's own outputs (where it wrote them) against the oracle."""
+        for mem, y in zip(layers[name][2], outs_or_none):
+            rows = _sample_rows(mem["qweight"].size(0), 5)
+            want = _oracle_rows(x[None, :], R[name], mem, rows, "stream_gemv")[0]
+            assert_close(y.cpu().numpy()[rows], want, f"{model} {name}")
+
+    for mode in ("full", "mlp"):
+        print(f"{model} chain mode {mode}", flush=True)
+        acc_o, acc_gu, acc_dn = (torch.zeros(CHAIN_ACC_BYTES, dtype=torch.uint8, device="cuda") for _ in range(3))
+        xr = x_res0.clone()
+        r_o = ext.shared_proj(attn[None, :], R["o"])[0]
+        o_y = torch.zeros(H, **f16)
+        if mode == "full":
+            pg["o"].run_chained(attn, CHAIN_PRO_PLAIN, CHAIN_EPI_RESIDUAL, r=r_o, outs=[o_y], resid=xr, next_norm_weight=ln2,
+                                next_Rt=Rt["gate_up"], acc_out=acc_o)
+            torch.cuda.synchronize()
+            check_rows("o", attn, [o_y])
+            np.testing.assert_array_equal(xr.cpu().numpy().view(np.uint16),
+                                          oracle.residual_add(x_res0.cpu().numpy(), o_y.cpu().numpy()).view(np.uint16))
+            c = ln2.double().cpu().numpy() * xr.double().cpu().numpy()
+            want_p = R["gate_up"].double().cpu().numpy() @ c
+            np.testing.assert_allclose(acc_p(acc_o), want_p, rtol=0, atol=2e-6 * (np.abs(R["gate_up"].double().cpu().numpy()) @ np.abs(c)).max() + 1e-6)
+            x_after_o = xr.clone()
+            gate_y, up_y, act = torch.zeros(I, **f16), torch.zeros(I, **f16), torch.zeros(I, **f16)
+            pg["gate_up"].run_chained(xr, CHAIN_PRO_NORM_ACC, CHAIN_EPI_SWIGLU, outs=[gate_y, up_y], norm_weight=ln2, eps=eps,
+                                      acc_in=acc_o, act=act, next_Rt=Rt["down"], acc_out=acc_gu)
+            h = torch.from_numpy(oracle.rmsnorm(x_after_o.cpu().numpy()[None, :], ln2.cpu().numpy(), eps)[0]).cuda()
+        else:
+            o_plain = pg["o"].run(attn[None, :], r=r_o[None, :], project=False)[0]
+            x_after_o, h2d, r_gu = torch.zeros(1, H, **f16), torch.zeros(1, H, **f16), torch.zeros(1, rank, **f16)
+            ext.add_rmsnorm_proj(xr[None, :], o_plain, ln2, x_after_o, h2d, R["gate_up"], r_gu, eps)
+            xr = x_after_o[0].clone()
+            x_after_o = xr.clone()
+            h = h2d[0]
+            gate_y, up_y, act = torch.zeros(I, **f16), torch.zeros(I, **f16), torch.zeros(I, **f16)
+            pg["gate_up"].run_chained(h, CHAIN_PRO_PLAIN, CHAIN_EPI_SWIGLU, r=r_gu[0], outs=[gate_y, up_y], act=act,
+                                      next_Rt=Rt["down"], acc_out=acc_gu)
+        torch.cuda.synchronize()
+        check_rows("gate_up", h, [gate_y, up_y])
+        ref_act = oracle.swiglu(gate_y.cpu().numpy(), up_y.cpu().numpy()).astype(np.float64)
+        got_act = act.double().cpu().numpy()
+        # (the hardware exponential and reciprocal can move fp16(silu(g)) by one fp16 ulp, the product's rounding adds half)
+        assert np.all(np.abs(got_act - ref_act) <= 2.0 ** -9 * np.abs(ref_act) + 1e-7)
+        want_p = R["down"].double().cpu().numpy() @ got_act
+        np.testing.assert_allclose(acc_p(acc_gu), want_p, rtol=0, atol=2e-6 * (np.abs(R["down"].double().cpu().numpy()) @ np.abs(got_act)).max() + 1e-6)
+        dn_y = torch.zeros(H, **f16)
+        pg["down"].run_chained(act, CHAIN_PRO_ACC, CHAIN_EPI_RESIDUAL, acc_in=acc_gu, outs=[dn_y], resid=xr, next_norm_weight=ln1n,
+                               next_Rt=Rt["qkv"], acc_out=acc_dn)
+        torch.cuda.synchronize()
+        check_rows("down", act, [dn_y])
+        np.testing.assert_array_equal(xr.cpu().numpy().view(np.uint16),
+                                      oracle.residual_add(x_after_o.cpu().numpy(), dn_y.cpu().numpy()).view(np.uint16))
+        qkv_y = [torch.zeros(N, **f16) for N in shapes["qkv"][1]]
+        pg["qkv"].run_chained(xr, CHAIN_PRO_NORM_ACC, CHAIN_EPI_NONE, outs=qkv_y, norm_weight=ln1n, eps=eps, acc_in=acc_dn)
+        torch.cuda.synchronize()
+        h_next = torch.from_numpy(oracle.rmsnorm(xr.cpu().numpy()[None, :], ln1n.cpu().numpy(), eps)[0]).cuda()
+        check_rows("qkv", h_next, qkv_y)
