@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libglowq_w4a16.so")
-SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_chain.hip", "gemv_quad.hip", "skinny.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
+SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_chain.hip", "gemv_quad.hip", "gemv_qstream.hip", "skinny.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
 ARCH = "gfx950"
 
 HIPCC_FLAGS = [
@@ -44,7 +44,8 @@ def _hipcc() -> str:
 # Sources whose kernels keep loads in flight that the compiler does not track (inline assembly with hand-placed waits):
 # a register spilled there would be stored before its load has returned, so these must compile without scratch memory,
 # and their assembly must not touch a register of a load that is still outstanding (isa_lint.py).
-NO_SCRATCH = {"gemv_stream.hip": "gemv_stream_kernel", "gemv_chain.hip": "gemv_stream_kernel"}
+NO_SCRATCH = {"gemv_stream.hip": "gemv_stream_kernel", "gemv_chain.hip": "gemv_stream_kernel",
+              "gemv_qstream.hip": "gemv_qstream_kernel"}
 
 
 def _check_no_scratch(src: str, kernel: str, remarks: str) -> None:

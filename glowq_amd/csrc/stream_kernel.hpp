@@ -127,6 +127,11 @@ __device__ __forceinline__ void wait_vm(u32x4& a, u32x4& b, int& idx) {
   asm volatile("s_waitcnt vmcnt(%3)" : "+v"(a), "+v"(b), "+v"(idx) : "n"(kN) : "memory");
 }
 template <int kN>
+__device__ __forceinline__ void wait_vm(u32x4& a, int& idx) {
+  static_assert(kN >= 0 && kN <= 63, "vmcnt is a 6-bit field");
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(idx) : "n"(kN) : "memory");
+}
+template <int kN>
 __device__ __forceinline__ void wait_vm(uint32_t& a) {
   static_assert(kN >= 0 && kN <= 63, "vmcnt is a 6-bit field");
   asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(kN) : "memory");

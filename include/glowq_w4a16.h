@@ -191,7 +191,8 @@ size_t glowq_static_scratch_bytes(void);
 /*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
  * 2 = tiled MFMA GEMM, 3 = generic (odd shapes), 4 = 4x4x4 matrix-core GEMV, 5 = stream GEMV (every request of a
- * wave in flight up front; the default at one token row).
+ * wave in flight up front; the default at one token row), 6 = the 4x4x4 matrix-core GEMV under the stream GEMV's
+ * memory schedule (the default at two to four token rows).
  */
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
 
@@ -206,8 +207,13 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * "stream_max_m" (0..4): token rows up to which the stream GEMV is used where its layout applies, ahead of the
  * others; 0 switches it off.  "stream_shape_rule" (0 / 1): with more than one token row, only for the shapes it was
  * measured faster on (1, the default) or for every shape (0).
+ * "qstream_max_m" (0..8, default 4): token rows, from two, up to which the stream-scheduled 4x4x4 matrix-core GEMV
+ * is used where it applies (groups of 128 to 2048 columns, rank a multiple of 8 up to 128 or of 16 up to 256, rows
+ * up to 16384 columns), ahead of all others; 0 switches it off.  "qstream_shape_rule" (0 / 1): only for the shapes it
+ * was measured faster on (1, the default) or for every shape it can take (0).
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
- * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M and GLOWQ_STREAM_SHAPE_RULE.
+ * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M, GLOWQ_STREAM_SHAPE_RULE,
+ * GLOWQ_QSTREAM_M and GLOWQ_QSTREAM_SHAPE_RULE.
  */
 int glowq_set_tuning(const char* key, int value);
 

@@ -27,20 +27,28 @@ def golden():
     return np.load(os.path.join(ROOT, "tests", "golden", "w4a16_golden.npz"))
 
 
-@pytest.fixture(params=["stream", "quad", "classic"])
+@pytest.fixture(params=["stream", "qstream", "quad", "classic"])
 def small_m_route(request, ext):
-    """Runs a test with the stream GEMV serving 1..4 token rows (the other kernels above), with the 4x4x4 matrix-core GEMV
-    serving 1..16 token rows, and with both switched off (wave-dot GEMV for 1..4 rows, skinny MFMA kernel above)."""
-    if request.param == "stream":
-        old = ext.set_tuning("stream_max_m", 4), ext.set_tuning("stream_shape_rule", 0)
+    """Runs a test with the stream GEMV serving 1..4 token rows (the other kernels above), with the stream-scheduled 4x4x4
+    matrix-core GEMV serving 2..8 token rows, with the 4x4x4 matrix-core GEMV serving 1..16 token rows, and with all
+    switched off (wave-dot GEMV for 1..4 rows, skinny MFMA kernel above)."""
+    if request.param == "qstream":
+        old = ext.set_tuning("qstream_max_m", 8), ext.set_tuning("qstream_shape_rule", 0)
         yield request.param
-        ext.set_tuning("stream_max_m", old[0]), ext.set_tuning("stream_shape_rule", old[1])
+        ext.set_tuning("qstream_max_m", old[0]), ext.set_tuning("qstream_shape_rule", old[1])
+        return
+    if request.param == "stream":
+        old = ext.set_tuning("stream_max_m", 4), ext.set_tuning("stream_shape_rule", 0), ext.set_tuning("qstream_max_m", 0)
+        yield request.param
+        ext.set_tuning("stream_max_m", old[0]), ext.set_tuning("stream_shape_rule", old[1]), ext.set_tuning("qstream_max_m", old[2])
         return
     old = ext.set_tuning("quad_max_m", 16 if request.param == "quad" else 0)
     old_min = ext.set_tuning("quad_min_m", 1)
     old_small = ext.set_tuning("small_group_mb", 0)  # no shape-dependent choice between the two at 2..4 rows
     old_stream = ext.set_tuning("stream_max_m", 0)   # the stream GEMV would take the single rows of both modes
+    old_qstream = ext.set_tuning("qstream_max_m", 0)
     yield request.param
+    ext.set_tuning("qstream_max_m", old_qstream)
     ext.set_tuning("quad_max_m", old)
     ext.set_tuning("quad_min_m", old_min)
     ext.set_tuning("small_group_mb", old_small)

@@ -81,7 +81,7 @@ def test_group_forward_large_m(ext, M, K, Ns, rank, alpha):
                                       (8, 2816, 200, 128), (24, 5632, 96, 128), (16, 18944, 64, 128), (40, 2304, 72, 128)])
 def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     print(f"case M={M} K={K} N={N} gs={gs}", flush=True)
-    if small_m_route != "stream":  # the stream mode leaves the limits of the kernels above 4 rows at their defaults
+    if small_m_route not in ("stream", "qstream"):  # those modes leave the limits of the other kernels at their defaults
         assert ext.lib.glowq_w4a16_route(M, K, N, gs, K // 8) == (4 if small_m_route == "quad" and M <= 16 else 1)
     x, (m,), _ = make_group(41 + M + N, M, K, [N], 0, group_size=gs)
     y = ext.w4a16_gemv_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs)
@@ -121,20 +121,25 @@ def test_skinny_split_k_through_workspace(ext, M, K, Ns, rank):
         ext._workspaces.update(saved[1])
 
 
-@pytest.mark.parametrize("stream", [True, False], ids=["stream", "no_stream"])
+@pytest.mark.parametrize("mode", ["default", "stream", "neither"])
 @pytest.mark.parametrize("M,K,Ns,rank", [(3, 4096, [512, 128, 128], 128), (4, 2048, [300], 64), (4, 5632, [96, 40], 128), (2, 4096, [256], 128)])
-def test_small_groups_at_two_to_four_rows(ext, stream, M, K, Ns, rank):
-    """Default route limits: a small group at two to four rows runs on the stream GEMV; with that one switched off, at
-    three or four rows on the skinny MFMA kernel and at two rows on the wave-dot GEMV.  All against the oracle, with
-    the shared correction."""
-    print(f"case M={M} K={K} Ns={Ns} rank={rank} stream={stream}", flush=True)
-    old = None if stream else ext.set_tuning("stream_max_m", 0)
+def test_small_groups_at_two_to_four_rows(ext, mode, M, K, Ns, rank):
+    """Default route limits: a small group at two to four rows runs on the stream-scheduled 4x4x4 matrix-core GEMV; with
+    that one switched off on the stream GEMV; with both off, at three or four rows on the skinny MFMA kernel and at two
+    rows on the wave-dot GEMV.  All against the oracle, with the shared correction."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank} mode={mode}", flush=True)
+    old = {}
+    if mode != "default":
+        old["qstream_max_m"] = ext.set_tuning("qstream_max_m", 0)
+    if mode == "neither":
+        old["stream_max_m"] = ext.set_tuning("stream_max_m", 0)
     try:
-        assert ext.lib.glowq_w4a16_route(M, K, sum(Ns), 128, K // 8) == (5 if stream else 0 if M == 2 else 1)
+        want = {"default": 6, "stream": 5, "neither": 0 if M == 2 else 1}[mode]
+        assert ext.lib.glowq_w4a16_route(M, K, sum(Ns), 128, K // 8) == want
         _small_group_case(ext, M, K, Ns, rank)
     finally:
-        if old is not None:
-            ext.set_tuning("stream_max_m", old)
+        for key, value in old.items():
+            ext.set_tuning(key, value)
 
 
 def _small_group_case(ext, M, K, Ns, rank):

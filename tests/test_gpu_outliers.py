@@ -20,7 +20,7 @@ from helpers import ABS_TOL, REL_TOL, dev, make_group, outlier_activations
 
 pytestmark = pytest.mark.gpu
 
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv"}
 
 # (token rows, K, member widths, rank, route mode); the default limits send 1 row to the wave-dot GEMV, 2..4 rows to the
 # wave-dot GEMV, the 4x4x4 GEMV or the skinny kernel by group size, 5..64 to the skinny kernel, more to the tiled GEMM
@@ -30,7 +30,8 @@ CASES = [
     (2, 4096, [4096], 128, "default"), (2, 14336, [8192], 128, "default"),
     (3, 2048, [300], 64, "default"), (4, 4096, [2048, 2048], 64, "default"),
     (4, 4096, [2048, 2048], 64, "quad"), (4, 4096, [2048, 2048], 64, "classic"),
-    (8, 4096, [512], 128, "default"), (8, 4096, [512], 128, "quad"),
+    (8, 4096, [512], 128, "default"), (8, 4096, [512], 128, "quad"), (8, 4096, [512], 128, "qstream"),
+    (4, 14336, [8192], 128, "qstream"), (3, 4096, [2048, 2048], 256, "qstream"),
     (16, 14336, [256], 128, "default"), (16, 4096, [1024, 256], 128, "quad"),
     (64, 4096, [512, 96], 256, "default"), (130, 2048, [512], 128, "default"), (300, 4096, [256, 128], 128, "default"),
 ]
@@ -46,9 +47,14 @@ def tuned(ext):
         if mode == "stream":
             saved["stream_max_m"] = ext.set_tuning("stream_max_m", 4)
             saved["stream_shape_rule"] = ext.set_tuning("stream_shape_rule", 0)
+            saved["qstream_max_m"] = ext.set_tuning("qstream_max_m", 0)
+            return
+        if mode == "qstream":
+            saved["qstream_max_m"] = ext.set_tuning("qstream_max_m", 8)
+            saved["qstream_shape_rule"] = ext.set_tuning("qstream_shape_rule", 0)
             return
         for key, value in (("quad_max_m", 16 if mode == "quad" else 0), ("quad_min_m", 1), ("small_group_mb", 0),
-                           ("stream_max_m", 0)):
+                           ("stream_max_m", 0), ("qstream_max_m", 0)):
             saved[key] = ext.set_tuning(key, value)
 
     yield apply

@@ -12,7 +12,8 @@ from helpers import assert_close, dev, make_group
 pytestmark = pytest.mark.gpu
 
 ROWS = [1, 2, 3, 4, 5, 7, 8, 13, 16, 17, 31, 32, 33, 48, 64, 65, 100, 130, 257]
-ROUTES = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv", 5: "stream_gemv"}
+ROUTES = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv", 5: "stream_gemv",
+          6: "quad_stream_gemv"}
 
 
 def random_cases(n, seed=20240):
@@ -43,23 +44,28 @@ def random_cases(n, seed=20240):
     return cases
 
 
-@pytest.fixture(params=["default", "stream", "quad", "classic"])
+@pytest.fixture(params=["default", "stream", "qstream", "quad", "classic"])
 def route_mode(request, ext):
-    """The library's own route limits, the stream GEMV for every case of 1..4 rows it can take, the 4x4x4 matrix-core
-    GEMV for every case of 1..16 rows it can take, or both switched off (wave-dot GEMV up to 4 rows, skinny MFMA kernel
-    above)."""
+    """The library's own route limits, the stream GEMV for every case of 1..4 rows it can take, the stream-scheduled
+    4x4x4 matrix-core GEMV for every case of 2..8 rows it can take, the 4x4x4 matrix-core GEMV for every case of 1..16
+    rows it can take, or all switched off (wave-dot GEMV up to 4 rows, skinny MFMA kernel above)."""
     if request.param == "default":
         yield request.param
         return
-    if request.param == "stream":
-        old = ext.set_tuning("stream_max_m", 4), ext.set_tuning("stream_shape_rule", 0)
+    if request.param == "qstream":
+        old = ext.set_tuning("qstream_max_m", 8), ext.set_tuning("qstream_shape_rule", 0)
         yield request.param
-        ext.set_tuning("stream_max_m", old[0]), ext.set_tuning("stream_shape_rule", old[1])
+        ext.set_tuning("qstream_max_m", old[0]), ext.set_tuning("qstream_shape_rule", old[1])
+        return
+    if request.param == "stream":
+        old = ext.set_tuning("stream_max_m", 4), ext.set_tuning("stream_shape_rule", 0), ext.set_tuning("qstream_max_m", 0)
+        yield request.param
+        ext.set_tuning("stream_max_m", old[0]), ext.set_tuning("stream_shape_rule", old[1]), ext.set_tuning("qstream_max_m", old[2])
         return
     old = [ext.set_tuning("quad_max_m", 16 if request.param == "quad" else 0), ext.set_tuning("quad_min_m", 1),
-           ext.set_tuning("small_group_mb", 0), ext.set_tuning("stream_max_m", 0)]
+           ext.set_tuning("small_group_mb", 0), ext.set_tuning("stream_max_m", 0), ext.set_tuning("qstream_max_m", 0)]
     yield request.param
-    for key, value in zip(("quad_max_m", "quad_min_m", "small_group_mb", "stream_max_m"), old):
+    for key, value in zip(("quad_max_m", "quad_min_m", "small_group_mb", "stream_max_m", "qstream_max_m"), old):
         ext.set_tuning(key, value)
 
 
