@@ -25,7 +25,7 @@ hipError_t launch_stream_chained(GroupDev& g, const streamk::ChainDev& ch, int p
 int quad_capacity(int M, int K, int rank, bool has_r);
 hipError_t launch_quad(GroupDev& g, int num_cus, hipStream_t stream);
 bool qstream_supported(const GroupDev& g);
-hipError_t launch_qstream(GroupDev& g, hipStream_t stream);
+hipError_t launch_qstream(GroupDev& g, int num_cus, hipStream_t stream);
 // misc.hip
 hipError_t launch_dequant(const int32_t*, const half_t*, const int32_t*, half_t*, int, int, int, int, int, int, int,
                           hipStream_t);
@@ -233,18 +233,18 @@ std::atomic<int> g_qstream_shape_rule{clampi(env_or("GLOWQ_QSTREAM_SHAPE_RULE", 
 // Group launch alone, us, this kernel / the route taken without it (6 to 32 layers of distinct weights back to back):
 //   four rows   4096 x 4096: 4.7 / 6.9   6144 x 4096 (q|k|v): 6.7 / 7.8   28672 x 4096: 16.2 / 18.7   4096 x 14336: 11.7 / 14.5
 //               4096 x 11008: 9.4 / 13.4   8192 x 8192: 10.9 / 14.2   10240 x 8192: 14.2 / 19.6   37888 x 3584: 19.9 / 23.4
-//               7168 x 5120: 9.7 / 12.3   5120 x 5120: 9.7 / 9.3   34816 x 5120: 34.4 / 31.7   28672 x 6144: 31.2 / 25.0
+//               7168 x 5120: 9.6 / 12.2   5120 x 5120: 8.2 / 9.3   34816 x 5120: 34.4 / 31.7   28672 x 6144: 31.2 / 25.0
 //   two rows    4096 x 4096: 4.6 / 5.1   6144 x 4096: 6.2 / 6.2   28672 x 4096: 14.3 / 15.9   4096 x 14336: 10.5 / 10.7
-//               5120 x 5120: 8.5 / 7.3   34816 x 5120: 27.0 / 26.7   10240 x 8192: 13.1 / 12.7
+//               5120 x 5120: 7.5 / 7.3   34816 x 5120: 27.0 / 26.7   10240 x 8192: 13.1 / 12.7
 // Every workgroup stages the whole activation rows for its 16 output rows: long rows with many workgroups per compute
-// unit pay for that (the persistent 4x4x4 kernel stages once per compute unit), and so does a last slice that is
-// mostly empty (K = 5120: 2.5 slices of 2048 columns).
+// unit pay for that (the persistent 4x4x4 kernel stages once per compute unit); at two rows a last slice that is mostly
+// empty (K = 5120: 2.5 slices of 2048 columns) is enough to fall behind the stream GEMV.
 bool qstream_pays(const GroupDev& g) {
   if (g_qstream_shape_rule.load(std::memory_order_relaxed) == 0) return true;
   long rows = 0;
   for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
   const int padded = (g.K + 2047) / 2048 * 2048;
-  if ((padded - g.K) * 100 > 15 * g.K) return false;
+  if (g.M == 2 && (padded - g.K) * 100 > 15 * g.K) return false;  // (level with the stream GEMV or behind it there)
   if (g.K > 4096 && rows >= 16384) return false;
   return true;
 }
@@ -304,7 +304,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   if (route == kRouteStream) {
     e = launch_stream(g, cus, stream);
   } else if (route == kRouteQStream) {
-    e = launch_qstream(g, stream);
+    e = launch_qstream(g, cus, stream);
   } else if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
   } else if (route == kRouteSkinny) {

@@ -371,7 +371,8 @@ struct QsPlan {
   size_t lds;
 };
 
-bool qs_plan(int M, int K, int rank, bool has_r, QsPlan& p) {
+// tiles_per_wg: 0 for the least that makes a workgroup, else that many (1..4)
+bool qs_plan(int M, int K, int rank, bool has_r, int tiles_per_wg, QsPlan& p) {
   static const int env_waves = qs_env("GLOWQ_QSTREAM_WAVES", 0);
   if (M < 2 || M > 8) return false;
   const int U = K >> 5;
@@ -394,6 +395,8 @@ bool qs_plan(int M, int K, int rank, bool has_r, QsPlan& p) {
   // each thread stages at most two 16-byte words of a token row (one with eight token rows, or the registers run out)
   const int max_words = p.tok == 8 ? 1 : 2;
   while (waves * kWave * max_words < (K >> 3) && waves + p.slices <= 16 && waves / p.slices < 4) waves += p.slices;
+  if (waves > 16 || waves / p.slices > 4) return false;
+  if (tiles_per_wg > waves / p.slices) waves = tiles_per_wg * p.slices;
   if (waves > 16 || waves / p.slices > 4) return false;
   p.waves = waves;
   const int threads = waves * kWave, words = K >> 3;
@@ -462,12 +465,39 @@ bool qstream_supported(const GroupDev& g) {
       return false;
   }
   QsPlan p;
-  return qs_plan(g.M, g.K, g.rank, has_r, p);
+  return qs_plan(g.M, g.K, g.rank, has_r, 0, p);
 }
 
-hipError_t launch_qstream(GroupDev& g, hipStream_t stream) {
+hipError_t launch_qstream(GroupDev& g, int num_cus, hipStream_t stream) {
+  static const int env_waves = qs_env("GLOWQ_QSTREAM_WAVES", 0);
   QsPlan p;
-  if (!qs_plan(g.M, g.K, g.rank, g.r != nullptr, p)) return hipErrorInvalidValue;
+  if (!qs_plan(g.M, g.K, g.rank, g.r != nullptr, 0, p)) return hipErrorInvalidValue;
+  // A launch of few workgroups is over when the compute unit with the most tiles is done: more tiles per workgroup
+  // where all workgroups then fit the compute units one each and the most loaded unit has fewer tiles (5120 rows of
+  // 5120 columns, 640 tiles on 256 units: two tiles per workgroup leave 64 units with four tiles, three leave every
+  // unit with three at most: 9.4 -> 8.3 us at four token rows).
+  if (env_waves == 0) {
+    auto workgroups = [&](int t) {
+      long n = 0;
+      for (int i = 0; i < g.n_members; ++i) n += ((g.mem[i].N + 4 * p.r - 1) / (4 * p.r) + t - 1) / t;
+      return n;
+    };
+    const int t0 = p.waves / p.slices;
+    const long wgs0 = workgroups(t0);
+    if (wgs0 > num_cus && wgs0 <= 2L * num_cus) {
+      long best = 2L * t0;
+      int pick = t0;
+      for (int t = t0 + 1; t <= 4; ++t) {
+        QsPlan q;
+        if (workgroups(t) <= num_cus && t < best && qs_plan(g.M, g.K, g.rank, g.r != nullptr, t, q)) {
+          best = t;
+          pick = t;
+          break;
+        }
+      }
+      if (pick != t0 && !qs_plan(g.M, g.K, g.rank, g.r != nullptr, pick, p)) return hipErrorInvalidValue;
+    }
+  }
   return launch_qs_l(g, p, stream);
 }
 

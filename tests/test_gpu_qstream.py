@@ -40,6 +40,7 @@ CASES = [
     (8, 8192, [100], 64, 128, False, ()),
     (5, 5120, [24, 9], 128, 128, False, ()),
     (6, 1024, [1, 2, 3, 5], 24, 128, False, ()),
+    (3, 4096, [5000], 64, 128, True, ()),   # between one and two workgroups per compute unit: three tiles per workgroup
 ]
 
 

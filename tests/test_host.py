@@ -305,11 +305,12 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     # last 2048-column slice of a row is mostly empty, not for long rows with many of them
     assert ext.route(2, 4096, 28672) == "quad_stream_gemv" and ext.route(4, 4096, 4096) == "quad_stream_gemv"
     assert ext.route(3, 14336, 4096) == "quad_stream_gemv" and ext.route(4, 8192, 10240) == "quad_stream_gemv"
-    assert ext.route(4, 5120, 5120) != "quad_stream_gemv" and ext.route(4, 6144, 28672) != "quad_stream_gemv"
+    assert ext.route(2, 5120, 5120) != "quad_stream_gemv" and ext.route(4, 6144, 28672) != "quad_stream_gemv"
+    assert ext.route(4, 5120, 5120) == "quad_stream_gemv"
     assert ext.route(1, 4096, 4096) != "quad_stream_gemv" and ext.route(5, 4096, 4096) != "quad_stream_gemv"
     assert ext.route(4, 4096, 4096, group_size=64) != "quad_stream_gemv" and ext.route(4, 17408, 5120) != "quad_stream_gemv"
     rule = ext.set_tuning("qstream_shape_rule", 0)
-    assert ext.route(4, 5120, 5120) == "quad_stream_gemv" and ext.route(4, 6144, 28672) == "quad_stream_gemv"
+    assert ext.route(2, 5120, 5120) == "quad_stream_gemv" and ext.route(4, 6144, 28672) == "quad_stream_gemv"
     ext.set_tuning("qstream_shape_rule", rule)
     assert ext.set_tuning("qstream_max_m", 8) == 4
     assert ext.route(8, 4096, 4096) == "quad_stream_gemv" and ext.route(8, 14336, 4096) != "quad_stream_gemv"
