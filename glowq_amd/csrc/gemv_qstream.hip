@@ -73,8 +73,8 @@ __device__ __forceinline__ float row_class_sum(float v) {
   return v;
 }
 
-// kLD: dwords of a row of L per lane (0, 4 or 8: sixteen lanes cover rank <= 32 kLD); kTok: token rows staged (2, 4 or
-// 8); kXW: 16-byte words of each token row per thread.  `slices` = ceil(K / (512 kC)) consecutive waves of a workgroup
+// kR: row blocks of a wave's tile (2 or 4; kC = 8 / kR columns of 16 units); kLD: dwords of a row of L per lane (0, 4
+// or 8: sixteen lanes cover rank <= 32 kLD); kTok: token rows staged (2, 4 or 8); kXW: 16-byte words of each token row per thread.  `slices` = ceil(K / (512 kC)) consecutive waves of a workgroup
 // share the rows of a tile, slice s taking units 16 kC s ... 16 kC (s + 1) - 1 (units past the row read its last unit
 // again and are weighted by zero).
 template <int kR, int kLD, int kTok, int kXW>
