@@ -223,29 +223,28 @@ bool stream_pays(const GroupDev& g) {
   return short_k && rows <= 4096;
 }
 
-//   qstream_max_m   token rows (2..8) up to which the stream-scheduled 4x4x4 matrix-core GEMV is used where it applies;
-//                   0 switches it off (GLOWQ_QSTREAM_M).  From five rows on it runs level with the skinny MFMA kernel.
+//   qstream_max_m   token rows (2..4) up to which the stream-scheduled 4x4x4 matrix-core GEMV is used where it applies;
+//                   0 switches it off (GLOWQ_QSTREAM_M).  (A form for five to eight rows, two sets of sums per row
+//                   block, ran level with the skinny MFMA kernel and was taken out.)
 //   qstream_shape_rule  1: only for the shapes it was measured faster on; 0: for every shape it can take
 //                   (GLOWQ_QSTREAM_SHAPE_RULE)
-std::atomic<int> g_qstream_max_m{clampi(env_or("GLOWQ_QSTREAM_M", 4), 0, 8)};
+std::atomic<int> g_qstream_max_m{clampi(env_or("GLOWQ_QSTREAM_M", 4), 0, 4)};
 std::atomic<int> g_qstream_shape_rule{clampi(env_or("GLOWQ_QSTREAM_SHAPE_RULE", 1), 0, 1)};
 
 // Group launch alone, us, this kernel / the route taken without it (6 to 32 layers of distinct weights back to back):
-//   four rows   4096 x 4096: 4.7 / 6.9   6144 x 4096 (q|k|v): 6.7 / 7.8   28672 x 4096: 16.2 / 18.7   4096 x 14336: 11.7 / 14.5
-//               4096 x 11008: 9.4 / 13.4   8192 x 8192: 10.9 / 14.2   10240 x 8192: 14.2 / 19.6   37888 x 3584: 19.9 / 23.4
-//               7168 x 5120: 9.6 / 12.2   5120 x 5120: 8.2 / 9.3   34816 x 5120: 34.4 / 31.7   28672 x 6144: 31.2 / 25.0
-//   two rows    4096 x 4096: 4.6 / 5.1   6144 x 4096: 6.2 / 6.2   28672 x 4096: 14.3 / 15.9   4096 x 14336: 10.5 / 10.7
-//               5120 x 5120: 7.5 / 7.3   34816 x 5120: 27.0 / 26.7   10240 x 8192: 13.1 / 12.7
-// Every workgroup stages the whole activation rows for its 16 output rows: long rows with many workgroups per compute
-// unit pay for that (the persistent 4x4x4 kernel stages once per compute unit); at two rows a last slice that is mostly
-// empty (K = 5120: 2.5 slices of 2048 columns) is enough to fall behind the stream GEMV.
+//   four rows   4096 x 4096: 4.7 / 6.9   6144 x 4096 (q|k|v): 6.7 / 7.6   28672 x 4096: 15.8 / 19.2   4096 x 14336: 11.7 / 14.5
+//               4096 x 11008: 9.4 / 13.4   8192 x 8192: 10.9 / 14.2   10240 x 8192: 13.5 / 19.7   37888 x 3584: 18.9 / 23.6
+//               7168 x 5120: 9.6 / 12.2   5120 x 5120: 8.2 / 9.3   34816 x 5120: 27.7 / 31.7   28672 x 6144: 24.0 / 25.6
+//   two rows    4096 x 4096: 4.6 / 5.1   6144 x 4096: 6.2 / 6.1   28672 x 4096: 14.1 / 16.2   4096 x 14336: 10.5 / 10.7
+//               5120 x 5120: 7.5 / 7.3   7168 x 5120: 8.5 / 8.4   34816 x 5120: 25.9 / 27.2   10240 x 8192: 12.9 / 13.2
+// At two rows a last slice that is mostly empty (K = 5120: 2.5 slices of 2048 columns) is enough to fall behind the
+// stream GEMV on groups of few rows.
 bool qstream_pays(const GroupDev& g) {
   if (g_qstream_shape_rule.load(std::memory_order_relaxed) == 0) return true;
   long rows = 0;
   for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
   const int padded = (g.K + 2047) / 2048 * 2048;
-  if (g.M == 2 && (padded - g.K) * 100 > 15 * g.K) return false;  // (level with the stream GEMV or behind it there)
-  if (g.K > 4096 && rows >= 16384) return false;
+  if (g.M == 2 && rows < 16384 && (padded - g.K) * 100 > 15 * g.K) return false;
   return true;
 }
 
@@ -655,7 +654,7 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "skinny_max_m") == 0) { slot = &g_skinny_max_m; hi = 64; }
   else if (strcmp(key, "small_group_mb") == 0) { slot = &g_small_group_mb; hi = 4096; }
   else if (strcmp(key, "stream_max_m") == 0) { slot = &g_stream_max_m; hi = 4; }
-  else if (strcmp(key, "qstream_max_m") == 0) { slot = &g_qstream_max_m; hi = 8; }
+  else if (strcmp(key, "qstream_max_m") == 0) { slot = &g_qstream_max_m; hi = 4; }
   else if (strcmp(key, "qstream_shape_rule") == 0) { slot = &g_qstream_shape_rule; hi = 1; }
   else if (strcmp(key, "stream_shape_rule") == 0) { slot = &g_stream_shape_rule; hi = 1; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);

@@ -1,4 +1,4 @@
-// Decode GEMV for 2..8 token rows: the arithmetic of the 4x4x4 matrix-core GEMV (gemv_quad.hip) under the memory
+// Decode GEMV for 2..4 token rows: the arithmetic of the 4x4x4 matrix-core GEMV (gemv_quad.hip) under the memory
 // schedule of the stream GEMV (stream_kernel.hpp).
 //
 // v_mfma_f32_4x4x4_16B_f16 multiplies sixteen independent 4x4x4 blocks: lanes 4b..4b+3 form block b, lane 4b + q
@@ -21,9 +21,11 @@
 //     a load covers 256 contiguous bytes of each of four rows -- so no lane exchange lies between load and use
 //     (with loads in memory order and a ds_bpermute per dword the LDS pipe was busy 80 % of the launch);
 //   * the activations of the upper nibbles are staged divided by 16, so one accumulator chain takes both nibbles;
-//   * the waves that share the rows of a tile (the slices of their K extent) meet in LDS once, at the end;
-//   * a workgroup is one or two tiles: small workgroups come and go independently, which is worth more than the
-//     activation rows they stage redundantly.
+//   * the waves that share the rows of a tile (the slices of their K extent) meet in LDS once per tile, at its end;
+//   * a workgroup is one or two tiles wide: small workgroups come and go independently, which is worth more than the
+//     activation rows they stage redundantly;
+//   * a launch of more workgroups than the compute units hold at once runs as many as they hold, each walking a list
+//     of tiles: the activations are staged once, and a wave's next requests go out as soon as its last tile is stored.
 #include <cstdlib>
 
 #include "stream_kernel.hpp"
@@ -45,7 +47,8 @@ constexpr int kQsPad = 4;          // 16-byte words between the token rows of xs
 //      x[32u + 8t + {0,4,2,6, 1,5,3,7}] (the order the two masked operands of a code word come out in)
 // sig  [U][tok4] floats: 2^-24 * sum of the 32 activations of unit u, per token
 // rs   [tok4][rank + 8] halves
-// part [waves][kR][sets][4 rows of lanes][4 rows][4 tokens] floats: what the waves leave for the final sum
+// part [2][waves][kR][sets][4 rows of lanes][4 rows][4 tokens] floats: what the waves leave for the final sum (two
+//      buffers, used in turn by the tiles a workgroup walks)
 struct QsLds {
   int tok4, x_stride, r_stride;
   size_t sig_off, r_off, part_off, total;
@@ -59,7 +62,7 @@ __host__ __device__ inline QsLds qs_lds(int tokens, int K, int rank, int waves, 
   l.sig_off = (size_t)tokens * l.x_stride * 16;
   l.r_off = l.sig_off + (size_t)U * l.tok4 * sizeof(float);
   l.part_off = l.r_off + (rank > 0 ? (size_t)l.tok4 * l.r_stride * sizeof(half_t) : 0);
-  l.total = l.part_off + (size_t)waves * r * (l.tok4 / 4) * 64 * sizeof(float);
+  l.total = l.part_off + (size_t)2 * waves * r * (l.tok4 / 4) * 64 * sizeof(float);
   return l;
 }
 
@@ -79,7 +82,7 @@ __device__ __forceinline__ float row_class_sum(float v) {
 // again and are weighted by zero).
 template <int kR, int kLD, int kTok, int kXW>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(2, 4)))
-void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per_wg) {
+void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per_wg, const int total_wgs) {
   constexpr int kC = qs_c(kR), kRows = 4 * kR;
   constexpr int kSets = (kTok + 3) / 4;
   constexpr int kTok4 = 4 * kSets;
@@ -120,30 +123,45 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
       rw[m] = ld_b32(g.r + (size_t)min(m, g.M - 1) * rank, (uint32_t)min((int)threadIdx.x, rd - 1) * 4u);
   }
 
-  // ---- member and tile of this wave
+  // ---- the wave's place in its workgroup (tiles_per_wg is 1..4: three comparisons instead of a division)
+  const int local_tile = (wave >= slices) + (wave >= 2 * slices) + (wave >= 3 * slices);
+  const int slice = wave - local_tile * slices;
+  const int unit0 = slice * (16 * kC);  // first unit of the slice
+  const int grp0 = unit0 >> upg_shift;  // and its group
+  const int l_chunks = kLD > 0 ? rank / (2 * kLD) : 1;  // lanes of a row that hold a part of L
+
+  // ---- what a wave holds of a tile: set by issue(), used by finish()
   MemberDev mem = g.mem[0];
+  bool valid = false, l_here = false;
+  int row0 = 0;
+  uint32_t sc[kSideLoads], zw[kSideLoads], sgrp[kSideLoads];
+  u32x4 lq[kLQ > 0 ? kR : 1][kLQ > 0 ? kLQ : 1];
+  u32x4 w[kC][kR];
+
+  // The launch is a list of total_wgs workgroups' worth of tiles (per member: its tiles in sets of tiles_per_wg); the
+  // workgroups that run take them round robin, vwg = blockIdx.x, blockIdx.x + gridDim.x, ...  A launch with more of
+  // them than the compute units hold at once runs that many workgroups and lets each walk its list: the activations
+  // are staged once, and a wave requests its next tile the moment it has stored the last one.
+  auto issue = [&](const int vwg) {
+  // ---- member and tile of this wave
+  mem = g.mem[0];
   int wg_begin = 0, total_tiles = g.task_end[0];
-#define GLOWQ_PICK(i)                                            \
-  if (g.n_members > i && (int)blockIdx.x >= g.wg_end[i - 1]) {  \
-    mem = g.mem[i];                                              \
-    wg_begin = g.wg_end[i - 1];                                  \
-    total_tiles = g.task_end[i] - g.task_end[i - 1];             \
+#define GLOWQ_PICK(i)                                  \
+  if (g.n_members > i && vwg >= g.wg_end[i - 1]) {    \
+    mem = g.mem[i];                                    \
+    wg_begin = g.wg_end[i - 1];                        \
+    total_tiles = g.task_end[i] - g.task_end[i - 1];   \
   }
   GLOWQ_PICK(1)
   GLOWQ_PICK(2)
   GLOWQ_PICK(3)
 #undef GLOWQ_PICK
-  // (tiles_per_wg is 1..4: three comparisons instead of a division)
-  const int local_tile = (wave >= slices) + (wave >= 2 * slices) + (wave >= 3 * slices);
-  const int slice = wave - local_tile * slices;
-  const int want = ((int)blockIdx.x - wg_begin) * tiles_per_wg + local_tile;
+  const int want = (vwg - wg_begin) * tiles_per_wg + local_tile;
   // waves past the member's last tile (and the waves a workgroup has beyond whole sets of slices) still issue their
   // loads (the wait counts stay what they are), all lanes on one address
-  const bool valid = want < total_tiles && local_tile < tiles_per_wg;
-  const int row0 = (valid ? want : 0) * kRows;
+  valid = want < total_tiles && local_tile < tiles_per_wg;
+  row0 = (valid ? want : 0) * kRows;
   const uint32_t live = valid ? 0xFFFFFFFFu : 0u;
-  const int unit0 = slice * (16 * kC);  // first unit of the slice
-  const int grp0 = unit0 >> upg_shift;  // and its group
   // Every member's buffers stay below 2 GiB (checked on the host): uniform base + 32-bit byte offset, row index and
   // row pitch below 2^24 each.  (24-bit multiplies: the 32-bit multiply-add this compiler would otherwise pick takes a
   // register pair as its addend, with whatever register lies next to the addend as the unused upper half -- possibly
@@ -153,9 +171,6 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
   // ---- every load of the tile
   // scale and zero-point word of one (row, group) pair per lane and load: pair p = 64 j + lane is group p % kGmax of the
   // slice, row p / kGmax of the tile
-  uint32_t sc[kSideLoads], zw[kSideLoads], sgrp[kSideLoads];
-  u32x4 lq[kLQ > 0 ? kR : 1][kLQ > 0 ? kLQ : 1];
-  u32x4 w[kC][kR];
 #pragma unroll
   for (int j = 0; j < kSideLoads; ++j) {
     const int p = 64 * j + lane;
@@ -167,9 +182,8 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
   uint32_t n_q[kR];  // the lane's row of each row block
 #pragma unroll
   for (int rb = 0; rb < kR; ++rb) n_q[rb] = (uint32_t)min(row0 + 4 * rb + qj, mem.N - 1);
-  const int l_chunks = kLD > 0 ? rank / (2 * kLD) : 1;            // lanes of a row that hold a part of L
   // the last slice, the one with the fewest columns left, adds the correction
-  const bool l_here = kLD > 0 && mem.L != nullptr && slice == slices - 1;
+  l_here = kLD > 0 && mem.L != nullptr && slice == slices - 1;
   if constexpr (kLD > 0) {
     // elsewhere: valid memory, weighted by zero
     const char* lb = l_here ? reinterpret_cast<const char*>(mem.L) : reinterpret_cast<const char*>(g.x);
@@ -186,6 +200,8 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
 #pragma unroll
     for (int rb = 0; rb < kR; ++rb) w[c][rb] = ld_b128_nt(mem.qweight, (__umul24(n_q[rb], ldw_bytes) + u * 16u) & live);
   }
+  };  // issue()
+  issue((int)blockIdx.x);
 
   // ---- stage the activations (every load of x and r lies ahead of the tile's: one count covers them all)
 #pragma unroll
@@ -224,7 +240,9 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
   }
   __syncthreads();
 
-  // ---- consume the tile in the order it was requested
+  // ---- consume the tile in the order it was requested, then reduce and store it.  `parity` picks one of the two
+  // buffers the waves leave their sums in: the sums of one tile are read while those of the next may be written.
+  auto finish = [&](const int parity) {
   f4 tot[kR][kSets];
 #pragma unroll
   for (int rb = 0; rb < kR; ++rb)
@@ -327,7 +345,7 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
   // ---- the 16 lanes of a row: four blocks per row of 16 lanes meet through lane rotations, the four rows of lanes and
   // the slices of the tile through LDS
   {
-    float* mine = part + (size_t)wave * (kR * kSets * 64);
+    float* mine = part + (size_t)(parity * waves + wave) * (kR * kSets * 64);
 #pragma unroll
     for (int rb = 0; rb < kR; ++rb) {
 #pragma unroll
@@ -348,7 +366,7 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
     const float bias = (writer && mem.bias) ? (float)mem.bias[n] : 0.f;
 #pragma unroll
     for (int s = 0; s < kSets; ++s) {
-      const float* src = part + (size_t)wave * (kR * kSets * 64) + ((((rowi >> 2) * kSets + s) * 4) * 4 + (rowi & 3)) * 4 + i;
+      const float* src = part + (size_t)(parity * waves + wave) * (kR * kSets * 64) + ((((rowi >> 2) * kSets + s) * 4) * 4 + (rowi & 3)) * 4 + i;
       float v = 0.f;
       for (int o = 0; o < slices; ++o)
 #pragma unroll
@@ -356,6 +374,15 @@ void gemv_qstream_kernel(const GroupDev g, const int slices, const int tiles_per
       const int m = 4 * s + i;
       if (writer && m < g.M) mem.y[(size_t)m * mem.ldy + n] = (half_t)(__builtin_fmaf(v, 0x1p24f, bias));
     }
+  }
+  };  // finish()
+  finish(0);
+  // the rest of this workgroup's list (the same for all its waves: the barriers inside stay matched)
+  int parity = 1;
+  for (int vwg = (int)blockIdx.x + (int)gridDim.x; vwg < total_wgs; vwg += (int)gridDim.x) {
+    issue(vwg);
+    finish(parity);
+    parity ^= 1;
   }
 }
 
@@ -367,16 +394,16 @@ int qs_env(const char* name, int fallback) {
 // How a shape is launched: slices per tile, waves per workgroup, words of a token row per
 // thread, token rows staged.
 struct QsPlan {
-  int r, slices, waves, xw, tok;
+  int r, slices, waves, xw, tok, num_cus;
   size_t lds;
 };
 
 // tiles_per_wg: 0 for the least that makes a workgroup, else that many (1..4)
 bool qs_plan(int M, int K, int rank, bool has_r, int tiles_per_wg, QsPlan& p) {
   static const int env_waves = qs_env("GLOWQ_QSTREAM_WAVES", 0);
-  if (M < 2 || M > 8) return false;
+  if (M < 2 || M > 4) return false;
   const int U = K >> 5;
-  p.tok = M <= 2 ? 2 : (M <= 4 ? 4 : 8);
+  p.tok = M <= 2 ? 2 : 4;
   // Tile: 8 rows by 2048 columns (8B-shape layer at four token rows, 8 x 2048 / 16 x 1024: q|k|v 6.6 / 6.9 us, o_proj
   // 4.7 / 5.0, gate|up 15.9 / 16.8, down_proj 11.5 / 12.3; K = 5120, 2.5 slices of 2048 columns against 5 of 1024:
   // 34.6 / 35.2 on 34816 rows).
@@ -422,7 +449,25 @@ hipError_t launch_qs_t(GroupDev& g, const QsPlan& p, hipStream_t stream) {
     grid += (tiles + tiles_per_wg - 1) / tiles_per_wg;
     g.wg_end[i] = grid;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(p.waves * kWave), p.lds, stream, g, p.slices, tiles_per_wg);
+  // More workgroups than the compute units hold at once: launch as many as they hold and let each walk its share of
+  // the list (GLOWQ_QSTREAM_PERSIST=0: one workgroup per entry of the list)
+  static const int env_persist = qs_env("GLOWQ_QSTREAM_PERSIST", 1);
+  int launch = grid;
+  if (env_persist && p.num_cus > 0) {
+    static std::atomic<long> seen_key{-1};
+    static std::atomic<int> seen_val{0};
+    const long key = ((long)p.waves << 32) | (long)p.lds;
+    int per_cu = seen_val.load(std::memory_order_acquire);
+    if (seen_key.load(std::memory_order_acquire) != key || per_cu <= 0) {
+      per_cu = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), p.waves * kWave, p.lds) != hipSuccess || per_cu <= 0)
+        per_cu = 0;
+      seen_val.store(per_cu, std::memory_order_release);
+      seen_key.store(key, std::memory_order_release);
+    }
+    if (per_cu > 0 && grid > p.num_cus * per_cu) launch = p.num_cus * per_cu;
+  }
+  hipLaunchKernelGGL(kern, dim3(launch), dim3(p.waves * kWave), p.lds, stream, g, p.slices, tiles_per_wg, grid);
   return hipGetLastError();
 }
 
@@ -431,7 +476,7 @@ hipError_t launch_qs_x(GroupDev& g, const QsPlan& p, hipStream_t stream) {
 #define GLOWQ_CASE(RR, TT, XX) \
   if (p.r == RR && p.tok == TT && p.xw == XX) return launch_qs_t<RR, kLD, TT, XX>(g, p, stream);
   GLOWQ_CASE(4, 2, 1) GLOWQ_CASE(4, 2, 2) GLOWQ_CASE(4, 4, 1) GLOWQ_CASE(4, 4, 2)
-  GLOWQ_CASE(2, 2, 1) GLOWQ_CASE(2, 2, 2) GLOWQ_CASE(2, 4, 1) GLOWQ_CASE(2, 4, 2) GLOWQ_CASE(2, 8, 1)
+  GLOWQ_CASE(2, 2, 1) GLOWQ_CASE(2, 2, 2) GLOWQ_CASE(2, 4, 1) GLOWQ_CASE(2, 4, 2)
 #undef GLOWQ_CASE
   return hipErrorInvalidValue;
 }
@@ -445,10 +490,10 @@ bool aligned_to(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t
 
 }  // namespace
 
-// 2..8 token rows from the canonical buffers, groups of 128 to 2048 columns (a power of two of 32-column units: the
+// 2..4 token rows from the canonical buffers, groups of 128 to 2048 columns (a power of two of 32-column units: the
 // caller's layout check), rank a multiple of 8 up to 128 or of 16 up to 256, buffers addressable with 32-bit offsets.
 bool qstream_supported(const GroupDev& g) {
-  if (g.M < 2 || g.M > 8 || g.group_size < 128 || g.group_size > 2048 || (g.K & 31) != 0 || !aligned_to(g.x, 16)) return false;
+  if (g.M < 2 || g.M > 4 || g.group_size < 128 || g.group_size > 2048 || (g.K & 31) != 0 || !aligned_to(g.x, 16)) return false;
   const bool has_r = g.r != nullptr || g.R != nullptr;
   if (has_r) {
     if (g.rank < 8 || g.rank > 256 || (g.rank & 7) != 0 || (g.rank > 128 && (g.rank & 15) != 0)) return false;
@@ -498,6 +543,7 @@ hipError_t launch_qstream(GroupDev& g, int num_cus, hipStream_t stream) {
       if (pick != t0 && !qs_plan(g.M, g.K, g.rank, g.r != nullptr, pick, p)) return hipErrorInvalidValue;
     }
   }
+  p.num_cus = num_cus;
   return launch_qs_l(g, p, stream);
 }
 

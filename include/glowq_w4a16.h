@@ -207,7 +207,7 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * "stream_max_m" (0..4): token rows up to which the stream GEMV is used where its layout applies, ahead of the
  * others; 0 switches it off.  "stream_shape_rule" (0 / 1): with more than one token row, only for the shapes it was
  * measured faster on (1, the default) or for every shape (0).
- * "qstream_max_m" (0..8, default 4): token rows, from two, up to which the stream-scheduled 4x4x4 matrix-core GEMV
+ * "qstream_max_m" (0..4, default 4): token rows, from two, up to which the stream-scheduled 4x4x4 matrix-core GEMV
  * is used where it applies (groups of 128 to 2048 columns, rank a multiple of 8 up to 128 or of 16 up to 256, rows
  * up to 16384 columns), ahead of all others; 0 switches it off.  "qstream_shape_rule" (0 / 1): only for the shapes it
  * was measured faster on (1, the default) or for every shape it can take (0).

@@ -30,10 +30,10 @@ def golden():
 @pytest.fixture(params=["stream", "qstream", "quad", "classic"])
 def small_m_route(request, ext):
     """Runs a test with the stream GEMV serving 1..4 token rows (the other kernels above), with the stream-scheduled 4x4x4
-    matrix-core GEMV serving 2..8 token rows, with the 4x4x4 matrix-core GEMV serving 1..16 token rows, and with all
+    matrix-core GEMV serving 2..4 token rows, with the 4x4x4 matrix-core GEMV serving 1..16 token rows, and with all
     switched off (wave-dot GEMV for 1..4 rows, skinny MFMA kernel above)."""
     if request.param == "qstream":
-        old = ext.set_tuning("qstream_max_m", 8), ext.set_tuning("qstream_shape_rule", 0)
+        old = ext.set_tuning("qstream_max_m", 4), ext.set_tuning("qstream_shape_rule", 0)
         yield request.param
         ext.set_tuning("qstream_max_m", old[0]), ext.set_tuning("qstream_shape_rule", old[1])
         return

@@ -30,7 +30,7 @@ CASES = [
     (2, 4096, [4096], 128, "default"), (2, 14336, [8192], 128, "default"),
     (3, 2048, [300], 64, "default"), (4, 4096, [2048, 2048], 64, "default"),
     (4, 4096, [2048, 2048], 64, "quad"), (4, 4096, [2048, 2048], 64, "classic"),
-    (8, 4096, [512], 128, "default"), (8, 4096, [512], 128, "quad"), (8, 4096, [512], 128, "qstream"),
+    (8, 4096, [512], 128, "default"), (8, 4096, [512], 128, "quad"), (4, 4096, [512], 128, "qstream"),
     (4, 14336, [8192], 128, "qstream"), (3, 4096, [2048, 2048], 256, "qstream"),
     (16, 14336, [256], 128, "default"), (16, 4096, [1024, 256], 128, "quad"),
     (64, 4096, [512, 96], 256, "default"), (130, 2048, [512], 128, "default"), (300, 4096, [256, 128], 128, "default"),
@@ -50,7 +50,7 @@ def tuned(ext):
             saved["qstream_max_m"] = ext.set_tuning("qstream_max_m", 0)
             return
         if mode == "qstream":
-            saved["qstream_max_m"] = ext.set_tuning("qstream_max_m", 8)
+            saved["qstream_max_m"] = ext.set_tuning("qstream_max_m", 4)
             saved["qstream_shape_rule"] = ext.set_tuning("qstream_shape_rule", 0)
             return
         for key, value in (("quad_max_m", 16 if mode == "quad" else 0), ("quad_min_m", 1), ("small_group_mb", 0),

@@ -1,4 +1,4 @@
-"""The stream-scheduled 4x4x4 matrix-core GEMV (2..8 token rows) through the C ABI against the float64 oracle: row
+"""The stream-scheduled 4x4x4 matrix-core GEMV (2..4 token rows) through the C ABI against the float64 oracle: row
 lengths of one step and less, of two, of an odd number of steps (the last slice half empty), long rows cut into
 slices, ranks on either side of the 16-byte chunking of L, group sizes up to one group per step, members whose row
 count is no multiple of four, members without L, bias, token counts between the staged ones."""
@@ -16,7 +16,7 @@ ROUTE = 6  # quad_stream_gemv
 
 @pytest.fixture()
 def qstream(ext):
-    old = ext.set_tuning("qstream_max_m", 8), ext.set_tuning("qstream_shape_rule", 0)
+    old = ext.set_tuning("qstream_max_m", 4), ext.set_tuning("qstream_shape_rule", 0)
     yield ext
     ext.set_tuning("qstream_max_m", old[0]), ext.set_tuning("qstream_shape_rule", old[1])
 
@@ -30,17 +30,19 @@ CASES = [
     (4, 5120, [257], 256, 128, True, ()),
     (4, 14336, [96, 33], 128, 128, False, ()),
     (2, 14336, [64], 0, 128, False, ()),
-    (5, 4096, [200], 8, 256, False, ()),
-    (7, 3584, [64, 64, 19], 128, 128, True, (0,)),
-    (8, 4096, [512], 128, 128, False, ()),
-    (8, 4096, [66], 0, 2048, False, ()),
-    (8, 2048, [40], 256, 512, False, ()),
+    (3, 4096, [200], 8, 256, False, ()),
+    (4, 3584, [64, 64, 19], 128, 128, True, (0,)),
+    (4, 4096, [512], 128, 128, False, ()),
+    (3, 4096, [66], 0, 2048, False, ()),
+    (2, 2048, [40], 256, 512, False, ()),
     (4, 16384, [48], 128, 128, False, ()),
     (3, 12288, [36, 4], 256, 128, True, ()),
-    (8, 8192, [100], 64, 128, False, ()),
-    (5, 5120, [24, 9], 128, 128, False, ()),
-    (6, 1024, [1, 2, 3, 5], 24, 128, False, ()),
+    (4, 8192, [100], 64, 128, False, ()),
+    (3, 5120, [24, 9], 128, 128, False, ()),
+    (4, 1024, [1, 2, 3, 5], 24, 128, False, ()),
     (3, 4096, [5000], 64, 128, True, ()),   # between one and two workgroups per compute unit: three tiles per workgroup
+    (4, 4096, [20000], 128, 128, False, ()),  # more workgroups than the compute units hold: each walks a list of tiles
+    (2, 2048, [9000, 9000, 2000], 0, 128, True, ()),
 ]
 
 

@@ -47,13 +47,13 @@ def random_cases(n, seed=20240):
 @pytest.fixture(params=["default", "stream", "qstream", "quad", "classic"])
 def route_mode(request, ext):
     """The library's own route limits, the stream GEMV for every case of 1..4 rows it can take, the stream-scheduled
-    4x4x4 matrix-core GEMV for every case of 2..8 rows it can take, the 4x4x4 matrix-core GEMV for every case of 1..16
+    4x4x4 matrix-core GEMV for every case of 2..4 rows it can take, the 4x4x4 matrix-core GEMV for every case of 1..16
     rows it can take, or all switched off (wave-dot GEMV up to 4 rows, skinny MFMA kernel above)."""
     if request.param == "default":
         yield request.param
         return
     if request.param == "qstream":
-        old = ext.set_tuning("qstream_max_m", 8), ext.set_tuning("qstream_shape_rule", 0)
+        old = ext.set_tuning("qstream_max_m", 4), ext.set_tuning("qstream_shape_rule", 0)
         yield request.param
         ext.set_tuning("qstream_max_m", old[0]), ext.set_tuning("qstream_shape_rule", old[1])
         return
