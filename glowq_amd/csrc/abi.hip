@@ -35,7 +35,8 @@ hipError_t launch_pack_side(const half_t*, const int32_t*, const half_t*, void*,
 // skinny.hip / gemm.hip
 bool skinny_supported(const GroupDev& g);
 bool skinny_group_form(const GroupDev& g);
-hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream);
+bool skinny_raw_form(const GroupDev& g);
+hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw);
 bool gemm_supported(const GroupDev& g);
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream);
 hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t, void* ws,
@@ -107,7 +108,7 @@ int num_cus() {
 
 namespace {
 
-constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4, kRouteStream = 5, kRouteQStream = 6;
+constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4, kRouteStream = 5, kRouteQStream = 6, kRouteSkinnyRaw = 7;
 constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
 
 // Route limits, settable at run time (glowq_set_tuning) and initialised from the environment:
@@ -248,7 +249,25 @@ bool qstream_pays(const GroupDev& g) {
   return true;
 }
 
+//   skinny_codes_max_m  token rows up to which the skinny MFMA kernel takes the codes as they are (unrounded
+//                   arithmetic, reported as a route of its own) where its second form applies to groups of 128 columns;
+//                   above, and with 0 everywhere, it dequantises to fp16 first (GLOWQ_SKINNY_CODES_M).
+// Group launch alone, 8B shapes, us, codes as they are / dequantised first: 8 rows q|k|v 7.9 / 7.8, o_proj 7.5 / 7.5,
+// gate|up 20.0 / 22.3, down_proj 14.3 / 15.4; 16 rows 9.2 / 8.7, 8.8 / 8.3, 22.7 / 23.5, 17.1 / 17.1; 32 rows 12.2 / 10.5,
+// 11.8 / 10.0, 28.2 / 27.0, 22.9 / 21.0; 64 rows 23.9 / 17.4, 23.5 / 16.9, 53.3 / 51.2, 43.5 / 33.0: applying scale and
+// zero-point to the sums costs two instructions per accumulator register and group, which grows with the rows, while
+// what it saves on the codes does not.
+std::atomic<int> g_skinny_codes_max_m{clampi(env_or("GLOWQ_SKINNY_CODES_M", 8), 0, 64)};
+
+int pick_route_rounded(const GroupDev& g, int force);
+
 int pick_route(const GroupDev& g, int force) {
+  const int route = pick_route_rounded(g, force);
+  if (route == kRouteSkinny && force < 0 && g.M <= g_skinny_codes_max_m.load(std::memory_order_relaxed) && skinny_raw_form(g)) return kRouteSkinnyRaw;
+  return route;
+}
+
+int pick_route_rounded(const GroupDev& g, int force) {
   if (!fast_layout(g)) return kRouteGeneric;
   if (force == kRouteGemm) return gemm_supported(g) ? kRouteGemm : kRouteGeneric;
   if (force < 0 && g.M >= 2 && g.M <= g_qstream_max_m.load(std::memory_order_relaxed) && qstream_supported(g) && qstream_pays(g))
@@ -306,8 +325,8 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     e = launch_qstream(g, cus, stream);
   } else if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
-  } else if (route == kRouteSkinny) {
-    e = launch_skinny(g, cus, stream);
+  } else if (route == kRouteSkinny || route == kRouteSkinnyRaw) {
+    e = launch_skinny(g, cus, stream, route == kRouteSkinnyRaw);
   } else {
     const int cap = (route == kRouteWaveDot) ? kWaveDotMaxM
                     : (route == kRouteQuad) ? quad_capacity(g.M, g.K, g.rank, g.r != nullptr) : 65535;
@@ -656,6 +675,7 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "stream_max_m") == 0) { slot = &g_stream_max_m; hi = 4; }
   else if (strcmp(key, "qstream_max_m") == 0) { slot = &g_qstream_max_m; hi = 4; }
   else if (strcmp(key, "qstream_shape_rule") == 0) { slot = &g_qstream_shape_rule; hi = 1; }
+  else if (strcmp(key, "skinny_codes_max_m") == 0) { slot = &g_skinny_codes_max_m; hi = 64; }
   else if (strcmp(key, "stream_shape_rule") == 0) { slot = &g_stream_shape_rule; hi = 1; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);

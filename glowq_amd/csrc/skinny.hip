@@ -52,6 +52,20 @@ __device__ __forceinline__ h8 nibble_order(const u32x4& v) {
   return __builtin_bit_cast(h8, o);
 }
 
+// total over a row of 16 lanes, in every lane of it
+__device__ __forceinline__ float row16_total(float v) {
+  int t;
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xF, 0xF, true);  // row_ror:1
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xF, 0xF, true);  // row_ror:2
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, true);  // row_ror:4
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, true);  // row_ror:8
+  v += __builtin_bit_cast(float, t);
+  return v;
+}
+
 __device__ __forceinline__ h8 dequant_word_sk(uint32_t w, h2 zb_lo, h2 zb_hi, h2 s2) {
   // the two exponent patterns (1024.0 and 64.0 in both halves) are held in vector registers: with the nibble mask as
   // the one scalar operand each mask-and-merge is a single v_and_or_b32 instead of an AND and an OR
@@ -262,7 +276,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
 // order (8 lanes per segment, every line requested once per instruction) and reads the fragments back in MFMA lane
 // order.  Loading the fragments straight from memory (one 16-byte request per lane and line) cost 22 us of the 45 us
 // of a 28672 x 4096 layer at 32 rows: every request pulls a whole line out of L2.
-template <int kMT, int kNT, bool kBulk>
+// kRaw (groups of 128 columns): the codes go to the matrix cores as they are -- masked in place they are the fp16
+// subnormals code * 2^-24 and code * 2^-20, the activations of the latter staged divided by 16 -- with all sixteen k
+// values of an instruction inside one group: lane (column c, half h) takes the 32-column quarters h and 2 + h of the
+// group instead of one whole group of the super-block.  The eight instructions of a group leave its plain sum of
+// code * x, and scale and zero-point are applied to that sum, y += s (sum c x - z sum x), with the fp32 sums of x per
+// token row and group taken when the activations are staged.  Five vector instructions per code word instead of
+// thirteen, and the arithmetic of the GEMV routes: weights never rounded to fp16.
+template <int kMT, int kNT, bool kBulk, bool kRaw>
 __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63;
@@ -302,8 +323,10 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   constexpr int kSegStride = 144;                      // 128 bytes of a row segment + 16: conflict-free fragment reads
   constexpr int kATile = kMT * 64 * kSegStride;        // bytes per wave
   constexpr int kBTile = kNT * 32 * kSegStride;
-  unsigned char* atile = smem + (size_t)wave * (kATile + kBTile);
+  constexpr int kSig = kRaw ? kMT * 32 * (int)sizeof(float) : 0;  // sums of x over the group being staged, per token row
+  unsigned char* atile = smem + (size_t)wave * (kATile + kBTile + kSig);
   unsigned char* btile = atile + kATile;
+  float* asig = reinterpret_cast<float*>(btile + kBTile);
   const bool corrected = mem.L != nullptr && g.r != nullptr && blockIdx.y == 0;  // the first slice carries the correction
   if (corrected) {
     // A 64-column block of [r | L] reaches the operands like the weights below: its 128-byte row segments are loaded in
@@ -373,7 +396,8 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   const int per = (sb_end - sb_begin + waves - 1) / waves;
   const int first = sb_begin + wave * per;
   const int mine = max(0, min(per, sb_end - first));
-  uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point of the super-block being computed
+  uint32_t cur_s[kNT], cur_z[kNT];  // scale bits and zero-point of the super-block being computed (kRaw: of both its
+                                    // groups: two halves, two nibbles)
 
   // With groups of 128 columns a lane's scales and zero-points of eight consecutive super-blocks are 32 and 8
   // contiguous bytes of its weight row: they are fetched once per eight super-blocks (runs counted from the wave's
@@ -384,7 +408,8 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   // fewer than four super-blocks.
   constexpr bool bulk = kBulk;
   u32x4 run_s[kNT];     // own scale of super-block j of the run: half j % 2 of dword j / 2
-  uint64_t run_z[kNT];  // own zero-point of super-block j: byte j
+  u32x4 run_s2[kRaw ? kNT : 1];  // kRaw: run_s, run_s2 = the sixteen scales as loaded, dword j = both groups of super-block j
+  uint64_t run_z[kNT];  // own zero-point of super-block j: byte j (kRaw: both groups' nibbles)
   int run_start = 0;    // first super-block of the run held
 #pragma unroll
   for (int tn = 0; tn < kNT; ++tn) {
@@ -400,6 +425,13 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       const u32x4 s0 = *reinterpret_cast<const u32x4*>(srow), s1 = *reinterpret_cast<const u32x4*>(srow + 4);
       const int32_t* zrow = mem.qzeros + (size_t)ncol[tn] * mem.ldz;
       const uint32_t z0 = (uint32_t)zrow[zword], z1 = (uint32_t)zrow[min(zword + 1, zlast)], z2 = (uint32_t)zrow[min(zword + 2, zlast)];
+      if constexpr (kRaw) {
+        run_s[tn] = s0;
+        run_s2[tn] = s1;
+        const int sh = 4 * ((2 * start) & 7);  // nibble of group 2 start
+        const uint64_t lo = ((uint64_t)z1 << 32) | z0;
+        run_z[tn] = sh ? (lo >> sh) | ((uint64_t)z2 << (64 - sh)) : lo;  // groups 2 start + 0..15, a nibble each
+      } else {
       const uint32_t sel = lh ? 0x07060302u : 0x05040100u;  // upper or lower half of both dwords
       run_s[tn] = u32x4{__builtin_amdgcn_perm(s0.y, s0.x, sel), __builtin_amdgcn_perm(s0.w, s0.z, sel),
                         __builtin_amdgcn_perm(s1.y, s1.x, sel), __builtin_amdgcn_perm(s1.w, s1.z, sel)};
@@ -407,6 +439,7 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       const uint64_t lo = ((uint64_t)z1 << 32) | z0;
       const uint64_t a = sh ? (lo >> sh) | ((uint64_t)z2 << (64 - sh)) : lo;  // groups 2 start + lh + 0..15, a nibble each
       run_z[tn] = a & 0x0F0F0F0F0F0F0F0Full;
+      }
     }
   };
   auto issue_b = [&](int i, BRegs& rb) {
@@ -420,7 +453,10 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
         rb.b[tn * 4 + q] = *reinterpret_cast<const u32x4*>(mem.qweight + (size_t)n * mem.ldw + sb * 32 + (lane & 7) * 4);
       }
       if (!bulk) {
-        rb.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
+        if constexpr (kRaw)  // both scales of the super-block (scale rows start on a 4-byte boundary: checked on the host)
+          rb.s[tn] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned short*>(mem.scales) + (size_t)ncol[tn] * mem.lds + 2 * sb);
+        else
+          rb.s[tn] = reinterpret_cast<const unsigned short*>(mem.scales)[(size_t)ncol[tn] * mem.lds + grp];
         rb.z[tn] = (uint32_t)mem.qzeros[(size_t)ncol[tn] * mem.ldz + (grp >> 3)];
       } else {
         rb.s[tn] = __builtin_nondeterministic_value(rb.s[tn]);
@@ -441,7 +477,16 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         *reinterpret_cast<u32x4*>(btile + (tn * 32 + q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = rb.b[tn * 4 + q];
-      if (bulk) {
+      if constexpr (kRaw) {
+        if (bulk) {
+          const u32x4 rs = (j & 4) ? run_s2[tn] : run_s[tn];
+          cur_s[tn] = (j & 2) ? ((j & 1) ? rs.w : rs.z) : ((j & 1) ? rs.y : rs.x);
+          cur_z[tn] = (uint32_t)(run_z[tn] >> (8 * j)) & 0xFFu;
+        } else {
+          cur_s[tn] = rb.s[tn];
+          cur_z[tn] = (rb.z[tn] >> (4 * ((2 * (first + i)) & 7))) & 0xFFu;
+        }
+      } else if (bulk) {
         const u32x4 rs = run_s[tn];
         const uint32_t sp = (j & 4) ? ((j & 2) ? rs.w : rs.z) : ((j & 2) ? rs.y : rs.x);
         cur_s[tn] = (j & 1) ? sp >> 16 : sp & 0xFFFFu;
@@ -452,15 +497,18 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       }
     }
   };
-  auto issue_a = [&](int i, int jj, ARegs& ra) {  // jj: first or second half of every lane's 128 columns
-    const int kbase = min(first + i, sblocks - 1) * 256 + jj * 64 + (lane & 7) * 8;
+  // jj: first or second half of every lane's 128 columns: the 64-column halves jj of both groups -- kRaw: both halves of
+  // group jj
+  auto issue_a = [&](int i, int jj, ARegs& ra) {
+    const int kbase = min(first + i, sblocks - 1) * 256 + jj * (kRaw ? 128 : 64) + (lane & 7) * 8;
+    constexpr int kSegCols = kRaw ? 64 : 128;  // columns between the two segments of a token row
 #pragma unroll
     for (int q = 0; q < kMT * 8; ++q) {
       const int seg = q * 8 + (lane >> 3);             // (token row, half of the super-block)
       const int row = min(seg >> 1, g.M - 1);
       // loads whose four token rows all lie past M are skipped, and so is their staging: those rows of the tile keep
       // whatever the LDS held, and the accumulator rows they feed are never stored
-      if (q * 4 < g.M) ra.a[q] = *reinterpret_cast<const u32x4*>(g.x + (size_t)row * g.K + kbase + (seg & 1) * 128);
+      if (q * 4 < g.M) ra.a[q] = *reinterpret_cast<const u32x4*>(g.x + (size_t)row * g.K + kbase + (seg & 1) * kSegCols);
       else ra.a[q] = __builtin_nondeterministic_value(ra.a[q]);  // no value carried round the loop: nothing to wait for
     }
   };
@@ -469,11 +517,82 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int q = 0; q < kMT * 8; ++q)  // staged in the order of the weight nibbles, so that fragment reads need no permute
-      if (q * 4 < g.M)
-        *reinterpret_cast<h8*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = nibble_order(ra.a[q]);
+      if (q * 4 < g.M) {
+        if constexpr (kRaw) {
+          // sixteen lanes hold the 128 columns of the group for token row 4 q + lane / 16: their sum, in fp32
+          const h8 v = __builtin_bit_cast(h8, ra.a[q]);
+          const h2 ones = {(half_t)1.f, (half_t)1.f};
+          float sum = __builtin_amdgcn_fdot2(h2{v[0], v[1]}, ones, 0.f, false);
+          sum = __builtin_amdgcn_fdot2(h2{v[2], v[3]}, ones, sum, false);
+          sum = __builtin_amdgcn_fdot2(h2{v[4], v[5]}, ones, sum, false);
+          sum = __builtin_amdgcn_fdot2(h2{v[6], v[7]}, ones, sum, false);
+          sum = row16_total(sum);
+          if ((lane & 15) == 0) asig[q * 4 + (lane >> 4)] = sum;
+          // the odd nibbles come out of the mask as code * 2^-20: their activations carry the 1/16 (exact but for
+          // values below 2^-10, which lose bits worth 2^-25 and less)
+          u32x4 o = __builtin_bit_cast(u32x4, nibble_order(ra.a[q]));
+          const h2 sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+          o.y = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.y) * sixteenth);
+          o.w = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.w) * sixteenth);
+          *reinterpret_cast<u32x4*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = o;
+        } else {
+          *reinterpret_cast<h8*>(atile + (q * 8 + (lane >> 3)) * kSegStride + (lane & 7) * 16) = nibble_order(ra.a[q]);
+        }
+      }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  // kRaw: group gi of the super-block, all of it: quarters lh and 2 + lh of its codes against the staged group
+  auto compute_raw = [&](int gi) {
+    f16v ag[kMT][kNT];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      h8 bf[kNT][4];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        const u32x4 bw = *reinterpret_cast<const u32x4*>(btile + (tn * 32 + ln) * kSegStride + gi * 64 + lh * 32 + jj * 16);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t wd = bw[t], hi = wd >> 8;
+          bf[tn][t] = __builtin_bit_cast(h8, u32x4{wd & 0x000F000Fu, wd & 0x00F000F0u, hi & 0x000F000Fu, hi & 0x00F000F0u});
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int tm = 0; tm < kMT; ++tm) {
+          const h8 af = *reinterpret_cast<const h8*>(atile + (((tm * 32 + ln) * 2 + lh) * kSegStride) + (4 * jj + t) * 16);
+#pragma unroll
+          for (int tn = 0; tn < kNT; ++tn) {
+            if (jj == 0 && t == 0) {
+              const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              ag[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf[tn][t], zero, 0, 0, 0);
+            } else {
+              ag[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf[tn][t], ag[tm][tn], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+    // scale and zero-point of the group on its sum: rows 8 k + 4 lh + e of the tile sit in registers 4 k + e
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) {
+      const float sc = (float)__builtin_bit_cast(half_t, (uint16_t)((cur_s[tn] >> (16 * gi)) & 0xFFFFu));
+      const float sf = sc * 0x1p24f, sz = -sc * (float)((cur_z[tn] >> (4 * gi)) & 0xFu);
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (tm * 32 + 8 * k < g.M) {
+            const f4 sg = *reinterpret_cast<const f4*>(asig + tm * 32 + 8 * k + 4 * lh);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[tm][tn][4 * k + e] = __builtin_fmaf(sf, ag[tm][tn][4 * k + e], __builtin_fmaf(sz, sg[e], acc[tm][tn][4 * k + e]));
+          }
+        }
+      }
+    }
   };
   auto compute = [&](int i, int j) {
     h8 bf[kNT][4];
@@ -513,10 +632,10 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   for (int i = 0; i < mine; ++i) {
     stage_b(B, i); stage_a(A);
     issue_a(i, 1, A); issue_b(i + 1, B); GLOWQ_PIN_LOADS();
-    compute(i, 0); compute(i, 1);
+    if constexpr (kRaw) compute_raw(0); else { compute(i, 0); compute(i, 1); }
     stage_a(A);
     issue_a(i + 1, 0, A); GLOWQ_PIN_LOADS();
-    compute(i, 2); compute(i, 3);
+    if constexpr (kRaw) compute_raw(1); else { compute(i, 2); compute(i, 3); }
   }
 #undef GLOWQ_PIN_LOADS
   __syncthreads();  // the reduction buffer below overlays the staging tiles
@@ -586,6 +705,17 @@ bool skinny_group_form(const GroupDev& g) {
   return (g.K & 255) == 0 && g.group_size >= 128 && env_form != 0;
 }
 
+// The raw-code form of the second form: groups of exactly 128 columns, scale rows that start on a 4-byte boundary.  Its
+// arithmetic is that of the GEMV routes (weights never rounded to fp16), so the route table reports it as a route of its
+// own.
+bool skinny_raw_form(const GroupDev& g) {
+  static const int env_raw = getenv("GLOWQ_SKINNY_RAW") ? atoi(getenv("GLOWQ_SKINNY_RAW")) : 1;
+  if (env_raw == 0 || !skinny_group_form(g) || g.group_size != 128) return false;
+  for (int i = 0; i < g.n_members; ++i)
+    if ((g.mem[i].lds & 1) != 0 || (reinterpret_cast<uintptr_t>(g.mem[i].scales) & 3u) != 0) return false;
+  return true;
+}
+
 bool skinny_supported(const GroupDev& g) {
   if (g.M < 1 || g.M > 64) return false;
   if ((g.K & 63) != 0 || (g.group_size & 31) != 0 || (g.group_size & (g.group_size - 1)) != 0) return false;
@@ -616,8 +746,9 @@ static bool skinny_bulk_runs(const SkinnyArgs& a, int waves) {
 // ws_bytes: room behind a.partials (0: none).  The second form cuts K into slices through it where the column tiles
 // alone leave half of the CUs or more without a workgroup and every wave still keeps three super-blocks and more
 // (4096 outputs of K = 14336: 128 workgroups -> 2 x 128; 8 rows 16.6 -> about 14.5 us, 64 rows 41 -> about 28).
-template <int kMT, int kNT, bool kGroupForm>
+template <int kMT, int kNT, bool kGroupForm, bool kRaw = false>
 static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t ws_bytes, hipStream_t stream) {
+  static_assert(kGroupForm || !kRaw, "the raw-code form is a variant of the second form");
   int total = 0;
   for (int i = 0; i < a.n_members; ++i) {
     total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
@@ -636,9 +767,10 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
   }
   const bool bulk = kGroupForm && skinny_bulk_runs(a, waves);
   auto kern = !kGroupForm ? skinny_mfma_kernel<kMT, kNT>
-              : bulk ? skinny_group_kernel<kMT, kNT, true> : skinny_group_kernel<kMT, kNT, false>;
+              : bulk ? skinny_group_kernel<kMT, kNT, true, kRaw> : skinny_group_kernel<kMT, kNT, false, kRaw>;
   size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
-  if (kGroupForm && lds < (size_t)waves * (kMT * 64 + kNT * 32) * 144) lds = (size_t)waves * (kMT * 64 + kNT * 32) * 144;
+  const size_t staging = (size_t)waves * ((kMT * 64 + kNT * 32) * 144 + (kRaw ? kMT * 32 * sizeof(float) : 0));
+  if (kGroupForm && lds < staging) lds = staging;
   static LdsLimit lds_limit[2];  // one per kernel this site launches
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit[bulk]); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(total, a.slices), dim3(waves * 64), lds, stream, a);
@@ -647,7 +779,7 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
   return hipGetLastError();
 }
 
-hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
+hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw) {
   SkinnyArgs a;
   a.x = g.x;
   a.r = g.r;
@@ -686,10 +818,15 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
     const bool wide = cols >= 64L * num_cus;
     if (env_waves < 1) waves = wide ? 4 : (g.M <= 32 ? 8 : 6);  // staging tiles: 18 / 13.5 / 22.5 KB of LDS per wave
     if (waves > (g.K >> 8)) waves = g.K >> 8;
-    if (g.M <= 32) return wide ? launch_skinny_t<1, 2, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true>(a, waves, num_cus, ws_bytes, stream);
+    if (raw && !skinny_raw_form(g)) return hipErrorInvalidValue;
+    if (g.M <= 32) {
+      if (raw) return wide ? launch_skinny_t<1, 2, true, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true, true>(a, waves, num_cus, ws_bytes, stream);
+      return wide ? launch_skinny_t<1, 2, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true>(a, waves, num_cus, ws_bytes, stream);
+    }
     if (!wide) {
       if (waves > 6) waves = 6;
-      return launch_skinny_t<2, 1, true>(a, waves, num_cus, ws_bytes, stream);  // 2 x 2 tiles do not fit the register file with the staging
+      // 2 x 2 tiles do not fit the register file with the staging
+      return raw ? launch_skinny_t<2, 1, true, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<2, 1, true>(a, waves, num_cus, ws_bytes, stream);
     }
     // many columns and more than 32 rows: two passes of 32 rows over the wide tile beat one pass over the narrow one
     for (int m0 = 0; m0 < g.M; m0 += 32) {
@@ -698,11 +835,12 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream) {
       c.x = a.x + (size_t)m0 * g.K;
       c.r = a.r ? a.r + (size_t)m0 * g.rank : nullptr;
       for (int i = 0; i < g.n_members; ++i) c.mem[i].y = a.mem[i].y + (size_t)m0 * a.mem[i].ldy;
-      hipError_t e = launch_skinny_t<1, 2, true>(c, waves, num_cus, ws_bytes, stream);
+      hipError_t e = raw ? launch_skinny_t<1, 2, true, true>(c, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 2, true>(c, waves, num_cus, ws_bytes, stream);
       if (e != hipSuccess) return e;
     }
     return hipSuccess;
   }
+  if (raw) return hipErrorInvalidValue;
   const int kblocks = g.K >> 6;
   if (waves > kblocks) waves = kblocks;
   if (g.M <= 32) return launch_skinny_t<1, 2, false>(a, waves, num_cus, ws_bytes, stream);

@@ -456,12 +456,13 @@ class W4A16Extension:
 
     def route(self, M: int, K: int, N: int, group_size: int = 128) -> str:
         names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv", 5: "stream_gemv",
-                 6: "quad_stream_gemv"}
+                 6: "quad_stream_gemv", 7: "skinny_codes_mfma"}
         return names[self.lib.glowq_w4a16_route(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
 
     def set_tuning(self, key: str, value: int) -> int:
         """Sets a route limit of the process ("quad_max_m", "quad_min_m", "wave_dot_max_m", "skinny_max_m",
-        "small_group_mb", "stream_max_m", "stream_shape_rule", "qstream_max_m"); returns the old value."""
+        "small_group_mb", "stream_max_m", "stream_shape_rule", "qstream_max_m", "qstream_shape_rule",
+        "skinny_codes_max_m"); returns the old value."""
         old = self.lib.glowq_set_tuning(key.encode(), int(value))
         if old < 0:
             raise ValueError(self.lib.glowq_last_error().decode())

@@ -63,8 +63,9 @@ const char* glowq_last_error(void);
  * Replaces `w4a16_gemv_forward_cuda` (src/cuda_w4a16/csrc/gemv_w4a16.cu:146-214; pybind
  * src/cuda_w4a16/csrc/pybind.cpp:19-23).  Any M is accepted; all M rows share one pass over the weights.
  * Weight rounding by row count: the GEMV kernels (1 token row; 2..4 rows by group size, see glowq_set_tuning) keep
- * (code - zero) * scale unrounded, as the reference's GEMV does (gemv_w4a16.cu:96-112).  From the row count at which
- * the MFMA kernels take over (3..5 rows, glowq_w4a16_route tells) the dequantised weight is rounded once to fp16
+ * (code - zero) * scale unrounded, as the reference's GEMV does (gemv_w4a16.cu:96-112), and so does the raw-code
+ * form of the skinny MFMA kernel (route 7: 5..8 rows by default, where K is a multiple of 256 and the groups have 128
+ * columns).  On the other MFMA routes (1 and 2, glowq_w4a16_route tells) the dequantised weight is rounded once to fp16
  * before the multiply, which is the arithmetic of the reference's dequantise-then-matmul route (gemm_w4a16.cu:46-49,132)
  * -- the reference itself switches to that arithmetic only above 128 rows.  On activations of order one the two differ
  * by far less than 1e-2 + 1e-3 |y|; with outlier channels in the thousands they differ by more than that, in the
@@ -192,7 +193,9 @@ size_t glowq_static_scratch_bytes(void);
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,
  * 2 = tiled MFMA GEMM, 3 = generic (odd shapes), 4 = 4x4x4 matrix-core GEMV, 5 = stream GEMV (every request of a
  * wave in flight up front; the default at one token row), 6 = the 4x4x4 matrix-core GEMV under the stream GEMV's
- * memory schedule (the default at two to four token rows).
+ * memory schedule (the default at two to four token rows), 7 = skinny MFMA with the int4 codes fed to the matrix
+ * cores as they are and scale and zero-point applied to each group's sum (unrounded arithmetic; the default at five to
+ * eight token rows).
  */
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
 
@@ -211,9 +214,11 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * is used where it applies (groups of 128 to 2048 columns, rank a multiple of 8 up to 128 or of 16 up to 256, rows
  * up to 16384 columns), ahead of all others; 0 switches it off.  "qstream_shape_rule" (0 / 1): only for the shapes it
  * was measured faster on (1, the default) or for every shape it can take (0).
+ * "skinny_codes_max_m" (0..64, default 8): token rows up to which the skinny MFMA kernel runs in its raw-code form
+ * (route 7) where that applies; above it is slower than dequantising first (the work on the sums grows with the rows).
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
  * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M, GLOWQ_STREAM_SHAPE_RULE,
- * GLOWQ_QSTREAM_M and GLOWQ_QSTREAM_SHAPE_RULE.
+ * GLOWQ_QSTREAM_M, GLOWQ_QSTREAM_SHAPE_RULE and GLOWQ_SKINNY_CODES_M.
  */
 int glowq_set_tuning(const char* key, int value);
 

@@ -29,7 +29,7 @@ MODELS = {
                       "down": (17408, [5120])}),
 }
 GROUPS = ["qkv", "o", "gate_up", "down"]
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma"}
 
 
 def _layer(model, name, M, seed, bias=False):

@@ -20,7 +20,7 @@ from helpers import ABS_TOL, REL_TOL, dev, make_group, outlier_activations
 
 pytestmark = pytest.mark.gpu
 
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma"}
 
 # (token rows, K, member widths, rank, route mode); the default limits send 1 row to the wave-dot GEMV, 2..4 rows to the
 # wave-dot GEMV, the 4x4x4 GEMV or the skinny kernel by group size, 5..64 to the skinny kernel, more to the tiled GEMM

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 ROWS = [1, 2, 3, 4, 5, 7, 8, 13, 16, 17, 31, 32, 33, 48, 64, 65, 100, 130, 257]
 ROUTES = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv", 5: "stream_gemv",
-          6: "quad_stream_gemv"}
+          6: "quad_stream_gemv", 7: "skinny_codes_mfma"}
 
 
 def random_cases(n, seed=20240):

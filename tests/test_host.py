@@ -326,13 +326,13 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     ext.set_tuning("stream_shape_rule", rule)
     stream = ext.set_tuning("stream_max_m", 0)                                  # the routes behind it
     old = ext.set_tuning("quad_max_m", 0)
-    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096) == "skinny_mfma"
+    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096) == "skinny_codes_mfma"
     ext.set_tuning("quad_max_m", 16)
     assert ext.route(8, 4096, 4096) == "quad_mfma_gemv"
     ext.set_tuning("quad_max_m", old)
     # 2..4 rows: small groups stay on the wave-dot GEMV, large ones take the 4x4x4 matrix-core GEMV
     assert ext.route(2, 4096, 4096) == "wave_dot_gemv" and ext.route(2, 4096, 28672) == "quad_mfma_gemv"
-    assert ext.route(4, 4096, 4096) == "skinny_mfma" and ext.route(4, 14336, 4096) == "quad_mfma_gemv"
+    assert ext.route(4, 4096, 4096) == "skinny_codes_mfma" and ext.route(4, 14336, 4096) == "quad_mfma_gemv"
     old = ext.set_tuning("small_group_mb", 0)
     assert ext.route(2, 4096, 4096) == "quad_mfma_gemv"
     ext.set_tuning("small_group_mb", old)
