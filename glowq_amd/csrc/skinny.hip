@@ -709,8 +709,7 @@ bool skinny_group_form(const GroupDev& g) {
 // arithmetic is that of the GEMV routes (weights never rounded to fp16), so the route table reports it as a route of its
 // own.
 bool skinny_raw_form(const GroupDev& g) {
-  static const int env_raw = getenv("GLOWQ_SKINNY_RAW") ? atoi(getenv("GLOWQ_SKINNY_RAW")) : 1;
-  if (env_raw == 0 || !skinny_group_form(g) || g.group_size != 128) return false;
+  if (!skinny_group_form(g) || g.group_size != 128) return false;
   for (int i = 0; i < g.n_members; ++i)
     if ((g.mem[i].lds & 1) != 0 || (reinterpret_cast<uintptr_t>(g.mem[i].scales) & 3u) != 0) return false;
   return true;
