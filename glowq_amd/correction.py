@@ -137,7 +137,11 @@ class AddSVDCorrection(nn.Module):
         key = (tuple(id(w) for w in wrappers), float(self.alpha_svd), corrected)
         cache = self.__dict__.setdefault("_prepared_groups", {})
         hit = cache.get(key)
-        ptrs = (self.A_q.data_ptr(), self.B_q.data_ptr())
+        # every tensor whose address sits in the descriptors: a buffer replaced by assignment (re-quantisation,
+        # load_state_dict(assign=True), a follower's factor swapped) rebuilds them
+        ptrs = (self.B_q.data_ptr(),) + tuple(
+            p for w in wrappers for p in (w.A_q.data_ptr(), w.inner.qweight_i32.data_ptr(), w.inner.scales_f16.data_ptr(),
+                                          w.inner.qzeros_i32.data_ptr(), w.inner.bias.data_ptr() if w.inner.bias is not None else 0))
         if hit is not None and hit[0] == ptrs and hit[1].generation == _kernels.generation():
             return hit[1]
         members = []
@@ -159,6 +163,7 @@ class AddSVDCorrection(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         inner = self.inner
+        KNOBS.sync()
         if self.alpha_svd == 0.0:
             # the reference returns inner(x) untouched (step3_eval_dataset.py:473-474)
             return inner(x)

@@ -63,11 +63,11 @@ namespace {
 // keeps its copy at comes from hipGetSymbolAddress, asked once per device with that device current.
 std::atomic<void*> g_scratch_ptr[64] = {};
 
-void* static_scratch() {
+void* static_scratch(bool lookup_allowed = true) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
-  if (p != nullptr) return p;
+  if (p != nullptr || !lookup_allowed) return p;
   if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return nullptr;
   g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing host threads store the same address
   return p;
@@ -642,13 +642,25 @@ int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r
   if (need > kStaticScratchBytes)
     return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: this shape wants %zu bytes of scratch, the static buffer holds %zu",
                 need, kStaticScratchBytes);
-  void* ws = static_scratch();
+  void* ws = static_scratch(false);
+  if (ws == nullptr) {
+    // first use on this device: the lookup must not run under a stream capture
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: call glowq_static_scratch_prepare() on this device before capturing");
+    ws = static_scratch();
+  }
   if (ws == nullptr) return fail(GLOWQ_ELAUNCH, "group_forward_fused_static: the address of the static scratch is not available");
   return group_forward_fused_impl(x, R, r_out, members, n_members, M, K, group_size, rank, alpha, ws, kStaticScratchBytes,
                                   stream);
 }
 
 size_t glowq_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int glowq_static_scratch_prepare(void) {
+  if (static_scratch() == nullptr) return fail(GLOWQ_ELAUNCH, "static_scratch_prepare: the address of the static scratch is not available");
+  return GLOWQ_OK;
+}
 
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
   GroupDev g;

@@ -278,9 +278,19 @@ __global__ __launch_bounds__(1024) void rope_attend_kernel(const half_t* __restr
     v0 = v_new[(size_t)kvh * d + i], v1 = v_new[(size_t)kvh * d + i + half_d];
   }
   const int pos = (int)*pos_p;
-  // A position outside the cache (a caller stepping past max_len - 1): nothing is written -- no cache row, no output,
-  // no partial -- instead of indexing the tables and the caches out of bounds.  Uniform over the grid.
-  if (pos < 0 || pos >= max_len) return;
+  // A position outside the cache (a caller stepping past max_len - 1): the tables and the caches are not indexed out of
+  // bounds and no cache row is written; the output (or this workgroup's partial) becomes NaN, so that everything
+  // computed from this step says so instead of carrying the last step's values on.  Uniform over the grid.
+  if (pos < 0 || pos >= max_len) {
+    const float bad = __builtin_nanf("");
+    if (part) {
+      float* mine = part + ((size_t)head * splits + split) * (d + 4);
+      for (int i = threadIdx.x; i < d + 4; i += blockDim.x) mine[i] = bad;
+    } else {
+      for (int i = threadIdx.x; i < d; i += blockDim.x) out[(size_t)head * d + i] = (half_t)bad;
+    }
+    return;
+  }
 
   // rotary embedding of q and k_new: out[i] = x[i] cos - x[i + d/2] sin, out[i + d/2] = x[i + d/2] cos + x[i] sin
   if (threadIdx.x < half_d) {

@@ -18,8 +18,10 @@ size_t wave_dot_lds_bytes(int M, int K, int rank, bool has_r);
 bool stream_supported(const GroupDev& g) {
   if (g.M < 1 || g.M > 4 || (g.K & 31) != 0 || g.K > 9 * 2048) return false;
   if (g.group_size < 128 || (g.group_size & (g.group_size - 1)) != 0) return false;
-  const bool has_r = g.r != nullptr;
-  if (has_r && ((g.rank & 1) != 0 || g.rank > 256 || g.rank < 2 || (reinterpret_cast<uintptr_t>(g.r) & 3u) != 0)) return false;
+  // r is either given or still to be produced from R into r_out by the projection launch that goes ahead of the group
+  const half_t* r = g.r != nullptr ? g.r : (g.R != nullptr ? g.r_out : nullptr);
+  const bool has_r = r != nullptr;
+  if (has_r && ((g.rank & 1) != 0 || g.rank > 256 || g.rank < 2 || (reinterpret_cast<uintptr_t>(r) & 3u) != 0)) return false;
   if ((reinterpret_cast<uintptr_t>(g.x) & 15u) != 0) return false;
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
@@ -72,7 +74,8 @@ hipError_t launch_stream_lw(GroupDev& g, int waves, hipStream_t stream) {
   const int lw = g.r ? (g.rank + 127) / 128 : 0;
   if (lw == 0) return launch_stream_m<kKit, 0>(g, waves, stream);
   if (lw == 1) return launch_stream_m<kKit, 1>(g, waves, stream);
-  return launch_stream_m<kKit, 2>(g, waves, stream);
+  if (lw == 2) return launch_stream_m<kKit, 2>(g, waves, stream);
+  return hipErrorInvalidValue;  // ranks above 256 belong to the wave-dot GEMV (stream_supported)
 }
 
 int env_int_s(const char* name, int fallback) {

@@ -68,6 +68,7 @@ _SIGNATURES = {
                                                 _P, ctypes.c_size_t, _P]),
     "glowq_w4a16_group_forward_fused_static": (_I, [_P, _P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),
     "glowq_static_scratch_bytes": (ctypes.c_size_t, []),
+    "glowq_static_scratch_prepare": (_I, []),
     "glowq_side_bytes": (ctypes.c_size_t, [_I, _I, _I, _I]),
     "glowq_pack_side": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "glowq_w4a16_group_forward": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, _I, ctypes.c_float, _P]),

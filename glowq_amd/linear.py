@@ -55,30 +55,41 @@ def _get_kernel_out_dtype() -> torch.dtype:
     return torch.float16 if v in ("fp16", "float16", "half") else torch.float32
 
 
-class _Knobs:
-    """The `W4A16_*` switches a forward depends on, read from the environment ONCE (at import, and again by
-    `refresh_env_knobs()`), not on every call as the reference does (linear.py:172-177).  `_configure_cuda_w4a16_env`
-    refreshes them itself; code that edits `os.environ` by hand afterwards calls `refresh_env_knobs()`."""
+_KNOB_ENV = ("W4A16_KERNEL_OUT_DTYPE", "MIXED_KERNEL_OUT_DTYPE", "W4A16_FORCE_GEMM", "CUDA_MIXED_FORCE_GEMM",
+             "W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV", "W4A16_USE_GEMV", "W4A16_SPLIT_K_ITERS")
 
-    __slots__ = ("out_dtype", "force_gemm", "force_gemv", "use_gemv", "split_k_iters")
+
+class _Knobs:
+    """The `W4A16_*` switches a forward depends on.  The reference reads them from the environment on every forward
+    (linear.py:172-177); here they are parsed once and a forward only compares the raw strings with the ones it parsed
+    last (`sync`), so a switch set with `os.environ[...] = ...` after import is honoured by the next forward, as in the
+    reference, without parsing anything on the calls in between."""
+
+    __slots__ = ("out_dtype", "force_gemm", "force_gemv", "use_gemv", "split_k_iters", "_raw")
 
     def __init__(self):
         self.read()
 
     def read(self) -> None:
+        self._raw = tuple(map(os.environ.get, _KNOB_ENV))
         self.out_dtype = _get_kernel_out_dtype()
         self.force_gemm = _env_flag("W4A16_FORCE_GEMM", "CUDA_MIXED_FORCE_GEMM")
         self.force_gemv = _env_flag("W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV")
         self.use_gemv = _env_flag("W4A16_USE_GEMV")
         self.split_k_iters = _env_number("W4A16_SPLIT_K_ITERS", default=1)
 
+    def sync(self) -> None:
+        if tuple(map(os.environ.get, _KNOB_ENV)) != self._raw:
+            self.read()
+
 
 KNOBS = _Knobs()
 
 
 def refresh_env_knobs() -> None:
-    """Re-reads the `W4A16_*` environment switches (output dtype, forced routes, split-K iterations) for every module.
-    The row threshold `W4A16_GEMV_M_MAX` is read when a module is constructed, as in the reference (linear.py:120)."""
+    """Re-reads the `W4A16_*` environment switches (output dtype, forced routes, split-K iterations) for every module;
+    every forward does the same when one of their strings has changed.  The row threshold `W4A16_GEMV_M_MAX` is read when
+    a module is constructed, as in the reference (linear.py:120)."""
     KNOBS.read()
 
 
@@ -191,17 +202,21 @@ class CudaW4A16Linear(nn.Module):
     def _bare_group(self):
         """The module alone as a prepared group (validated once, side stream packed once); rebuilt when a buffer has
         been replaced since."""
+        # the bias rides in the kernel's epilogue, y = fp16(acc + bias), where the output stays fp16; with fp32 output the
+        # reference adds it in fp32 after the cast (linear.py:183-186) and so does `_finish`
+        fold_bias = self.bias is not None and KNOBS.out_dtype == torch.float16
         key = (self.qweight_i32.data_ptr(), self.scales_f16.data_ptr(), self.qzeros_i32.data_ptr(),
-               self.bias.data_ptr() if self.bias is not None else 0)
+               self.bias.data_ptr() if fold_bias else 0)
         if self._prepared is None or self._prepared[0] != key:
             from .kernels import PreparedGroup
 
             member = self._member()
-            member["bias"] = self.bias.data if self.bias is not None else None
+            member["bias"] = self.bias.data if fold_bias else None
             self._prepared = (key, PreparedGroup(self._get_ext(), [member], self.in_features, self.group_size, 0.0))
         return self._prepared[1]
 
     def _prefer_gemv(self, m: int) -> bool:
+        KNOBS.sync()
         if KNOBS.force_gemm:
             return False
         return KNOBS.force_gemv or KNOBS.use_gemv or m <= self._gemv_threshold
@@ -223,12 +238,13 @@ class CudaW4A16Linear(nn.Module):
         lead = x.shape[:-1]
         x2d = self._as_rows(x)
         self._require_gpu(x2d)
+        KNOBS.sync()
         if KNOBS.force_gemm or (not self._prefer_gemv(x2d.size(0))):
             out = self._get_ext().w4a16_gemm_forward_cuda(x2d, self.qweight_i32, self.scales_f16, self.qzeros_i32,
                                                           self.group_size, KNOBS.split_k_iters)
             return self._finish(out, lead)
         # the decode kernels through descriptors validated once (the bias rides in the kernel's epilogue)
-        return self._finish(self._bare_group().run(x2d)[0], lead, bias_applied=True)
+        return self._finish(self._bare_group().run(x2d)[0], lead, bias_applied=KNOBS.out_dtype == torch.float16)
 
     def dequantize(self) -> torch.Tensor:
         """fp16 [out_features, in_features] weight, fp16((code - zero) * scale); the device twin of the

@@ -182,12 +182,18 @@ int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out
  * the call allocates and frees nothing.  At most GLOWQ_STATIC_MAX_ROWS token rows, and shapes whose projection would
  * want a larger workspace (glowq_proj_workspace_bytes) are refused with GLOWQ_EUNSUPPORTED.  Every call on a GPU shares
  * that GPU's array: calls that overlap on one GPU (two streams, two threads) race; nothing in it has to start at zero.
+ * The first use on a device looks the array's address up (a symbol lookup, possibly a lazy load of the code object):
+ * a caller that records the entry point into a graph calls glowq_static_scratch_prepare() on that device beforehand,
+ * outside the capture; a call on a capturing stream of a device that was never prepared is refused with
+ * GLOWQ_EUNSUPPORTED instead of doing that lookup under capture.
  */
 #define GLOWQ_STATIC_MAX_ROWS 64
 int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r_out, const glowq_member_t* members,
                                            int n_members, int M, int K, int group_size, int rank, float alpha,
                                            void* stream);
 size_t glowq_static_scratch_bytes(void);
+/* Resolves the static scratch of the current device (idempotent, allocates nothing); GLOWQ_OK or GLOWQ_ELAUNCH. */
+int glowq_static_scratch_prepare(void);
 
 /*
  * Kernel route chosen for a given row count, for reporting: 0 = wave-dot GEMV, 1 = skinny MFMA,

@@ -255,7 +255,7 @@ def test_appended_key_is_bit_identical_to_the_tensor_expression(ext, fp16_out):
         run(d, 8, 8, 200, int(rng.integers(0, 200)), 1000 + i, int(rng.choice([2, 4])))
 
 
-def test_position_outside_the_cache_writes_nothing(ext, fp16_out):
+def test_position_outside_the_cache_touches_no_cache_row_and_poisons_the_output(ext, fp16_out):
     heads, kvh, d, max_len = 8, 2, 64, 96
     g = torch.Generator(device="cuda").manual_seed(1)
     q = torch.randn(heads * d, device="cuda", generator=g).half()
@@ -274,7 +274,12 @@ def test_position_outside_the_cache_writes_nothing(ext, fp16_out):
         ext.rope_attend(q, k, v, cos, sin, p, ck2, cv2, out, d ** -0.5)
         ext.rope_attend_split(q, k, v, cos, sin, p, ck2, cv2, part, d ** -0.5)
         torch.cuda.synchronize()
-        assert torch.equal(ck2, ck) and torch.equal(cv2, cv) and (out == 7.0).all() and (part == 7.0).all()
+        assert torch.equal(ck2, ck) and torch.equal(cv2, cv)
+        # the step is marked, not silently skipped: whatever is computed from it is NaN
+        assert torch.isnan(out).all() and torch.isnan(part).all()
+        merged = torch.empty(heads * d, dtype=torch.float16, device="cuda")
+        ext.attend_combine_proj(part, merged)
+        assert torch.isnan(merged).all()
 
 
 @pytest.mark.parametrize("pos,splits", [(0, 4), (1, 4), (3, 8), (37, 4), (300, 4), (300, 7)])

@@ -55,3 +55,22 @@ def test_fused_equals_two_launch_form(ext, small_m_route):
     assert np.abs(r1.float().cpu().numpy() - r2.float().cpu().numpy()).max() <= 2e-3
     for a, b in zip(one, two):
         assert np.abs(a.float().cpu().numpy() - b.float().cpu().numpy()).max() <= 4e-3
+
+
+@pytest.mark.parametrize("M", [1, 3])
+@pytest.mark.parametrize("rank", [384, 512])
+def test_fused_call_with_a_rank_above_the_stream_gemv(ext, M, rank):
+    """The stream GEMV holds at most 256 columns of L per row; a fused call (r still to be produced from R when the
+    route is picked) with a larger rank has to land on a route that applies all of L r."""
+    K, Ns = 4096, [192, 64]
+    x, members, R = make_group(500 + rank + M, M, K, Ns, rank)
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]), "L": dev(m["L"])} for m in members]
+    r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+    outs = ext.group_forward(dev(x), r, mem, 128, 1.0, R=dev(R))
+    torch.cuda.synchronize()
+    for i, (m, y) in enumerate(zip(members, outs)):
+        want = oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0)
+        assert_close(y.cpu().numpy(), want, f"rank {rank} member {i}")
+        # the correction is not small against the tolerance here: losing the columns past 256 would be seen
+        bare = oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)
+        assert np.abs(want - bare).max() > 5e-2

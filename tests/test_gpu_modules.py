@@ -45,10 +45,12 @@ def test_converted_linear_forward(fp16_out, monkeypatch):
         assert_close(y.cpu().numpy().reshape(-1, 96), _ref(x.numpy().reshape(-1, 512), mod), f"linear {shape}")
     # fp32 inputs are cast; fp32 output is the reference's module default
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp32")
-    assert mod(torch.randn(4, 512).cuda()).dtype == torch.float16      # the switches are cached: not honoured yet ...
-    linear.refresh_env_knobs()
-    y32 = mod(torch.randn(4, 512).cuda())
-    assert y32.dtype == torch.float32                                   # ... but after a refresh
+    x4 = torch.randn(4, 512).half()
+    y32 = mod(x4.cuda())                                                # a switch set after import is seen by the next forward
+    assert y32.dtype == torch.float32
+    # with fp32 output the bias is added in fp32 after the cast of the fp16 kernel output (linear.py:183-186)
+    bare = mod._bare_group().run(x4.cuda())[0]
+    assert torch.equal(y32, bare.float() + mod.bias.float())
     # forced routes agree with each other within tolerance
     x = torch.randn(3, 512).half()
     monkeypatch.setenv("W4A16_KERNEL_OUT_DTYPE", "fp16")
@@ -119,6 +121,30 @@ def test_followers_recompute_on_miss_and_on_a_different_input(fp16_out):
     sa.q_proj(x1.cuda()); sa.q_proj(x2.cuda())
     yv = sa.v_proj(x2.cuda())
     assert_close(yv.cpu().numpy(), _ref(x2.numpy(), sa.v_proj.inner, shared["layer1_qkv.v_proj.A"], R), "v after 2x q")
+
+
+def test_replaced_buffers_are_picked_up_by_the_next_forward(fp16_out):
+    """The group launch runs on descriptors built once from tensor addresses: a follower's factor or a member's weight
+    replaced by attribute assignment (re-quantisation, cumulative patching) must rebuild them."""
+    model, shared = _patched_toy()
+    sa = model.model.layers[0].self_attn
+    R = shared["layer0_qkv.B_shared"]
+    x = torch.randn(2, 256).half()
+    xd = x.cuda()
+    sa.q_proj(xd), sa.k_proj(xd), sa.v_proj(xd)  # descriptors of the three-member group exist now
+    new_A = (torch.randn_like(sa.k_proj.A_q) * 0.05).contiguous()
+    sa.k_proj.A_q = new_A                        # a follower's left factor swapped
+    lin = nn.Linear(256, 64, bias=True).half()
+    lin.weight.data.mul_(0.3)
+    fresh = linear.CudaW4A16Linear.from_float(lin, 128).cuda()
+    sa.v_proj.inner.qweight_i32 = fresh.qweight_i32  # a member re-quantised in place
+    sa.v_proj.inner.scales_f16 = fresh.scales_f16
+    sa.v_proj.inner.qzeros_i32 = fresh.qzeros_i32
+    yq, yk, yv = sa.q_proj(xd), sa.k_proj(xd), sa.v_proj(xd)
+    torch.cuda.synchronize()
+    assert_close(yk.cpu().numpy(), _ref(x.numpy(), sa.k_proj.inner, new_A, R), "k after its factor was replaced")
+    assert_close(yv.cpu().numpy(), _ref(x.numpy(), sa.v_proj.inner, shared["layer0_qkv.v_proj.A"], R), "v after re-quantisation")
+    assert_close(yq.cpu().numpy(), _ref(x.numpy(), sa.q_proj.inner, shared["layer0_qkv.q_proj.A"], R), "q unchanged")
 
 
 def test_alpha_switch_and_scaling(fp16_out):

@@ -96,16 +96,17 @@ def test_env_knobs(monkeypatch):
     monkeypatch.setenv("W4A16_GEMV_M_MAX", "7")
     m = linear.CudaW4A16Linear(64, 8, 32)
     assert m._gemv_threshold == 7 and m._prefer_gemv(7) and not m._prefer_gemv(8)
+    assert not m._prefer_gemv(1000)
     monkeypatch.setenv("W4A16_FORCE_GEMV", "1")
-    assert not m._prefer_gemv(1000)            # forced routes are read once and again on refresh, not per call
-    linear.refresh_env_knobs()
-    assert m._prefer_gemv(1000)
+    assert m._prefer_gemv(1000)                # as in the reference, a switch set between two forwards is seen by the next
     monkeypatch.setenv("W4A16_FORCE_GEMM", "true")
-    linear.refresh_env_knobs()
     assert not m._prefer_gemv(1)
     monkeypatch.setenv("W4A16_SPLIT_K_ITERS", "4")
-    linear.refresh_env_knobs()
+    linear.KNOBS.sync()
     assert linear.KNOBS.split_k_iters == 4 and linear.KNOBS.out_dtype == torch.float16
+    raw = linear.KNOBS._raw
+    linear.KNOBS.sync()                        # nothing changed: nothing is parsed again
+    assert linear.KNOBS._raw is raw
     monkeypatch.delenv("W4A16_GEMV_M_MAX")
     monkeypatch.setenv("CUDA_MIXED_GEMV_M_MAX", "3")  # legacy alias
     assert linear.CudaW4A16Linear(64, 8, 32)._gemv_threshold == 3

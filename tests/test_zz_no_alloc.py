@@ -102,3 +102,42 @@ def test_static_scratch_entry_point_refuses_what_it_cannot_hold(ext):
     rc = ext.lib.glowq_w4a16_group_forward_fused_static(x.data_ptr(), None, r.data_ptr(), arr, 1, 8, K, GS, rank, 1.0,
                                                         torch.cuda.current_stream().cuda_stream)
     assert rc == -1                                            # the argument checks of the workspace entry point apply
+
+
+def test_static_scratch_entry_point_under_graph_capture(ext):
+    """Recorded into a HIP graph after glowq_static_scratch_prepare() and replayed with eager work in between: every
+    replay equals the workspace entry point bit for bit."""
+    assert ext.lib.glowq_static_scratch_prepare() == 0
+    g = torch.Generator(device="cuda").manual_seed(9)
+    M, K, Ns, rank = 24, 14336, [1024, 256], 128
+    x = torch.randn(M, K, device="cuda", generator=g).half()
+    R = (torch.randn(rank, K, device="cuda", generator=g) * K ** -0.5).half()
+    members = [_random_member(g, N, K, rank) for N in Ns]
+    ws = torch.empty(ext.lib.glowq_static_scratch_bytes(), dtype=torch.uint8, device="cuda")
+    outs_ws = [torch.empty((M, N), dtype=torch.float16, device="cuda") for N in Ns]
+    r_ws = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+    outs_st = [torch.empty((M, N), dtype=torch.float16, device="cuda") for N in Ns]
+    r_st = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+    arr_ws, arr_st = _descriptors(members, outs_ws), _descriptors(members, outs_st)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = ext.lib.glowq_w4a16_group_forward_fused_static(x.data_ptr(), R.data_ptr(), r_st.data_ptr(), arr_st, len(Ns), M, K,
+                                                                GS, rank, 1.0, side.cuda_stream)
+    assert rc == 0, ext.lib.glowq_last_error()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.copy_(torch.randn(M, K, device="cuda", generator=g).half())   # eager work between the replays
+        for t in outs_st + [r_st]:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        rc = ext.lib.glowq_w4a16_group_forward_fused_ws(x.data_ptr(), R.data_ptr(), r_ws.data_ptr(), arr_ws, len(Ns), M, K, GS,
+                                                        rank, 1.0, ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, ext.lib.glowq_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(r_ws, r_st), f"replay {rep}"
+        for a, b in zip(outs_ws, outs_st):
+            assert torch.equal(a, b) and torch.isfinite(b.float()).all(), f"replay {rep}"
