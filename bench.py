@@ -313,6 +313,53 @@ def selective_leg(torch, ext, dev):
     return out
 
 
+def stream_read_probe(torch, ext, capture, pool, sink, nbytes, launch):
+    """GB/s of the library's bare streaming-read kernel over `nbytes` per launch, launched with the grid and workgroup
+    size of `launch` on the buffers of `pool` in turn (None where the launch record holds no grid)."""
+    if not launch["grid"][0] or not launch["block"]:
+        return None
+    nbytes = nbytes // 16 * 16
+    dev = pool[0].device
+    gr = capture(lambda: [ext.lib.glowq_probe_stream_read(b.data_ptr(), nbytes, sink.data_ptr(), launch["grid"][0] * max(1, launch["grid"][1]),
+                                                          launch["block"], ext._stream(dev)) for b in pool])
+    us = timed_replays(torch, gr, 20) * 1e3 / len(pool)
+    return round(nbytes / us / 1e3, 1)
+
+
+def module_eager_leg(torch, model, iters=300):
+    """Host cost of the torch modules outside a graph: wall time per module-group forward at one token (the q|k|v
+    wrappers fuse into one library call on the lead's forward, gate|up likewise), launches queued without waiting for
+    the GPU, on the first layer of the decode loop's model."""
+    layer = model.model.layers[0]
+    attn, mlp = layer.self_attn, layer.mlp
+    dev = next(model.parameters()).device
+    cfg = model.cfg
+    x = torch.randn(1, cfg.hidden, device=dev).half()
+    a = torch.randn(1, cfg.heads * cfg.head_dim, device=dev).half()
+    h = torch.randn(1, cfg.intermediate, device=dev).half()
+    groups = {
+        "qkv": lambda: (attn.q_proj(x), attn.k_proj(x), attn.v_proj(x)),
+        "o_proj": lambda: attn.o_proj(a),
+        "gate_up": lambda: (mlp.gate_proj(x), mlp.up_proj(x)),
+        "down_proj": lambda: mlp.down_proj(h),
+    }
+    out = {}
+    with torch.no_grad():
+        for name, fn in groups.items():
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                fn()
+            host = time.perf_counter() - t0   # the queue is not waited for: host time per call unless the GPU is slower
+            torch.cuda.synchronize()
+            total = time.perf_counter() - t0
+            out[name] = {"host_us_per_group_forward": round(host / iters * 1e6, 2), "with_gpu_drain_us": round(total / iters * 1e6, 2)}
+    out["sum_host_us_per_layer"] = round(sum(v["host_us_per_group_forward"] for v in out.values()), 2)
+    return out
+
+
 def calibrate_copy(torch, dev, graph):
     """Eight plain device copies of 256 MiB each from cold sources (the kernel shows up in a profile as a copy kernel):
     262144 KiB read and 262144 KiB written per copy, the yardstick the FETCH_SIZE / WRITE_SIZE counts are scaled by."""
@@ -326,9 +373,9 @@ def calibrate_copy(torch, dev, graph):
 
 
 def summarize_pmc(fetch_csv, write_csv):
-    """Reads the per-dispatch counter files of two rocprofv3 --pmc runs of `bench.py --dominant-only --calibrate-copy`
-    (FETCH_SIZE, then WRITE_SIZE) and writes the traffic sidecar: bytes per launch of the dominant kernel, each counter
-    scaled by what it reads for the 256 MiB device copies of the same run."""
+    """Reads the per-dispatch counter files of two rocprofv3 --pmc runs of `bench.py --groups-only --calibrate-copy`
+    (FETCH_SIZE, then WRITE_SIZE) and writes the traffic sidecar: bytes per launch of every group's GEMV launch, each
+    counter scaled by what it reads for the 256 MiB device copies of the same run.  The only writer of that file."""
     import csv
 
     def per_kernel(path, counter):
@@ -336,38 +383,65 @@ def summarize_pmc(fetch_csv, write_csv):
         with open(path, newline="") as f:
             for row in csv.DictReader(f):
                 if row.get("Counter_Name") == counter:
-                    per.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+                    per.setdefault((row["Kernel_Name"], int(row.get("Grid_Size", 0) or 0)), []).append(float(row["Counter_Value"]))
         return per
 
+    # a stream GEMV launch is one wave per two output rows: threads = 32 N; its first template argument is ceil(K / 2048)
+    label = {(-(-K // 2048), 32 * sum(Ns)): name for name, (K, Ns) in GROUPS.items()}
     out = {"kernel": None, "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py "
-                                      "--dominant-only --calibrate-copy", "copy_bytes_each_way": 256 << 20}
-    total = 0.0
+                                      "--groups-only --calibrate-copy", "copy_bytes_each_way": 256 << 20, "groups": {}}
     for path, counter in ((fetch_csv, "FETCH_SIZE"), (write_csv, "WRITE_SIZE")):
         per = per_kernel(path, counter)
         # the 256 MiB copies are the largest dispatches of any copy kernel in the run (smaller ones move parameters)
-        copies = [v for k, vs in per.items() if "copy" in k.lower() for v in vs]
-        dom = [k for k in per if "gemv_stream_kernel" in k or "gemv_wave_dot_kernel" in k]
-        if not copies or not dom:
-            raise SystemExit(f"{path}: need the copy kernel and the GEMV kernel in the counter file, found {sorted(per)}")
+        copies = [v for (k, _), vs in per.items() if "copy" in k.lower() for v in vs]
+        gemv = {key: vs for key, vs in per.items() if "gemv_stream_kernel" in key[0] or "gemv_wave_dot_kernel" in key[0]}
+        if not copies or not gemv:
+            raise SystemExit(f"{path}: need the copy kernel and the GEMV kernels in the counter file, found {sorted(k for k, _ in per)}")
         big = [v for v in copies if v >= 0.5 * max(copies)]
-        per_copy, per_launch = sum(big) / len(big), sum(per[dom[0]]) / len(per[dom[0]])
+        per_copy = sum(big) / len(big)
         factor = (256 << 20) / 1024.0 / per_copy          # KiB per count
-        kib = per_launch * factor
-        out["kernel"] = dom[0][:120]
-        out[counter] = {"count_per_launch": round(per_launch, 1), "count_per_copy": round(per_copy, 1),
-                        "KiB_per_count": round(factor, 4), "KiB_per_launch": round(kib, 1)}
-        total += kib * 1024.0
-    out["traffic_bytes_per_launch"] = int(round(total))
+        out[counter + "_KiB_per_count"] = round(factor, 4)
+        out[counter + "_count_per_copy"] = round(per_copy, 1)
+        for (kname, threads), vs in gemv.items():
+            targs = template_args(kname) or [0]
+            name = label.get((targs[0], threads), f"{threads} threads")
+            entry = out["groups"].setdefault(name, {"kernel": kname[:140], "launches_counted": len(vs)})
+            entry[counter + "_KiB_per_launch"] = round(sum(vs) / len(vs) * factor, 1)
+    for name, entry in out["groups"].items():
+        K, Ns = GROUPS.get(name, (0, [0]))
+        entry["algorithmic_KiB_per_launch"] = round((algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK) - 2 * RANK * K) / 1024.0, 1) if K else None
+        entry["traffic_bytes_per_launch"] = int(round((entry.get("FETCH_SIZE_KiB_per_launch", 0) + entry.get("WRITE_SIZE_KiB_per_launch", 0)) * 1024))
+    if DOMINANT not in out["groups"]:
+        raise SystemExit(f"no launch of the {DOMINANT} group in the counter files: {sorted(out['groups'])}")
+    out["kernel"] = out["groups"][DOMINANT]["kernel"]
+    out["traffic_bytes_per_launch"] = out["groups"][DOMINANT]["traffic_bytes_per_launch"]
     with open(TRAFFIC_SIDECAR, "w") as f:
         json.dump(out, f, indent=1)
         f.write("\n")
     print(json.dumps(out))
 
 
-def read_traffic_sidecar():
+def template_args(kernel_name):
+    """The integer template arguments of a kernel name, from the mangled symbol a counter file holds (...ILi2ELi1ELb0E...)
+    or from the library's launch record (name<2,1,0,...>)."""
+    import re
+    m = re.search(r"<([0-9, ]+)>", kernel_name)
+    if m:
+        return [int(t) for t in m.group(1).split(",")]
+    m = re.search(r"kernelI((?:L[ib]\d+E)+)E", kernel_name)
+    return [int(t) for t in re.findall(r"L[ib](\d+)E", m.group(1))] if m else None
+
+
+def read_traffic_sidecar(launched_kernel):
+    """Traffic of the dominant launch from the counter file, if that file was taken on the instantiation this run
+    launched (same kernel, same template arguments); else (None, why)."""
     try:
         with open(TRAFFIC_SIDECAR) as f:
             d = json.load(f)
+        counted = d["kernel"]
+        base = launched_kernel.split("<")[0]
+        if base not in counted or template_args(counted) != template_args(launched_kernel):
+            return None, f"{os.path.relpath(TRAFFIC_SIDECAR, ROOT)} was counted on {counted[:100]}, this run launched {launched_kernel}"
         return int(d["traffic_bytes_per_launch"]), os.path.relpath(TRAFFIC_SIDECAR, ROOT)
     except (OSError, ValueError, KeyError):
         return None, None
@@ -384,6 +458,8 @@ def main():
     ap.add_argument("--no-decode-loop", action="store_true", help="skip the full decode loop leg (profiling runs)")
     ap.add_argument("--dominant-only", action="store_true",
                     help="run only the graph of the dominant kernel (32 launches per replay) and print its timing (profiling runs)")
+    ap.add_argument("--groups-only", action="store_true",
+                    help="run only the graph of the four group launches per layer on a given r and print its timing (profiling runs)")
     ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: turn the counter files of two --pmc runs into the traffic sidecar under profiles/")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -451,6 +527,14 @@ def main():
     # the group kernel's own bytes: the group total minus R, which the projection launch reads
     dom_bytes = algorithmic_bytes(M_TOKENS, K_d, sum(Ns_d), RANK) - 2 * RANK * K_d
     gdom = capture(lambda: [run_group(li, DOMINANT, project=False) for li in range(LAYERS)])
+    dom_launch = ext.last_launch()  # the instantiation, grid and workgroup size the library used for it
+    if args.groups_only:
+        gg_ = capture(lambda: [run_group(li, name, project=False) for li in range(LAYERS) for name in GROUPS])
+        us = timed_replays(torch, gg_, max(10, min(args.steps, 50))) * 1e3 / LAYERS
+        if args.calibrate_copy:
+            calibrate_copy(torch, dev, gg_)
+        print(json.dumps({"r_given_us_per_layer": round(us, 3), "dominant_launch": dom_launch}))
+        return
     if args.dominant_only:
         dom_us = timed_replays(torch, gdom, max(10, min(args.steps, 50))) * 1e3 / LAYERS
         if args.calibrate_copy:
@@ -487,6 +571,15 @@ def main():
     given_us = timed_replays(torch, g_given, max(10, min(args.steps, 50))) * 1e3 / LAYERS
     given_bytes = sum(algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK) - 2 * RANK * K for K, Ns in GROUPS.values())
 
+    # what the memory system gives a kernel of the same launch shape that only reads: 32 cold buffers of the launch's
+    # algorithmic bytes each, back to back in one graph like the launches themselves; and the cost of launching nothing
+    pool = [torch.full(((dom_bytes + 15) // 16 * 16,), 1 + i, dtype=torch.uint8, device=dev) for i in range(LAYERS)]
+    sink = torch.zeros(4, dtype=torch.uint8, device=dev)
+    stream_read = stream_read_probe(torch, ext, capture, pool, sink, dom_bytes, dom_launch)
+    g_empty = capture(lambda: [ext.lib.glowq_probe_empty_launch(dom_launch["grid"][0], dom_launch["block"],
+                                                                 ext._stream(dev)) for _ in range(LAYERS)])
+    empty_us = timed_replays(torch, g_empty, 20) * 1e3 / LAYERS
+
     # per-group split of the step, from graphs of one group kind each (reported, not the metric)
     per_group = {}
     for name in GROUPS:
@@ -494,7 +587,10 @@ def main():
         by = algorithmic_bytes(M_TOKENS, K, sum(Ns), RANK)
         us = timed_replays(torch, capture(lambda: [run_group(li, name) for li in range(LAYERS)]), 10) * 1e3 / LAYERS
         us_g = timed_replays(torch, capture(lambda: [run_group(li, name, project=False) for li in range(LAYERS)]), 10) * 1e3 / LAYERS
-        per_group[name] = {"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+        launch = ext.last_launch()
+        read_gbps = stream_read_probe(torch, ext, capture, pool, sink, by - 2 * RANK * K, launch)
+        per_group[name] = {"launch": launch, "stream_read_GBps": read_gbps,
+                           "frac_of_stream_read": round((by - 2 * RANK * K) / us_g / 1e3 / read_gbps, 4) if read_gbps else None,"us": round(us, 3), "GBps": round(by / us / 1e3, 1), "pct_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS * 100, 2),
                            "group_launch_only_us": round(us_g, 3),
                            "group_launch_only_pct_hbm_peak": round((by - 2 * RANK * K) / us_g / 1e3 / HBM_PEAK_GBPS * 100, 2)}
 
@@ -523,12 +619,12 @@ def main():
     if args.calibrate_copy:
         calibrate_copy(torch, dev, graph)
 
-    del layers, calls, graph, gdom, g_given
+    del layers, calls, graph, gdom, g_given, pool, g_empty
     torch.cuda.empty_cache()
     selective = selective_leg(torch, ext, dev)
     # the whole decode loop of the same benchmark (32-layer random-init model, 512-token prompt, 256 new tokens, greedy)
     torch.cuda.empty_cache()
-    decode = None
+    decode, module_eager = None, None
     if not args.no_decode_loop:
         import contextlib
         from glowq_amd import decode as decode_loop
@@ -540,9 +636,10 @@ def main():
             # between them, under a graph
             mod = decode_loop.measure(32, 512, 64, fused=False, model=model)
             decode["module_path"] = {k: mod[k] for k in ("new_tokens", "graph", "module_glue", "decode_tok_per_s", "ms_per_token")}
+            module_eager = module_eager_leg(torch, model)
             del model
 
-    traffic, traffic_source = read_traffic_sidecar()
+    traffic, traffic_source = read_traffic_sidecar(dom_launch["kernel"])
     result = {
         "metric": "W4A16+GlowQ decode linears, microseconds per layer (Llama-3.1-8B shape, batch 1)",
         "value": round(us_per_layer, 3),
@@ -583,10 +680,12 @@ def main():
         "prefill": prefill,
         "selective": selective,
         "decode_loop": decode,
+        "module_forward_eager_us": module_eager,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_stream_kernel (gate|up group launch, N=28672, K=4096, M=1, rank 128, r given)",
+            "kernel": f"{dom_launch['kernel']} (gate|up group launch, N=28672, K=4096, M=1, rank 128, r given; grid "
+                      f"{dom_launch['grid'][0]} x {dom_launch['block']} threads)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -595,6 +694,11 @@ def main():
             "algorithmic_bytes_per_launch": dom_bytes,
             # the same group with its projection launch: all of the group's bytes over the time of both launches
             "frac_with_projection_launch": round(per_group[DOMINANT]["pct_hbm_peak"] / 100, 4),
+            # a kernel of the same grid that only reads the launch's algorithmic bytes (glowq_probe_stream_read), and one
+            # that does nothing (back-to-back launches in a graph): what the memory system and the launch path leave
+            "stream_read_GBps": stream_read,
+            "frac_of_stream_read": round(achieved / stream_read, 4) if stream_read else None,
+            "empty_launch_us": round(empty_us, 3),
             # HBM bytes per launch counted by rocprofv3 (FETCH_SIZE + WRITE_SIZE scaled on a copy of known size) in an
             # earlier profiling run of this script: read from the file named next to it, null without that file
             "traffic": traffic,

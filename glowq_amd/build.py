@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libglowq_w4a16.so")
-SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_chain.hip", "gemv_quad.hip", "gemv_qstream.hip", "skinny.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
+SOURCES = ["abi.hip", "gemv.hip", "gemv_stream.hip", "gemv_chain.hip", "gemv_quad.hip", "gemv_qstream.hip", "skinny.hip", "skinny_tiled.hip", "gemm.hip", "misc.hip", "decode_glue.hip"]
 ARCH = "gfx950"
 
 HIPCC_FLAGS = [

@@ -1,5 +1,6 @@
 // C ABI of the library: argument validation, route selection, launches.  No torch types, no
 // allocation, no synchronisation; see include/glowq_w4a16.h for the contract of each entry point.
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
@@ -8,6 +9,7 @@
 
 #include "common.hpp"
 #include "side_stream.hpp"
+#include "tiled.hpp"
 
 namespace glowq {
 // gemv.hip
@@ -39,6 +41,16 @@ bool skinny_raw_form(const GroupDev& g);
 hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw);
 bool gemm_supported(const GroupDev& g);
 hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream);
+// misc.hip
+hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, int grid, int block, hipStream_t stream);
+hipError_t launch_probe_empty(int grid, int block, hipStream_t stream);
+size_t skinny_split_workspace_bytes(int M, int num_cus);  // skinny.hip
+// skinny_tiled.hip
+size_t tiled_split_workspace_bytes(int M, int num_cus);
+bool skinny_tiled_supported(const GroupDev& g);
+hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream);
+hipError_t launch_pack_tiled(const int32_t*, const half_t*, const int32_t*, void*, int, int, int, int, int, int, int, hipStream_t);
+hipError_t launch_pack_tiled_left(const half_t*, void*, int, int, int, hipStream_t);
 hipError_t launch_shared_proj_mfma(const half_t*, const half_t*, half_t*, int, int, int, int, hipStream_t, void* ws,
                                    size_t ws_bytes);
 size_t proj_workspace_bytes(int M, int K, int rank, int num_cus);
@@ -75,7 +87,25 @@ void* static_scratch(bool lookup_allowed = true) {
 
 }  // namespace
 
+namespace {
+struct LaunchNote {
+  char kernel[160];
+  int grid_x, grid_y, block;
+};
+thread_local LaunchNote g_note = {};
+}  // namespace
+
 namespace glowq {
+void note_launch(int grid_x, int grid_y, int block, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_note.kernel, sizeof(g_note.kernel), fmt, ap);
+  va_end(ap);
+  g_note.grid_x = grid_x;
+  g_note.grid_y = grid_y;
+  g_note.block = block;
+}
+
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -108,7 +138,8 @@ int num_cus() {
 
 namespace {
 
-constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4, kRouteStream = 5, kRouteQStream = 6, kRouteSkinnyRaw = 7;
+constexpr int kRouteWaveDot = 0, kRouteSkinny = 1, kRouteGemm = 2, kRouteGeneric = 3, kRouteQuad = 4, kRouteStream = 5, kRouteQStream = 6, kRouteSkinnyRaw = 7,
+              kRouteSkinnyTiled = 8;
 constexpr int kWaveDotMaxM = 4;  // row capacity of the wave-dot kernel
 
 // Route limits, settable at run time (glowq_set_tuning) and initialised from the environment:
@@ -196,6 +227,9 @@ void to_dev(const glowq_member_t& s, MemberDev& d) {
   d.y = static_cast<half_t*>(s.y);
   d.side = aligned16(s.side) ? static_cast<const unsigned char*>(s.side) : nullptr;
   d.side_rank = s.side_rank;
+  d.tiled = s.tiled;
+  d.tiled_L = s.tiled_L;
+  d.tiled_rank = s.tiled_rank;
   d.N = s.N;
   d.ldw = s.ldw_i32;
   d.lds = s.lds;
@@ -261,7 +295,30 @@ std::atomic<int> g_skinny_codes_max_m{clampi(env_or("GLOWQ_SKINNY_CODES_M", 8), 
 
 int pick_route_rounded(const GroupDev& g, int force);
 
+//   tiled_min_m / tiled_max_m  token rows served by the matrix-core kernel that reads the tiled copy of the weights, where
+//                   every member of the group brings one (GLOWQ_TILED_MIN_M, GLOWQ_TILED_MAX_M; max 0 switches it off)
+std::atomic<int> g_tiled_min_m{clampi(env_or("GLOWQ_TILED_MIN_M", 5), 1, 64)};
+std::atomic<int> g_tiled_max_m{clampi(env_or("GLOWQ_TILED_MAX_M", 64), 0, 64)};
+//   tiled_shape_rule  1: up to 32 rows only groups whose stream is long enough to pay for the kernel's start-up take the
+//                   tiled route, the others stay on the skinny kernel (GLOWQ_TILED_SHAPE_RULE; 0: every group that can).
+//                   Group launch with the projection in front, us, tiled / skinny.  8B shapes: q|k|v (13 MB of codes) 8 rows
+//                   14.9 / 11.3, 32 rows 17.8 / 15.2, 64 rows 24.6 / 24.5; o_proj (8 MB) 13.8 / 10.7, 16.4 / 14.8, 22.6 /
+//                   23.9; gate|up (59 MB) 22.4 / 24.1, 26.3 / 31.1, 37.4 / 56.0; down_proj (29 MB) 21.3 / 19.5, 16 rows
+//                   22.3 / 21.5, 32 rows 25.5 / 28.2, 64 rows 32.2 / 41.2.  14B shapes: gate|up (89 MB) 33.2 / 40.8,
+//                   41.7 / 52.3, 62.7 / 93.9; down_proj (45 MB) 27.7 / 28.5, 32.0 / 40.2, 42.6 / 63.0.
+std::atomic<int> g_tiled_shape_rule{clampi(env_or("GLOWQ_TILED_SHAPE_RULE", 1), 0, 1)};
+bool tiled_pays(const GroupDev& g) {
+  if (g.M > 32 || g_tiled_shape_rule.load(std::memory_order_relaxed) == 0) return true;
+  long rows = 0;
+  for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
+  const long code_bytes = rows * (long)g.K / 2;
+  return code_bytes >= 40L * 1000 * 1000 || (g.M > 16 && code_bytes >= 24L * 1000 * 1000);
+}
+
 int pick_route(const GroupDev& g, int force) {
+  if (force < 0 && g.M >= g_tiled_min_m.load(std::memory_order_relaxed) && g.M <= g_tiled_max_m.load(std::memory_order_relaxed) &&
+      skinny_tiled_supported(g) && tiled_pays(g))
+    return kRouteSkinnyTiled;
   const int route = pick_route_rounded(g, force);
   if (route == kRouteSkinny && force < 0 && g.M <= g_skinny_codes_max_m.load(std::memory_order_relaxed) && skinny_raw_form(g)) return kRouteSkinnyRaw;
   return route;
@@ -319,12 +376,17 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr && g.mem[i].side_rank == (g.r ? g.rank : 0);
   if (!packed)
     for (int i = 0; i < g.n_members; ++i) g.mem[i].side = nullptr;
+  static const char* const kRouteNames[] = {"wave_dot_gemv", "skinny_mfma", "tiled_mfma_gemm", "generic", "quad_mfma_gemv",
+                                            "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma", "skinny_tiled_mfma"};
+  note_launch(0, 0, 0, "%s", (route >= 0 && route <= kRouteSkinnyTiled) ? kRouteNames[route] : "?");  // launchers that know more overwrite it
   if (route == kRouteStream) {
     e = launch_stream(g, cus, stream);
   } else if (route == kRouteQStream) {
     e = launch_qstream(g, cus, stream);
   } else if (route == kRouteGemm) {
     e = launch_gemm(g, cus, stream);
+  } else if (route == kRouteSkinnyTiled) {
+    e = launch_skinny_tiled(g, cus, stream);
   } else if (route == kRouteSkinny || route == kRouteSkinnyRaw) {
     e = launch_skinny(g, cus, stream, route == kRouteSkinnyRaw);
   } else {
@@ -498,6 +560,35 @@ int glowq_pack_side(const void* scales, const int32_t* qzeros, const void* L, vo
   return GLOWQ_OK;
 }
 
+size_t glowq_tiled_bytes(int N, int K, int group_size) {
+  return (N > 0 && tiled::applies(K, group_size)) ? tiled::weight_bytes(N, K) : 0;
+}
+
+int glowq_pack_tiled(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out, int N, int K, int group_size,
+                     int ldw_i32, int lds, int ldz_i32, void* stream) {
+  if (!qweight || !scales || !qzeros || !out) return fail(GLOWQ_EINVAL, "pack_tiled: NULL pointer");
+  if (glowq_tiled_bytes(N, K, group_size) == 0)
+    return fail(GLOWQ_EUNSUPPORTED, "pack_tiled: no tiled layout for N=%d K=%d group_size=%d", N, K, group_size);
+  const int groups = K / group_size;
+  if (ldw_i32 < K / 8 || lds < groups || ldz_i32 < (groups + 7) / 8) return fail(GLOWQ_ESHAPE, "pack_tiled: qweight / scales / qzeros rows too short");
+  if (!aligned16(out)) return fail(GLOWQ_EINVAL, "pack_tiled: the output must be 16-byte aligned");
+  hipError_t e = launch_pack_tiled(qweight, static_cast<const half_t*>(scales), qzeros, out, N, K, group_size, ldw_i32, lds, ldz_i32,
+                                   num_cus(), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "pack_tiled launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+size_t glowq_tiled_left_bytes(int N, int rank) { return (N > 0 && rank >= 8 && (rank & 7) == 0) ? tiled::left_bytes(N, rank) : 0; }
+
+int glowq_pack_tiled_left(const void* L, void* out, int N, int rank, void* stream) {
+  if (!L || !out) return fail(GLOWQ_EINVAL, "pack_tiled_left: NULL pointer");
+  if (glowq_tiled_left_bytes(N, rank) == 0) return fail(GLOWQ_EUNSUPPORTED, "pack_tiled_left: no tiled layout for N=%d rank=%d", N, rank);
+  if (!aligned16(out)) return fail(GLOWQ_EINVAL, "pack_tiled_left: the output must be 16-byte aligned");
+  hipError_t e = launch_pack_tiled_left(static_cast<const half_t*>(L), out, N, rank, num_cus(), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "pack_tiled_left launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
 int glowq_unpack_int4(const int32_t* packed, uint8_t* codes, int rows, int total_vals, int ld_i32, void* stream) {
   if (!packed || !codes) return fail(GLOWQ_EINVAL, "unpack: NULL pointer");
   if (rows <= 0 || total_vals <= 0) return fail(GLOWQ_EINVAL, "unpack: rows and total_vals must be > 0");
@@ -634,11 +725,13 @@ int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r
   if (M > GLOWQ_STATIC_MAX_ROWS)
     return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: %d token rows, the static scratch serves at most %d", M,
                 GLOWQ_STATIC_MAX_ROWS);
-  // what the two users of the workspace ask for at this shape: the projection's split of K, and the skinny kernel's
-  // (at most one 32-column fp32 tile per token row for each of num_cus workgroup slots)
+  // what the users of the workspace ask for at this shape: the projection's split of K, the skinny kernel's and that of
+  // the kernel that streams the tiled copy (each states its own bound next to its split rule)
   size_t need = (M > 0 && K > 0 && rank > 0) ? proj_workspace_bytes(M, K, rank, num_cus()) : 0;
-  const size_t skinny_need = M > 4 ? (size_t)num_cus() * (size_t)M * 32 * sizeof(float) : 0;
-  if (skinny_need > need) need = skinny_need;
+  need = std::max(need, glowq::skinny_split_workspace_bytes(M, num_cus()));
+  bool any_tiled = false;
+  for (int i = 0; members != nullptr && i < n_members && i < GLOWQ_MAX_MEMBERS; ++i) any_tiled = any_tiled || members[i].tiled != nullptr;
+  if (any_tiled) need = std::max(need, glowq::tiled_split_workspace_bytes(M, num_cus()));
   if (need > kStaticScratchBytes)
     return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: this shape wants %zu bytes of scratch, the static buffer holds %zu",
                 need, kStaticScratchBytes);
@@ -662,7 +755,7 @@ int glowq_static_scratch_prepare(void) {
   return GLOWQ_OK;
 }
 
-int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
+static int route_query(int M, int K, int N, int group_size, int ldw_i32, bool with_tiled) {
   GroupDev g;
   memset(&g, 0, sizeof(g));
   g.n_members = 1;
@@ -671,9 +764,37 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) {
   g.group_size = group_size;
   g.mem[0].N = N;
   g.mem[0].ldw = ldw_i32;
+  if (with_tiled && tiled::applies(K, group_size)) g.mem[0].tiled = reinterpret_cast<const void*>(uintptr_t{16});  // never read
   return pick_route(g, -1);
 }
 
+int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32) { return route_query(M, K, N, group_size, ldw_i32, false); }
+
+int glowq_w4a16_route_tiled(int M, int K, int N, int group_size, int ldw_i32) { return route_query(M, K, N, group_size, ldw_i32, true); }
+
+
+int glowq_last_launch(char* kernel, size_t bytes, int* grid_x, int* grid_y, int* block) {
+  if (kernel != nullptr && bytes > 0) snprintf(kernel, bytes, "%s", g_note.kernel);
+  if (grid_x) *grid_x = g_note.grid_x;
+  if (grid_y) *grid_y = g_note.grid_y;
+  if (block) *block = g_note.block;
+  return GLOWQ_OK;
+}
+
+int glowq_probe_stream_read(const void* src, size_t bytes, void* sink, int grid, int block, void* stream) {
+  if (!src || !sink || grid <= 0 || block <= 0 || block > 1024 || (block & 63) != 0 || !aligned16(src) || (bytes & 15) != 0)
+    return fail(GLOWQ_EINVAL, "probe_stream_read: 16-byte aligned source, whole 16-byte units, a grid and a workgroup of whole waves");
+  hipError_t e = launch_probe_read(src, bytes, sink, grid, block, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "probe_stream_read launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
+
+int glowq_probe_empty_launch(int grid, int block, void* stream) {
+  if (grid <= 0 || block <= 0 || block > 1024) return fail(GLOWQ_EINVAL, "probe_empty_launch: a grid and a workgroup size");
+  hipError_t e = launch_probe_empty(grid, block, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "probe_empty_launch launch failed: %s", hipGetErrorString(e));
+  return GLOWQ_OK;
+}
 
 int glowq_set_tuning(const char* key, int value) {
   if (key == nullptr) return fail(GLOWQ_EINVAL, "tuning key must not be NULL");
@@ -689,6 +810,9 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "qstream_shape_rule") == 0) { slot = &g_qstream_shape_rule; hi = 1; }
   else if (strcmp(key, "skinny_codes_max_m") == 0) { slot = &g_skinny_codes_max_m; hi = 64; }
   else if (strcmp(key, "stream_shape_rule") == 0) { slot = &g_stream_shape_rule; hi = 1; }
+  else if (strcmp(key, "tiled_min_m") == 0) { slot = &g_tiled_min_m; lo = 1; hi = 64; }
+  else if (strcmp(key, "tiled_max_m") == 0) { slot = &g_tiled_max_m; hi = 64; }
+  else if (strcmp(key, "tiled_shape_rule") == 0) { slot = &g_tiled_shape_rule; hi = 1; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

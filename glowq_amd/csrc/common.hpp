@@ -31,6 +31,9 @@ struct MemberDev {
   half_t* y;
   const unsigned char* side;  // the member's side stream (side_stream.hpp) or nullptr
   int side_rank;              // the rank it was packed for
+  const void* tiled;          // the member's tiled weights (tiled.hpp) or nullptr
+  const void* tiled_L;        // its tiled left factor or nullptr
+  int tiled_rank;             // the rank tiled_L was packed for
   int N, ldw, lds, ldz, ldy;
 };
 
@@ -74,6 +77,9 @@ struct ChainDev {
 int fail(int code, const char* fmt, ...);
 // Compute units of the current device (cached).
 int num_cus();
+// Leaves the kernel a group launch used in the calling thread's launch record (glowq_last_launch): its name with the
+// template arguments of the instantiation, grid and workgroup size.
+void note_launch(int grid_x, int grid_y, int block, const char* fmt, ...);
 
 // Raises a kernel's dynamic LDS limit to `bytes` on the current device when that is above the 48 KB default and above
 // what this call site asked for before.  `raised` is the call site's own table (one slot per device); host threads may

@@ -52,6 +52,8 @@ hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), lds, stream, g.x, g.r, g.K, g.r ? g.rank : 0, g.group_size,
                        g.alpha, g, ChainDev{});
+    note_launch(grid, 1, waves * kWave, "gemv_stream_kernel<%d,%d,%d,%d,%d,%d,%d,%d>", kKit, kLW, kM, (int)kPacked, kProPlain, kEpiNone,
+                stream_xw(kKit), 0);
     return hipGetLastError();
   }
 }

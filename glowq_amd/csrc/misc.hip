@@ -229,4 +229,41 @@ hipError_t launch_shared_proj_small(const half_t* x, const half_t* R, half_t* r,
   return hipGetLastError();
 }
 
+// ---- measurement probes ---------------------------------------------------------------------------------------------
+// A bare streaming read: workgroup b takes the b-th contiguous share of the buffer, every lane 16 bytes per load, eight
+// loads in flight per lane, and nothing is done with the data but an xor (the store never happens: the sum of eight
+// words is compared with a value no buffer of a benchmark holds by design of the check below).  What a memory-bound
+// kernel of the same grid could reach if it did no arithmetic at all.
+__global__ __launch_bounds__(1024) void probe_read_kernel(const u32x4* __restrict__ src, size_t units, uint32_t* __restrict__ sink) {
+  const size_t per = (units + gridDim.x - 1) / gridDim.x;
+  const size_t begin = (size_t)blockIdx.x * per;
+  const size_t end = begin + per < units ? begin + per : units;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  for (size_t i = begin + threadIdx.x; i < end; i += 8 * (size_t)blockDim.x) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const size_t at = i + (size_t)u * blockDim.x;
+      v[u] = at < end ? __builtin_nontemporal_load(src + at) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  const uint32_t f = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  if (f == 0x9E3779B9u && (acc.x & acc.y) == 0xDEADBEEFu) sink[0] = f;  // keeps the loads alive
+}
+
+__global__ void probe_empty_kernel() {}
+
+hipError_t launch_probe_read(const void* src, size_t bytes, void* sink, int grid, int block, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(block), 0, stream, static_cast<const u32x4*>(src), bytes / 16,
+                     static_cast<uint32_t*>(sink));
+  return hipGetLastError();
+}
+
+hipError_t launch_probe_empty(int grid, int block, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(block), 0, stream);
+  return hipGetLastError();
+}
+
 }  // namespace glowq

@@ -778,6 +778,11 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
   return hipGetLastError();
 }
 
+// The most workspace the split of K above asks for: it cuts only while slices x column tiles stay within num_cus
+// workgroups, and a split launch has 32-column tiles (the 64-column ones belong to groups that fill the chip without it):
+// one 32-column fp32 tile per token row for each of num_cus workgroups.
+size_t skinny_split_workspace_bytes(int M, int num_cus) { return M > 4 ? (size_t)num_cus * (size_t)M * 32 * sizeof(float) : 0; }
+
 hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw) {
   SkinnyArgs a;
   a.x = g.x;

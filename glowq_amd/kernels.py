@@ -36,7 +36,7 @@ class _Member(ctypes.Structure):
         ("qweight", _P), ("scales", _P), ("qzeros", _P), ("L", _P), ("bias", _P), ("y", _P),
         ("N", ctypes.c_int32), ("ldw_i32", ctypes.c_int32), ("lds", ctypes.c_int32),
         ("ldz_i32", ctypes.c_int32), ("ldy", ctypes.c_int32), ("side_rank", ctypes.c_int32),
-        ("side", _P),
+        ("side", _P), ("tiled", _P), ("tiled_L", _P), ("tiled_rank", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -76,6 +76,15 @@ _SIGNATURES = {
     "glowq_w4a16_group_forward_chained": (_I, [_P, _P, ctypes.POINTER(_Member), _I, _I, _I, _I, ctypes.c_float,
                                                ctypes.POINTER(_Chain), _P]),
     "glowq_w4a16_route": (_I, [_I, _I, _I, _I, _I]),
+    "glowq_w4a16_route_tiled": (_I, [_I, _I, _I, _I, _I]),
+    "glowq_last_launch": (_I, [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                ctypes.POINTER(ctypes.c_int)]),
+    "glowq_probe_stream_read": (_I, [_P, ctypes.c_size_t, _P, _I, _I, _P]),
+    "glowq_probe_empty_launch": (_I, [_I, _I, _P]),
+    "glowq_tiled_bytes": (ctypes.c_size_t, [_I, _I, _I]),
+    "glowq_pack_tiled": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "glowq_tiled_left_bytes": (ctypes.c_size_t, [_I, _I]),
+    "glowq_pack_tiled_left": (_I, [_P, _P, _I, _I, _P]),
     "glowq_set_tuning": (_I, [ctypes.c_char_p, _I]),
     "glowq_add_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, ctypes.c_float, _P]),
     "glowq_silu_mul": (_I, [_P, _P, _P, ctypes.c_long, _P]),
@@ -86,6 +95,15 @@ _SIGNATURES = {
     "glowq_attend_combine_proj": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "glowq_argmax_advance": (_I, [_P, _I, _P, _P, _P, _P]),
 }
+
+
+# Calls with this many token rows and more bring the tiled copy of the weights along when they build descriptors per call.
+TILED_MIN_ROWS = 5
+
+
+def tiled_enabled() -> bool:
+    """GLOWQ_TILED=0 keeps every route on the canonical buffers (no second copy of the weights in device memory)."""
+    return os.environ.get("GLOWQ_TILED", "1").lower() not in {"0", "false", "no", "off"}
 
 
 def _check(cond: bool, msg: str) -> None:
@@ -238,6 +256,74 @@ class W4A16Extension:
             self._raise(rc, "pack_side")
         return out
 
+    def pack_tiled(self, qweight, scales, qzeros, in_features: int, group_size: int) -> Optional[torch.Tensor]:
+        """The tiled copy of a member's weights for the matrix-core routes (a uint8 tensor; layout in csrc/tiled.hpp), or
+        None where the layout does not apply.  Built once per weight tensor and kept on it (`qweight._glowq_tiled`) until
+        the tensor is written to in place; a module moved with `.to()` gets new tensors and with them a new copy."""
+        if not tiled_enabled():
+            return None
+        N = qweight.size(0)
+        nbytes = self.lib.glowq_tiled_bytes(N, int(in_features), int(group_size))
+        if nbytes == 0 or not qweight.is_cuda:
+            return None
+        key = (qweight._version, scales.data_ptr(), scales._version, qzeros.data_ptr(), qzeros._version, int(in_features), int(group_size))
+        hit = getattr(qweight, "_glowq_tiled", None)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        if torch.cuda.is_current_stream_capturing():
+            return None  # not under a graph capture: the copy would come from the graph's own memory pool
+        _check(qweight.dtype == torch.int32 and scales.dtype == torch.float16 and qzeros.dtype == torch.int32 and
+               qweight.is_contiguous() and scales.is_contiguous() and qzeros.is_contiguous(), "pack_tiled: contiguous canonical buffers")
+        out = torch.empty(nbytes, dtype=torch.uint8, device=qweight.device)
+        with torch.cuda.device(qweight.device):
+            rc = self.lib.glowq_pack_tiled(qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(), out.data_ptr(), N, int(in_features),
+                                           int(group_size), qweight.size(1), scales.size(1), qzeros.size(1), self._stream(qweight.device))
+        if rc:
+            self._raise(rc, "pack_tiled")
+        qweight._glowq_tiled = (key, out)
+        return out
+
+    def pack_tiled_left(self, L) -> Optional[torch.Tensor]:
+        """The tiled copy of a left factor [N, rank] (fp16 B operand of the correction blocks), kept on the tensor."""
+        if not tiled_enabled() or L is None or not L.is_cuda:
+            return None
+        N, rank = L.shape
+        nbytes = self.lib.glowq_tiled_left_bytes(int(N), int(rank))
+        if nbytes == 0:
+            return None
+        hit = getattr(L, "_glowq_tiled", None)
+        if hit is not None and hit[0] == L._version:
+            return hit[1]
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        _check(L.dtype == torch.float16 and L.is_contiguous(), "pack_tiled_left: contiguous fp16 [OC, rank]")
+        out = torch.empty(nbytes, dtype=torch.uint8, device=L.device)
+        with torch.cuda.device(L.device):
+            rc = self.lib.glowq_pack_tiled_left(L.data_ptr(), out.data_ptr(), int(N), int(rank), self._stream(L.device))
+        if rc:
+            self._raise(rc, "pack_tiled_left")
+        L._glowq_tiled = (L._version, out)
+        return out
+
+    def wants_tiled(self, M: int, K: int, N_total: int, group_size: int, ldw_i32: int) -> bool:
+        """Whether a group of this shape would take the route that reads the tiled copies: they are built (and kept in device
+        memory beside the canonical buffers) only for such groups."""
+        return (M >= TILED_MIN_ROWS and tiled_enabled()
+                and self.lib.glowq_w4a16_route_tiled(int(M), int(K), int(N_total), int(group_size), int(ldw_i32)) == 8)
+
+    def _set_tiled(self, e, qw, sc, qz, L, in_features: int, group_size: int):
+        """Fills the tiled fields of descriptor `e`; returns what has to stay alive with it."""
+        tw = self.pack_tiled(qw, sc, qz, in_features, group_size)
+        if tw is None:
+            return None
+        tl = self.pack_tiled_left(L) if L is not None else None
+        if L is not None and tl is None:
+            return None
+        e.tiled = tw.data_ptr()
+        e.tiled_L = tl.data_ptr() if tl is not None else None
+        e.tiled_rank = int(L.size(1)) if L is not None else 0
+        return (tw, tl)
+
     def shared_proj(self, x, R, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """r = fp16(x @ R^T); x [M, K] fp16, R [rank, K] fp16."""
         _check(x.is_cuda and R.is_cuda, "shared_proj: tensors must be CUDA")
@@ -278,6 +364,8 @@ class W4A16Extension:
             _check(r.is_cuda and r.dtype == torch.float16 and r.dim() == 2 and r.size(0) == M and r.is_contiguous(),
                    "group_forward: r must be a contiguous CUDA fp16 [M, rank] tensor")
             rank = r.size(1)
+        want_tiled = self.wants_tiled(M, K, sum(int(m["qweight"].size(0)) for m in members), group_size,
+                                      int(members[0]["qweight"].size(1)))
         result = []
         for i, m in enumerate(members):
             qw, sc, qz = m["qweight"], m["scales"], m["qzeros"]
@@ -306,6 +394,8 @@ class W4A16Extension:
             e.bias = bias.data_ptr() if bias is not None else None
             e.y = y.data_ptr()
             e.N, e.ldw_i32, e.lds, e.ldz_i32, e.ldy = N, qw.size(1), sc.size(1), qz.size(1), y.stride(0)
+            if want_tiled:
+                keep.append(self._set_tiled(e, qw, sc, qz, L, K, group_size))
             result.append(y)
         if M == 0:
             return result
@@ -455,10 +545,19 @@ class W4A16Extension:
         if rc:
             self._raise(rc, "argmax_advance")
 
-    def route(self, M: int, K: int, N: int, group_size: int = 128) -> str:
+    def last_launch(self) -> dict:
+        """The kernel the calling thread's last group launch used (name with template arguments where the launcher records
+        them, else the route's name), its grid and its workgroup size."""
+        buf = ctypes.create_string_buffer(160)
+        gx, gy, blk = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        self.lib.glowq_last_launch(buf, 160, ctypes.byref(gx), ctypes.byref(gy), ctypes.byref(blk))
+        return {"kernel": buf.value.decode(), "grid": [gx.value, gy.value], "block": blk.value}
+
+    def route(self, M: int, K: int, N: int, group_size: int = 128, tiled: Optional[bool] = None) -> str:
         names = {0: "wave_dot_gemv", 1: "skinny_mfma", 2: "tiled_mfma_gemm", 3: "generic", 4: "quad_mfma_gemv", 5: "stream_gemv",
-                 6: "quad_stream_gemv", 7: "skinny_codes_mfma"}
-        return names[self.lib.glowq_w4a16_route(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
+                 6: "quad_stream_gemv", 7: "skinny_codes_mfma", 8: "skinny_tiled_mfma"}
+        fn = self.lib.glowq_w4a16_route_tiled if (tiled_enabled() if tiled is None else tiled) else self.lib.glowq_w4a16_route
+        return names[fn(int(M), int(K), int(N), int(group_size), (int(K) + 7) // 8)]
 
     def set_tuning(self, key: str, value: int) -> int:
         """Sets a route limit of the process ("quad_max_m", "quad_min_m", "wave_dot_max_m", "skinny_max_m",
@@ -538,6 +637,7 @@ class PreparedGroup:
             self.Ns.append(N)
             self.keep.append((qw, sc, qz, L, bias, side))
         self.corrected = corrected
+        self._tiled_keep = None  # the tiled copies of the members' weights: built by the first call with five token rows or more
 
     def run(self, x: torch.Tensor, r: Optional[torch.Tensor] = None, outs: Optional[List[torch.Tensor]] = None,
             project: bool = True) -> List[torch.Tensor]:
@@ -547,6 +647,9 @@ class PreparedGroup:
         _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2 and x.size(1) == self.K and x.is_contiguous(),
                "inputs must be contiguous CUDA fp16 [M, IC]")
         M = x.size(0)
+        if self._tiled_keep is None and self.ext.wants_tiled(M, self.K, sum(self.Ns), self.group_size, self.arr[0].ldw_i32):
+            self._tiled_keep = [self.ext._set_tiled(e, k[0], k[1], k[2], k[3] if self.corrected else None, self.K, self.group_size)
+                                for e, k in zip(self.arr, self.keep)]
         if outs is None:
             outs = [torch.empty((M, N), dtype=torch.float16, device=x.device) for N in self.Ns]
         for e, y, N in zip(self.arr, outs, self.Ns):

@@ -52,6 +52,10 @@ typedef struct glowq_member {
   int32_t ldy;
   int32_t side_rank;      /* the rank `side` was packed for (0: packed without a left factor) */
   const void* side;       /* the member's side stream written by glowq_pack_side for this K and group_size, or NULL */
+  const void* tiled;      /* the member's tiled weights written by glowq_pack_tiled for this K and group_size, or NULL */
+  const void* tiled_L;    /* its tiled left factor written by glowq_pack_tiled_left for tiled_rank, or NULL */
+  int32_t tiled_rank;
+  int32_t reserved;
 } glowq_member_t;
 
 /* Library / device information. */
@@ -175,6 +179,24 @@ int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out
                                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Tiled copy of a member's weights for the matrix-core routes (5..64 token rows): the codes of 32 output rows and 256
+ * input columns at a time in the order in which one coalesced 16-byte-per-lane load hands every lane the B operand of
+ * the 32x32x16 matrix instruction, with each lane's scale and -(1024 + zero-point) behind them (4352 bytes per
+ * (row block, super-block); layout in glowq_amd/csrc/tiled.hpp).  A deterministic function of the canonical buffers,
+ * which stay the state-dict form and what every other route reads; the reference has no counterpart (its large-M
+ * route writes a dequantised fp16 copy of the whole weight on every call, src/cuda_w4a16/csrc/gemm_w4a16.cu:106-129).
+ * glowq_tiled_bytes / glowq_tiled_left_bytes give the sizes (16-byte aligned device memory), 0 where the layout does not
+ * apply (it needs K % 256 == 0 and power-of-two groups of 128 columns and more; ranks that are multiples of 8).
+ * A member whose `tiled` is set must have been packed for the K and group_size of the call; `tiled_L` for its L and
+ * `tiled_rank`.  Calls use them when every member of the group brings them, and ignore them otherwise.
+ */
+size_t glowq_tiled_bytes(int N, int K, int group_size);
+int glowq_pack_tiled(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* tiled, int N, int K,
+                     int group_size, int ldw_i32, int lds, int ldz_i32, void* stream);
+size_t glowq_tiled_left_bytes(int N, int rank);
+int glowq_pack_tiled_left(const void* L, void* tiled_L, int N, int rank, void* stream);
+
+/*
  * glowq_w4a16_group_forward_fused_ws for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * glowq_w4a16_group_forward_fused_ws called with a workspace of glowq_static_scratch_bytes() bytes, but the workspace
@@ -204,6 +226,24 @@ int glowq_static_scratch_prepare(void);
  * eight token rows).
  */
 int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
+/* The same for a member that brings the tiled copy of its weights (glowq_pack_tiled): 8 = the matrix-core kernel that
+ * streams the tiled copy: 33..64 token rows, and 5..32 where the group's codes are 40 MB and more (24 MB from 17 rows);
+ * "tiled_min_m" / "tiled_max_m" / "tiled_shape_rule" of glowq_set_tuning. */
+int glowq_w4a16_route_tiled(int M, int K, int N, int group_size, int ldw_i32);
+
+/*
+ * Measurement helpers of bench.py; no counterpart in the reference.
+ * glowq_last_launch: what the calling thread's last group launch used -- the kernel with the template arguments of the
+ *   instantiation where the launcher records them (the stream GEMV, the tiled-copy kernel), else the route's name --
+ *   and its grid and workgroup size (0 where not recorded).
+ * glowq_probe_stream_read: a kernel that does nothing but read `bytes` (16-byte loads, eight in flight per lane,
+ *   workgroup b the b-th contiguous share) with the given grid and workgroup size: the rate a memory-bound kernel of
+ *   that launch shape could reach with no arithmetic at all.  `sink` (4 bytes of device memory) is never written.
+ * glowq_probe_empty_launch: a kernel of that launch shape that returns at once (back-to-back launch cost).
+ */
+int glowq_last_launch(char* kernel, size_t bytes, int* grid_x, int* grid_y, int* block);
+int glowq_probe_stream_read(const void* src, size_t bytes, void* sink, int grid, int block, void* stream);
+int glowq_probe_empty_launch(int grid, int block, void* stream);
 
 /*
  * Route limits of the process (the reference's counterpart is the W4A16_GEMV_M_MAX family of environment
@@ -222,9 +262,13 @@ int glowq_w4a16_route(int M, int K, int N, int group_size, int ldw_i32);
  * was measured faster on (1, the default) or for every shape it can take (0).
  * "skinny_codes_max_m" (0..64, default 8): token rows up to which the skinny MFMA kernel runs in its raw-code form
  * (route 7) where that applies; above it is slower than dequantising first (the work on the sums grows with the rows).
+ * "tiled_min_m" / "tiled_max_m" (default 5 / 64; max 0 switches the route off): token rows served by the kernel that
+ * streams the tiled copy of the weights where every member brings one; "tiled_shape_rule" (0 / 1): up to 32 rows only
+ * for groups whose stream is long enough to pay for its start-up (1, the default) or for every group (0).
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
  * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M, GLOWQ_STREAM_SHAPE_RULE,
- * GLOWQ_QSTREAM_M, GLOWQ_QSTREAM_SHAPE_RULE and GLOWQ_SKINNY_CODES_M.
+ * GLOWQ_QSTREAM_M, GLOWQ_QSTREAM_SHAPE_RULE, GLOWQ_SKINNY_CODES_M, GLOWQ_TILED_MIN_M, GLOWQ_TILED_MAX_M and
+ * GLOWQ_TILED_SHAPE_RULE.
  */
 int glowq_set_tuning(const char* key, int value);
 

@@ -1,4 +1,6 @@
 """Seeded synthetic inputs for the parity tests and the tolerance they are judged with."""
+import contextlib
+
 import numpy as np
 import torch
 
@@ -54,3 +56,14 @@ def assert_close(got, want64, what=""):
     worst = np.unravel_index(np.argmax(err - bound), err.shape)
     assert np.all(err <= bound), f"{what}: max err {err.max():.3e} at {worst} (got {got[worst]}, want {want64[worst]})"
     return float(err.max())
+
+
+@contextlib.contextmanager
+def tuning(ext, **limits):
+    """Route limits of the library set for the body of a `with` and put back afterwards."""
+    old = {key: ext.set_tuning(key, value) for key, value in limits.items()}
+    try:
+        yield
+    finally:
+        for key, value in old.items():
+            ext.set_tuning(key, value)

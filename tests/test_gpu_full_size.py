@@ -6,8 +6,9 @@ the full-size launch on the same buffers, and size-independent properties cover 
 dequantised columns exactly, a group launch equals its members launched alone bit for bit, token rows of a batched
 launch equal single-row launches within tolerance, and the result is additive in x within tolerance.
 
-Yardstick by kernel route: the GEMV routes keep the dequantised weight unrounded (`corrected_linear_exact`), the MFMA
-routes round it to fp16 once like the reference's dequantise-then-matmul (`corrected_linear_rounded_exact`); tolerance
+Yardstick by kernel route: the GEMV routes and the kernels that feed the codes to the matrix cores as they are keep the
+dequantised weight unrounded (`corrected_linear_exact`), the dequantising MFMA routes round it to fp16 once like the
+reference's dequantise-then-matmul (`corrected_linear_rounded_exact`); tolerance
 |a - b| <= 1e-2 + 1e-3 |b| in both cases."""
 import numpy as np
 import pytest
@@ -29,7 +30,7 @@ MODELS = {
                       "down": (17408, [5120])}),
 }
 GROUPS = ["qkv", "o", "gate_up", "down"]
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma", "skinny_tiled_mfma"}
 
 
 def _layer(model, name, M, seed, bias=False):

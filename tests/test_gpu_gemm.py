@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import glowq_oracle as oracle
-from helpers import assert_close, dev, make_group
+from helpers import assert_close, dev, make_group, tuning
 
 pytestmark = pytest.mark.gpu
 
@@ -84,8 +84,9 @@ def test_skinny_route_matches_oracle(ext, small_m_route, M, K, N, gs):
     if small_m_route not in ("stream", "qstream"):  # those modes leave the limits of the other kernels at their defaults
         assert ext.lib.glowq_w4a16_route(M, K, N, gs, K // 8) in ((4,) if small_m_route == "quad" and M <= 16 else (1, 7))
     x, (m,), _ = make_group(41 + M + N, M, K, [N], 0, group_size=gs)
-    y = ext.w4a16_gemv_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs)
-    torch.cuda.synchronize()
+    with tuning(ext, tiled_max_m=0):  # (above 32 rows the kernel that streams the tiled copy would take over)
+        y = ext.w4a16_gemv_forward_cuda(dev(x), dev(m["qweight"]), dev(m["scales"]), dev(m["qzeros"]), gs)
+        torch.cuda.synchronize()
     w = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], K, gs).astype(np.float64)
     assert_close(y.cpu().numpy(), x.astype(np.float64) @ w.T, f"skinny M={M} K={K} N={N}")
 
@@ -103,6 +104,7 @@ def test_skinny_split_k_through_workspace(ext, M, K, Ns, rank):
     want = [(oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 0.5) if rank else
              oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)) + m["bias"].astype(np.float64)[None, :] for m in members]
     r = torch.empty(M, rank, dtype=torch.float16, device="cuda") if rank else None
+    old_tiled = ext.set_tuning("tiled_max_m", 0)  # (above 32 rows the kernel that streams the tiled copy would take over)
     outs = ext.group_forward(dev(x), r, mem, 128, 0.5, R=dev(R) if rank else None)
     torch.cuda.synchronize()
     for i, (w, y) in enumerate(zip(want, outs)):
@@ -116,6 +118,7 @@ def test_skinny_split_k_through_workspace(ext, M, K, Ns, rank):
         for i, (w, y) in enumerate(zip(want, outs2)):
             assert_close(y.cpu().numpy(), w, f"unsplit skinny member {i}")
     finally:
+        ext.set_tuning("tiled_max_m", old_tiled)
         ext.WORKSPACE_BYTES = saved[0]
         ext._workspaces.clear()
         ext._workspaces.update(saved[1])

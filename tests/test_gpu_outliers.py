@@ -4,9 +4,10 @@
 On such inputs the reference's two routes differ from each other by more than the tolerance (shown on the CPU in
 tests/test_oracle.py::test_two_reference_semantics_part_on_outlier_activations), so each kernel is judged against the
 semantics it implements:
-  * the stream, wave-dot and 4x4x4 GEMV keep the dequantised weight unrounded, like the reference's GEMV kernel
+  * the stream, wave-dot and 4x4x4 GEMV, the skinny kernel's raw-code form and the kernel that streams the tiled copy of
+    the weights keep the dequantised weight unrounded, like the reference's GEMV kernel
     (src/cuda_w4a16/csrc/gemv_w4a16.cu:96-112): yardstick `corrected_linear_exact`;
-  * the skinny and the tiled MFMA kernels round the dequantised weight to fp16 once, like the reference's
+  * the skinny MFMA kernel and the tiled MFMA GEMM round the dequantised weight to fp16 once, like the reference's
     dequantise-then-matmul route (src/cuda_w4a16/csrc/gemm_w4a16.cu:46-49,132): yardstick
     `corrected_linear_rounded_exact`.
 Tolerance |a - b| <= 1e-2 + 1e-3 |b| in both cases, plus the effect of rounding r = x R^T to fp16 (the path under test
@@ -20,10 +21,11 @@ from helpers import ABS_TOL, REL_TOL, dev, make_group, outlier_activations
 
 pytestmark = pytest.mark.gpu
 
-UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma"}
+UNROUNDED = {"wave_dot_gemv", "quad_mfma_gemv", "generic", "stream_gemv", "quad_stream_gemv", "skinny_codes_mfma", "skinny_tiled_mfma"}
 
 # (token rows, K, member widths, rank, route mode); the default limits send 1 row to the wave-dot GEMV, 2..4 rows to the
-# wave-dot GEMV, the 4x4x4 GEMV or the skinny kernel by group size, 5..64 to the skinny kernel, more to the tiled GEMM
+# wave-dot GEMV, the 4x4x4 GEMV or the skinny kernel by group size, 5..32 to the skinny kernel, 33..64 to the kernel that
+# streams the tiled copy of the weights, more to the tiled GEMM
 CASES = [
     (1, 4096, [512, 128], 128, "default"), (1, 14336, [128], 128, "default"), (1, 4096, [512, 128], 128, "classic"),
     (2, 4096, [4096], 128, "stream"), (3, 2048, [300], 64, "stream"), (4, 14336, [2048, 2048], 128, "stream"),

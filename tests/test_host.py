@@ -282,7 +282,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert set(kernels._SIGNATURES) == declared
-    assert ctypes.sizeof(kernels._Member) == 6 * 8 + 6 * 4 + 8  # matches glowq_member_t
+    assert ctypes.sizeof(kernels._Member) == 6 * 8 + 6 * 4 + 8 + 2 * 8 + 2 * 4  # matches glowq_member_t
     assert kernels._Member.side.offset == 72 and kernels._Member.side_rank.offset == 68
 
 
@@ -327,13 +327,27 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     ext.set_tuning("stream_shape_rule", rule)
     stream = ext.set_tuning("stream_max_m", 0)                                  # the routes behind it
     old = ext.set_tuning("quad_max_m", 0)
-    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096) == "skinny_codes_mfma"
+    assert ext.route(1, 4096, 4096) == "wave_dot_gemv" and ext.route(8, 4096, 4096, tiled=False) == "skinny_codes_mfma"
+    # a member that brings the tiled copy of its weights: 33..64 token rows go to the kernel that streams it, 5..32 where
+    # the stream is long enough (40 MB of codes and more; 24 MB from 17 rows)
+    assert ext.route(64, 4096, 4096, tiled=True) == "skinny_tiled_mfma" and ext.route(64, 14336, 4096, tiled=True) == "skinny_tiled_mfma"
+    assert ext.route(8, 4096, 28672, tiled=True) == "skinny_tiled_mfma" and ext.route(8, 4096, 4096, tiled=True) == "skinny_codes_mfma"
+    assert ext.route(16, 14336, 4096, tiled=True) == "skinny_mfma" and ext.route(17, 14336, 4096, tiled=True) == "skinny_tiled_mfma"
+    assert ext.route(4, 4096, 28672, tiled=True) != "skinny_tiled_mfma" and ext.route(65, 4096, 28672, tiled=True) == "tiled_mfma_gemm"
+    rule = ext.set_tuning("tiled_shape_rule", 0)
+    assert rule == 1 and ext.route(8, 4096, 4096, tiled=True) == "skinny_tiled_mfma" and ext.route(5, 256, 32, tiled=True) == "skinny_tiled_mfma"
+    assert ext.route(8, 4096 + 128, 4096, tiled=True) != "skinny_tiled_mfma"   # K must be whole super-blocks of 256 columns
+    assert ext.route(8, 4096, 4096, group_size=64, tiled=True) != "skinny_tiled_mfma"
+    tmax = ext.set_tuning("tiled_max_m", 0)
+    assert tmax == 64 and ext.route(8, 4096, 4096, tiled=True) == "skinny_codes_mfma"
+    ext.set_tuning("tiled_max_m", tmax)
+    ext.set_tuning("tiled_shape_rule", rule)
     ext.set_tuning("quad_max_m", 16)
-    assert ext.route(8, 4096, 4096) == "quad_mfma_gemv"
+    assert ext.route(8, 4096, 4096, tiled=False) == "quad_mfma_gemv"
     ext.set_tuning("quad_max_m", old)
     # 2..4 rows: small groups stay on the wave-dot GEMV, large ones take the 4x4x4 matrix-core GEMV
     assert ext.route(2, 4096, 4096) == "wave_dot_gemv" and ext.route(2, 4096, 28672) == "quad_mfma_gemv"
-    assert ext.route(4, 4096, 4096) == "skinny_codes_mfma" and ext.route(4, 14336, 4096) == "quad_mfma_gemv"
+    assert ext.route(4, 4096, 4096, tiled=False) == "skinny_codes_mfma" and ext.route(4, 14336, 4096) == "quad_mfma_gemv"
     old = ext.set_tuning("small_group_mb", 0)
     assert ext.route(2, 4096, 4096) == "quad_mfma_gemv"
     ext.set_tuning("small_group_mb", old)
