@@ -365,7 +365,8 @@ def calibrate_copy(torch, dev, graph):
     262144 KiB read and 262144 KiB written per copy, the yardstick the FETCH_SIZE / WRITE_SIZE counts are scaled by."""
     srcs = [torch.full((128 * 1024 * 1024,), float(i), dtype=torch.float16, device=dev) for i in range(8)]
     dst = torch.empty_like(srcs[0])
-    graph.replay()  # push the sources out of the last-level cache
+    if graph is not None:
+        graph.replay()  # push the sources out of the last-level cache
     torch.cuda.synchronize()
     for s_ in srcs:
         dst.copy_(s_)
@@ -489,6 +490,8 @@ def main():
 
     if args.selective_only:
         print(json.dumps({"selective": selective_leg(torch, ext, dev)}))
+        if args.calibrate_copy:
+            calibrate_copy(torch, dev, None)
         return
 
     from glowq_amd.kernels import PreparedGroup

@@ -102,9 +102,15 @@ class AddSVDCorrection(nn.Module):
 
     # -- checks ---------------------------------------------------------------------------------------
     def _shapes_ok(self) -> bool:
+        A, B = self._buffers["A_q"], self._buffers["B_q"]
+        memo = self.__dict__.get("_shapes_memo")
+        if memo is not None and memo[0] is A and memo[1] is B:  # a tensor's shape does not change under the same object
+            return memo[2]
         inner = self.inner
-        return (self.A_q.dim() == 2 and self.B_q.dim() == 2 and self.A_q.size(1) == self.B_q.size(0)
-                and self.A_q.size(0) == inner.out_features and self.B_q.size(1) == inner.in_features)
+        ok = (A.dim() == 2 and B.dim() == 2 and A.size(1) == B.size(0)
+              and A.size(0) == inner.out_features and B.size(1) == inner.in_features)
+        self.__dict__["_shapes_memo"] = (A, B, ok)
+        return ok
 
     def _same_right_factor(self, lead: "AddSVDCorrection") -> bool:
         """True when both wrappers hold the same R.  Wrappers built from one artifact tensor share storage;
@@ -139,9 +145,13 @@ class AddSVDCorrection(nn.Module):
         hit = cache.get(key)
         # every tensor whose address sits in the descriptors: a buffer replaced by assignment (re-quantisation,
         # load_state_dict(assign=True), a follower's factor swapped) rebuilds them
-        ptrs = (self.B_q.data_ptr(),) + tuple(
-            p for w in wrappers for p in (w.A_q.data_ptr(), w.inner.qweight_i32.data_ptr(), w.inner.scales_f16.data_ptr(),
-                                          w.inner.qzeros_i32.data_ptr(), w.inner.bias.data_ptr() if w.inner.bias is not None else 0))
+        # (read out of the modules' buffer tables: nn.Module's attribute lookup costs several times a dict access)
+        ptrs = [self._buffers["B_q"].data_ptr()]
+        for w in wrappers:
+            inner = w._modules["inner"]
+            ib, bias = inner._buffers, inner._parameters.get("bias")
+            ptrs += (w._buffers["A_q"].data_ptr(), ib["qweight_i32"].data_ptr(), ib["scales_f16"].data_ptr(), ib["qzeros_i32"].data_ptr(),
+                     bias.data_ptr() if bias is not None else 0)
         if hit is not None and hit[0] == ptrs and hit[1].generation == _kernels.generation():
             return hit[1]
         members = []

@@ -19,8 +19,10 @@
 #include <cstdlib>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "common.hpp"
+#include "tiled.hpp"
 
 namespace glowq {
 
@@ -36,6 +38,8 @@ struct GemmArgs {
   const half_t* bmat;     // [N, ldb] fp16 B operand: L for the correction, or the whole B of a plain GEMM
   const half_t* bias;
   half_t* y;              // [M, ldy]
+  const unsigned char* wt;  // the member's tiled weights (tiled.hpp) or nullptr
+  const unsigned char* lt;  // its tiled left factor or nullptr
   int M, N, K, group_size, rank;
   int ldw, lds, ldz, ldb, ldy;
   float alpha;
@@ -520,6 +524,319 @@ void gemm_mfma_kernel(const GemmGroup gg, const int m_blocks) {
   }
 }
 
+// ---- the same GEMM on the tiled copy of the weights (tiled.hpp) ---------------------------------------------------
+// Same tiles, same workgroup -> tile map, same split of K, same partial tiles and epilogue as gemm_mfma_kernel's
+// super-block form, same arithmetic (the weight is rounded to fp16 once).  What differs is how the operands arrive:
+//   * B: a wave's 16-byte loads of a chunk of the tiled stream ARE the B operands of its 32 x 256 block, in lane order;
+//     scale and zero-point ride in the same chunk (one 8-byte load per lane and super-block).  No pass of the weights
+//     through LDS, no gathers of scales and zero-point words, no per-wave barriers around a staging tile.  One set of
+//     registers holds a super-block; each 16-byte piece is refilled with the next super-block's as soon as its four
+//     words have been dequantised, a whole super-block of matrix instructions ahead of its use.
+//   * A: the tiled copy holds the nibbles of a code word in the order in which the masks deliver them, so the
+//     activations need no permutation and go from memory straight into LDS (buffer_load ... lds: no registers, no
+//     vector instructions, no ds_write).  Stages of 128 columns (one quantisation-group half of a super-block)
+//     instead of 64: half the barriers per matrix instruction.  A load of a wave fills one contiguous kilobyte of
+//     LDS -- four rows of 256 bytes, no padding -- so bank conflicts are avoided by the choice of what goes where:
+//     slot c' of row r holds the 16-byte piece c' ^ (r % 16) of that row, and a fragment read of piece c looks in
+//     slot c ^ (r % 16): sixteen consecutive rows land in sixteen different slots.
+//   * The correction runs first as before, with the tiled left factor as B operand (its pairs at positions 2, 3, 6, 7
+//     of every octet are stored times 16, so r is staged through registers with those pairs divided by 16).
+constexpr int kTRow = 256;  // bytes of a staged row: 128 halves, swizzled instead of padded
+#ifndef GLOWQ_GDBG
+#define GLOWQ_GDBG 0
+#endif
+
+template <int kMT, int kNT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
+void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
+  int wg = (int)blockIdx.x, slice = (int)blockIdx.y, nslices = gg.slices, part_tile = (int)blockIdx.x, part_tiles = (int)gridDim.x;
+  if (gg.tail_slices > 1) {
+    nslices = 1;
+    if (wg >= gg.full) {
+      const int t = wg - gg.full;
+      part_tile = t / gg.tail_slices;
+      slice = t - part_tile * gg.tail_slices;
+      wg = gg.full + part_tile;
+      nslices = gg.tail_slices;
+      part_tiles = ((int)gridDim.x - gg.full) / gg.tail_slices;
+    }
+  }
+  GemmArgs a = gg.m[0];
+  int blk_base = 0;
+#define GLOWQ_PICK(i)                                         \
+  if (gg.n > i && wg >= gg.blk_end[i - 1]) {                 \
+    a = gg.m[i];                                              \
+    blk_base = gg.blk_end[i - 1];                             \
+  }
+  GLOWQ_PICK(1)
+  GLOWQ_PICK(2)
+  GLOWQ_PICK(3)
+#undef GLOWQ_PICK
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int BM = 32 * kMT;
+  constexpr int BN = 128 * kNT;
+  constexpr int kAL = 2 * kMT;  // 16-byte pieces of a stage (BM rows x 256 bytes) per thread
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int blk = wg - blk_base;
+  const int bm = blk % m_blocks;  // row blocks vary fastest: neighbouring workgroups share weight columns
+  const int bn = blk / m_blocks;
+  const int m0 = bm * BM;
+  const int ln = lane & 31, lh = lane >> 5;
+
+  f16v acc[kMT][kNT];
+#pragma unroll
+  for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[tm][tn][i] = 0.f;
+
+  const auto rsrc = [](const void* p, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(uint32_t)bytes, 0x00020000);
+  };
+  const int RB = (a.N + 31) >> 5;
+  const int SB = a.K >> 8;
+  // row block of column tile tn of this wave, clamped into the member (columns past N are computed and dropped)
+  int rb[kNT];
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) rb[tn] = min(bn * (BN / 32) + wave * kNT + tn, RB - 1);
+
+  // ---- activations: piece q of thread t fills slot (t & 15) of row 16 q + (t >> 4) of the stage, which holds the
+  // 16-byte piece (t & 15) ^ (row % 16) of that row's 256 bytes (row % 16 = (t >> 4) % 16 for every q)
+  const int srow = tid >> 4;                    // 0..15: the row within a block of sixteen
+  const int spiece = (tid & 15) ^ srow;         // the piece of the row this thread moves
+  uint32_t a_row[kAL];
+#pragma unroll
+  for (int q = 0; q < kAL; ++q) a_row[q] = (uint32_t)min(m0 + srow + 16 * q, a.M - 1);
+  // A fragment of row tile tm, piece c of the staged row (which 16 columns: see the callers)
+  auto read_a = [&](int stage, int tm, int c) __attribute__((always_inline)) {
+    return *reinterpret_cast<const h8*>(smem + (size_t)stage * BM * kTRow + (tm * 32 + ln) * kTRow + ((c ^ (ln & 15)) << 4));
+  };
+
+  int stage = 0;
+  constexpr int kChunk = kMT < 4 ? kMT : 4;  // row tiles whose A fragments are live at once
+
+  // ---- phase 1: the correction, acc = r . L^T, 128 rank columns (two blocks of the tiled left factor) per stage ----------
+  if (a.r != nullptr && a.lt != nullptr && slice == 0) {
+    const int LB = (a.rank + 63) >> 6;
+    const __amdgpu_buffer_rsrc_t rs_r = rsrc(a.r, (size_t)a.M * a.rank * 2);
+    const __amdgpu_buffer_rsrc_t rs_l = rsrc(a.lt, (size_t)RB * LB * tiled::kLChunk);
+    const int steps = (a.rank + 127) >> 7;
+    u32x4 areg[kAL];
+    auto load_r = [&](int st) __attribute__((always_inline)) {
+#pragma unroll
+      for (int q = 0; q < kAL; ++q) {
+        // columns past the rank meet zeros of the left factor
+        const uint32_t col = (uint32_t)st * 128u + (uint32_t)spiece * 8u;
+        areg[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_r, (int)((a_row[q] * (uint32_t)a.rank + min(col, (uint32_t)a.rank - 8u)) * 2u), 0, 0);
+        if (col >= (uint32_t)a.rank) areg[q] = u32x4{0u, 0u, 0u, 0u};
+      }
+    };
+    auto store_r = [&](int stg) __attribute__((always_inline)) {
+      unsigned char* dst = smem + (size_t)stg * BM * kTRow + srow * kTRow + (tid & 15) * 16;
+      const h2 k16 = {(half_t)0.0625f, (half_t)0.0625f};
+#pragma unroll
+      for (int q = 0; q < kAL; ++q) {
+        u32x4 o = areg[q];
+        o.y = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.y) * k16);
+        o.w = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.w) * k16);
+        *reinterpret_cast<u32x4*>(dst + 16 * q * kTRow) = o;
+      }
+    };
+    load_r(0);
+    store_r(stage);
+    __syncthreads();
+    for (int st = 0; st < steps; ++st) {
+      u32x4 lf[kNT][2][4];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int jb = 2 * st + q;
+          // a block past the rank: an offset past the end of the descriptor (zeros)
+          const uint32_t base = jb < LB ? (uint32_t)(rb[tn] * LB + jb) * (uint32_t)tiled::kLChunk : 0xFFFF0000u;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) lf[tn][q][t] = __builtin_amdgcn_raw_buffer_load_b128(rs_l, lane * 16 + t * 1024, (int)base, 0);
+        }
+      if (st + 1 < steps) load_r(st + 1);
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int c = 0; c < kMT; c += kChunk) {
+            h8 af[kChunk];
+#pragma unroll
+            for (int i = 0; i < kChunk; ++i) af[i] = read_a(stage, c + i, 8 * q + 4 * lh + t);
+#pragma unroll
+            for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+              for (int i = 0; i < kChunk; ++i)
+                acc[c + i][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], __builtin_bit_cast(h8, lf[tn][q][t]), acc[c + i][tn], 0, 0, 0);
+          }
+      if (st + 1 < steps) store_r(stage ^ 1);
+      __syncthreads();
+      stage ^= 1;
+    }
+    if (a.alpha != 1.0f) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= a.alpha;
+    }
+  }
+
+  // ---- phase 2: the quantised K loop, a half of a super-block (128 columns, one quantisation group) per stage --------
+  {
+    const __amdgpu_buffer_rsrc_t rs_x = rsrc(a.x, (size_t)a.M * a.K * 2);
+    const __amdgpu_buffer_rsrc_t rs_w = rsrc(a.wt, (size_t)RB * SB * tiled::kChunk);
+    const uint32_t chunk_stride = (uint32_t)RB * (uint32_t)tiled::kChunk;
+    uint32_t a_off[kAL], w_off[kNT];
+#pragma unroll
+    for (int q = 0; q < kAL; ++q) a_off[q] = (a_row[q] * (uint32_t)a.K + (uint32_t)spiece * 8u) * 2u;
+#pragma unroll
+    for (int tn = 0; tn < kNT; ++tn) w_off[tn] = (uint32_t)rb[tn] * (uint32_t)tiled::kChunk + (uint32_t)lane * 16u;
+    // this workgroup's super-blocks: all of them, or slice `slice` of `nslices`
+    const int sb_per = (SB + nslices - 1) / nslices;
+    const int sb0 = min(slice * sb_per, SB), sb1 = min(sb0 + sb_per, SB);
+    // half-step hs = 2 sb + g (clamped into the slice) of the activations into stage `stg`: every wave fills the four rows
+    // 16 q + 4 wave + [0, 4) of piece q, one contiguous kilobyte of LDS per load
+    auto load_x = [&](int hs, int stg) __attribute__((always_inline)) {
+      const int h = min(hs, 2 * sb1 - 1);
+      typedef __attribute__((address_space(3))) void* lds_ptr_t;
+#pragma unroll
+      for (int q = 0; q < kAL; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lds_ptr_t)(smem + (size_t)stg * BM * kTRow + (16 * q + 4 * wave) * kTRow), 16, (int)a_off[q],
+                                                 h * 256, 0, 0);
+    };
+    // The activations of the next stage have landed before the workgroup's barrier: loads return in order, so it is enough
+    // to wait until no more loads are outstanding than were issued behind them (the refills of this half-step, which
+    // stay in flight).  The scheduling barriers keep the loads where they are written: left alone, the compiler sinks
+    // the refills to the end of the half-step, where nothing hides them.
+    auto wait_loads_but = [&](auto n_const) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_const)::value;
+      __builtin_amdgcn_s_waitcnt((n & 15) | 0x0F70 | ((n >> 4) << 14));  // vmcnt(n), nothing else
+    };
+    // Two sets of weight registers take turns: while the pieces of one are dequantised, the same pieces of the other are
+    // refilled with the next super-block (a set refilled in place would have to be copied at the loop's back edge, and a
+    // copy waits for the load).
+    struct BSet {
+      u32x4 w[kNT][4];
+      u32x2 side[kNT];
+    };
+    BSet b0, b1;
+    const int side_off = tiled::kCodeBytes + ln * 8;
+    if (sb0 < sb1) {
+      load_x(2 * sb0, stage);
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b0.w[tn][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)w_off[tn] + j * 1024, sb0 * (int)chunk_stride, 0);
+        b0.side[tn] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, (int)((uint32_t)rb[tn] * (uint32_t)tiled::kChunk) + side_off,
+                                                                                     sb0 * (int)chunk_stride, 0));
+      }
+      wait_loads_but(std::integral_constant<int, 0>{});
+      __syncthreads();
+    }
+    // g is a compile-time constant at every call site; `cur` holds super-block sb, `nxt` receives sb + 1
+    auto half_step = [&](int sb, auto g_const, const BSet& cur, BSet& nxt) __attribute__((always_inline)) {
+      constexpr int g = decltype(g_const)::value;
+      const int sbn = min(sb + 1, sb1 - 1);  // the last super-block loads itself once more: a uniform number of loads per step
+      if (!(GLOWQ_GDBG & 8)) load_x(2 * sb + g + 1, stage ^ 1);
+      if (g == 1) {
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+          nxt.side[tn] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, (int)((uint32_t)rb[tn] * (uint32_t)tiled::kChunk) + side_off,
+                                                                                        sbn * (int)chunk_stride, 0));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      h2 zb_lo[kNT], zb_hi[kNT], s2[kNT];
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn) {
+        const uint32_t sw = cur.side[tn][g];
+        const float nz = (float)__builtin_bit_cast(half_t, (uint16_t)(sw >> 16)) * 65536.0f;  // -zero
+        const half_t zl = (half_t)(nz - 1024.0f), zh = (half_t)(nz - 64.0f);
+        zb_lo[tn] = h2{zl, zl};
+        zb_hi[tn] = h2{zh, zh};
+        s2[tn] = bitcast_u32<h2>(__builtin_amdgcn_perm(sw, sw, 0x01000100u));
+      }
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+          nxt.w[tn][2 * g + p] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)w_off[tn] + (2 * g + p) * 1024, sbn * (int)chunk_stride, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          h8 bf[kNT];
+#pragma unroll
+          for (int tn = 0; tn < kNT; ++tn)
+            bf[tn] = (GLOWQ_GDBG & 1) ? __builtin_bit_cast(h8, u32x4{cur.w[tn][2 * g + p][i], cur.w[tn][2 * g + p][i] ^ cur.side[tn].x, 0u, 0u})
+                                      : dequant_word(cur.w[tn][2 * g + p][i], zb_lo[tn], zb_hi[tn], s2[tn]);
+#pragma unroll
+          for (int c = 0; c < kMT; c += kChunk) {
+            h8 af[kChunk];
+#pragma unroll
+            for (int u = 0; u < kChunk; ++u)
+              af[u] = (GLOWQ_GDBG & 2) ? __builtin_bit_cast(h8, u32x4{(uint32_t)(c + u + i), (uint32_t)p, (uint32_t)lane, 0u})
+                                       : read_a(stage, c + u, 8 * lh + 4 * p + i);
+#pragma unroll
+            for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+              for (int u = 0; u < kChunk; ++u)
+                acc[c + u][tn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[u], bf[tn], acc[c + u][tn], 0, 0, 0);
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      wait_loads_but(std::integral_constant<int, 2 * kNT + (g == 1 ? kNT : 0)>{});
+      if (!(GLOWQ_GDBG & 4)) __syncthreads();
+      stage ^= 1;
+    };
+    int sb = sb0;
+    for (; sb + 1 < sb1; sb += 2) {
+      half_step(sb, std::integral_constant<int, 0>{}, b0, b1);
+      half_step(sb, std::integral_constant<int, 1>{}, b0, b1);
+      half_step(sb + 1, std::integral_constant<int, 0>{}, b1, b0);
+      half_step(sb + 1, std::integral_constant<int, 1>{}, b1, b0);
+    }
+    if (sb < sb1) {
+      half_step(sb, std::integral_constant<int, 0>{}, b0, b1);
+      half_step(sb, std::integral_constant<int, 1>{}, b0, b1);
+    }
+  }
+
+  // ---- epilogue: accumulator register i of a 32x32 tile is row 8*(i/4) + 4*lh + i%4, column ln ---------
+  if (nslices > 1) {
+    float* part = gg.partials + ((size_t)slice * part_tiles + part_tile) * (BM * BN);
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) part[((tm * kNT + tn) * 16 + i) * 256 + tid] = acc[tm][tn][i];
+    return;
+  }
+#pragma unroll
+  for (int tn = 0; tn < kNT; ++tn) {
+    const int n = bn * BN + wave * (32 * kNT) + tn * 32 + ln;
+    if (n >= a.N) continue;
+    const float b = a.bias ? (float)a.bias[n] : 0.f;
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int m = m0 + tm * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+        if (m < a.M) a.y[(size_t)m * a.ldy + n] = (half_t)(acc[tm][tn][i] + b);
+      }
+    }
+  }
+}
+
 // y = fp16(sum over the slices, in slice order, of the partial tiles of gemm_mfma_kernel<kMT, kNT> + bias); same grid
 // in x, same workgroup -> (member, row block, column block) map and accumulator-register order as the producer.
 // gridDim.y = kMT * kNT: workgroup y of a tile sums one 32 x 32 accumulator tile of each wave (a tile per workgroup
@@ -565,13 +882,16 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, co
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-template <int kMT, int kNT, bool kQuant, bool kSuper = false>
+template <int kMT, int kNT, bool kQuant, bool kSuper = false, bool kTiled = false>
 static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
+  static_assert(!kTiled || (kQuant && kSuper), "the tiled copy serves the super-block form");
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
-  auto kern = gemm_mfma_kernel<kMT, kNT, kQuant, kSuper>;
-  const size_t lds = (size_t)2 * BM * kARow * sizeof(half_t) + (kSuper ? (size_t)4 * (32 * kNT) * 144 : 0);
+  auto kern = kTiled ? gemm_tiled_kernel<kMT, kNT> : gemm_mfma_kernel<kMT, kNT, kQuant, kSuper>;
+  const size_t lds = kTiled ? (size_t)2 * BM * kTRow
+                            : (size_t)2 * BM * kARow * sizeof(half_t) + (kSuper ? (size_t)4 * (32 * kNT) * 144 : 0);
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
+  note_launch(0, 0, 256, "%s<%d,%d>", kTiled ? "gemm_tiled_kernel" : "gemm_mfma_kernel", kMT, kNT);
   const int m_blocks = (gg.m[0].M + BM - 1) / BM;
   int total = 0;
   for (int i = 0; i < gg.n; ++i) {
@@ -689,9 +1009,17 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, size_t ws_bytes,
       }
     }
   }
+  // the tiled copy of the weights where every member brings one (and its tiled left factor where it is corrected)
+  static const int env_tiled = getenv("GLOWQ_GEMM_TILED") ? atoi(getenv("GLOWQ_GEMM_TILED")) : 1;
+  bool tiled_ok = super && env_tiled != 0 && tiled::applies(gg.m[0].K, gg.m[0].group_size);
+  for (int i = 0; i < gg.n; ++i)
+    tiled_ok = tiled_ok && gg.m[i].wt != nullptr && (gg.m[i].r == nullptr || gg.m[i].lt != nullptr) &&
+               tiled::weight_bytes(gg.m[i].N, gg.m[i].K) < (1ull << 32);
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
   if (mt == MT && nt == NT)                                                                \
-    return super ? launch_gemm_t<MT, NT, true, true>(gg, stream) : launch_gemm_t<MT, NT, true>(gg, stream);
+    return tiled_ok ? launch_gemm_t<MT, NT, true, true, true>(gg, stream)                  \
+           : super  ? launch_gemm_t<MT, NT, true, true>(gg, stream)                        \
+                    : launch_gemm_t<MT, NT, true>(gg, stream);
   GLOWQ_GEMM_CASE(8, 2) GLOWQ_GEMM_CASE(4, 2) GLOWQ_GEMM_CASE(2, 2) GLOWQ_GEMM_CASE(1, 2)
   GLOWQ_GEMM_CASE(8, 1) GLOWQ_GEMM_CASE(4, 1) GLOWQ_GEMM_CASE(2, 1) GLOWQ_GEMM_CASE(1, 1)
 #undef GLOWQ_GEMM_CASE
@@ -729,6 +1057,8 @@ hipError_t launch_gemm(GroupDev& g, int num_cus, hipStream_t stream) {
     a.bmat = m.L;
     a.bias = m.bias;
     a.y = m.y;
+    a.wt = static_cast<const unsigned char*>(m.tiled);
+    a.lt = (m.L != nullptr && m.tiled_L != nullptr && m.tiled_rank == g.rank) ? static_cast<const unsigned char*>(m.tiled_L) : nullptr;
     a.M = g.M;
     a.N = m.N;
     a.K = g.K;

@@ -20,8 +20,9 @@
 //   * Consumers keep kD sets of weight registers in rotation: the set of super-block v is refilled with super-block
 //     v + kD as soon as its words have been masked, so up to kD - 1 super-blocks of a wave are in flight while it
 //     computes.  They wait for nothing but their weights.
-//   * Producers load the activations of the next super-block (token rows x 512 bytes) in memory order, permute every
-//     octet into the order the nibble masks deliver the codes, divide the odd pairs by 16, sum every row's two
+//   * Producers load the activations of the next super-block (token rows x 512 bytes) in memory order (the tiled copy
+//     holds the nibbles of a word in the order the masks deliver them: no permutation), divide the pairs at positions
+//     2, 3 and 6, 7 of every octet by 16, sum every row's two
 //     128-column halves in fp32, and leave all of it in the LDS stage the consumers do not read (528-byte rows:
 //     conflict-free 16-byte reads).  One barrier per super-block.  A wave's loads return in order: a consumer that
 //     fetched activations as well would have to drain its weight requests with every step.
@@ -65,13 +66,12 @@ struct TileArgs {
 
 namespace {
 
-__device__ __forceinline__ u32x4 nibble_order_t(const u32x4& v) {
-  // halves (0..7) -> (0,4,1,5,2,6,3,7): two byte permutes per output dword
-  u32x4 o;
-  o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
-  o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
-  o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
-  o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+// The code of column k of a word (nibble k in the canonical buffers) moves to nibble (0,4,1,5,2,6,3,7)[k]: the four
+// masks of the kernels then deliver the eight codes in column order.
+__device__ __forceinline__ uint32_t mask_order_word(uint32_t w) {
+  uint32_t o = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) o |= ((w >> (4 * k)) & 0xFu) << (4 * ((k >> 1) + 4 * (k & 1)));
   return o;
 }
 
@@ -91,6 +91,10 @@ __device__ __forceinline__ float row16_total_t(float v) {
 
 constexpr int kRowBytes = 528;  // 512 bytes of a token row's super-block + 16: rows 8 apart share no bank
 constexpr int kD = 4;           // weight register sets in rotation
+#ifndef GLOWQ_TILED_AUX
+#define GLOWQ_TILED_AUX 2
+#endif
+constexpr int kStreamAux = GLOWQ_TILED_AUX;  // cache policy of the weight loads: non-temporal, every byte is used once
 
 }  // namespace
 
@@ -185,7 +189,7 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
         sum = __builtin_amdgcn_fdot2(h2{v[4], v[5]}, ones, sum, false);
         sum = __builtin_amdgcn_fdot2(h2{v[6], v[7]}, ones, sum, false);
         sum = row16_total_t(sum);
-        u32x4 o = nibble_order_t(av[q]);
+        u32x4 o = av[q];
         o.y = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.y) * sixteenth);
         o.w = __builtin_bit_cast(uint32_t, bitcast_u32<h2>(o.w) * sixteenth);
         *reinterpret_cast<u32x4*>(dst + 2 * kPW * q * kRowBytes) = o;
@@ -255,8 +259,8 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
   BSet bs[kD];
   auto request = [&](BSet& b, int sbq) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + j * 1024, sbq * chunk_stride, 0);
-    b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sbq * chunk_stride + tiled::kCodeBytes, 0));
+    for (int j = 0; j < 4; ++j) b.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + j * 1024, sbq * chunk_stride, kStreamAux);
+    b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sbq * chunk_stride + tiled::kCodeBytes, kStreamAux));
   };
   // two super-blocks up front, the other two once the first activations are staged: with all four at once the whole
   // chip asks for half a long matrix before any wave can begin
@@ -291,12 +295,12 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const u32x4 raw = b.w[j];
-        if constexpr (kRefill) b.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + j * 1024, sb_next * chunk_stride, 0);
+        if constexpr (kRefill) b.w[j] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + j * 1024, sb_next * chunk_stride, kStreamAux);
         f ^= raw.x ^ raw.y ^ raw.z ^ raw.w;
       }
       acc[0][0] += __builtin_bit_cast(float, f & 0x3FFFFFFFu) + *reinterpret_cast<const float*>(st + arow_off);
       if constexpr (kRefill)
-        b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sb_next * chunk_stride + tiled::kCodeBytes, 0));
+        b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sb_next * chunk_stride + tiled::kCodeBytes, kStreamAux));
       return;
     }
 #endif
@@ -306,7 +310,7 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
         const u32x4 raw = b.w[2 * gh + p];
-        if constexpr (kRefill) b.w[2 * gh + p] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + (2 * gh + p) * 1024, sb_next * chunk_stride, 0);
+        if constexpr (kRefill) b.w[2 * gh + p] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, b_off + (2 * gh + p) * 1024, sb_next * chunk_stride, kStreamAux);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t wd = raw[i], hi = wd >> 8;
@@ -336,7 +340,7 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
       }
     }
     if constexpr (kRefill)
-      b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sb_next * chunk_stride + tiled::kCodeBytes, 0));
+      b.side = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_w, ln * 8, sb_next * chunk_stride + tiled::kCodeBytes, kStreamAux));
   };
 
   __syncthreads();
@@ -498,7 +502,8 @@ __global__ __launch_bounds__(256) void pack_tiled_weights_kernel(const int32_t* 
       u32x4 v = {0u, 0u, 0u, 0u};
       if (in) {
         const int32_t* src = qweight + (size_t)row * ldw + sb * 32 + 16 * (j >> 1) + 8 * h + 4 * (j & 1);
-        v = u32x4{(uint32_t)src[0], (uint32_t)src[1], (uint32_t)src[2], (uint32_t)src[3]};
+        v = u32x4{mask_order_word((uint32_t)src[0]), mask_order_word((uint32_t)src[1]), mask_order_word((uint32_t)src[2]),
+                  mask_order_word((uint32_t)src[3])};
       }
       *reinterpret_cast<u32x4*>(dst + 1024 * j + 16 * l) = v;
     }
@@ -518,8 +523,8 @@ __global__ __launch_bounds__(256) void pack_tiled_weights_kernel(const int32_t* 
   }
 }
 
-// One thread per (row block, rank block, lane, k-step): 8 halves of L in nibble order (0,4,1,5,2,6,3,7), those at the
-// odd pairs of the order (elements 1, 5, 3, 7) times 16.
+// One thread per (row block, rank block, lane, k-step): 8 consecutive halves of a row of L, those at positions 2, 3, 6, 7
+// times 16.
 __global__ __launch_bounds__(256) void pack_tiled_left_kernel(const half_t* __restrict__ L, unsigned char* __restrict__ out, int N,
                                                               int rank) {
   const int LB = (rank + 63) >> 6;
@@ -532,9 +537,8 @@ __global__ __launch_bounds__(256) void pack_tiled_left_kernel(const half_t* __re
     h8 v;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int src = (e >> 1) + 4 * (e & 1);  // position e holds element (0,4,1,5,2,6,3,7)[e]
-      const half_t val = (row < N && k0 + src < rank) ? L[(size_t)row * rank + k0 + src] : (half_t)0.f;
-      v[e] = (e & 2) ? val * (half_t)16.f : val;  // positions 2,3 and 6,7: the pairs the activations carry divided by 16
+      const half_t val = (row < N && k0 + e < rank) ? L[(size_t)row * rank + k0 + e] : (half_t)0.f;
+      v[e] = (e & 2) ? val * (half_t)16.f : val;  // the pairs the activations carry divided by 16
     }
     *reinterpret_cast<h8*>(out + (size_t)chunk * tiled::kLChunk + 1024 * t + 16 * l) = v;
   }

@@ -10,7 +10,10 @@
 //     bytes [1024 j + 16 l, +16), j = 2 g + p (g, p in {0, 1}), lane l = 32 h + c:
 //         the 16 bytes (4 words, 32 codes) at byte 64 g + 32 h + 16 p of the 128-byte segment sb of row 32 rb + c,
 //         i.e. the codes of columns 256 sb + 128 g + 64 h + 32 p + [0, 32): word i of it feeds the matrix instruction
-//         (g, p, i), whose sixteen k values (eight per lane half h) all lie in half g -- one quantisation group
+//         (g, p, i), whose sixteen k values (eight per lane half h) all lie in half g -- one quantisation group.
+//         Inside a word the code of its column k (nibble k of the canonical word) sits in nibble (0,4,1,5,2,6,3,7)[k]:
+//         the masks w & 0x000F000F, w & 0x00F000F0, (w >> 8) & 0x000F000F, (w >> 8) & 0x00F000F0 then yield the pairs of
+//         columns (0,1), (2,3), (4,5), (6,7) in order, and the activations need no permutation
 //     bytes [4096 + 8 c + 4 g, +4): low half = fp16 scale of (row 32 rb + c, the group of column 256 sb + 128 g),
 //         high half = fp16(-zero-point * 2^-16) of the same group
 //   rows past N hold zero codes, scale 0 and zero-point 0.
@@ -18,8 +21,9 @@
 //
 // Tiled left factor (fp16 B operand of the correction blocks [r | L]): rank blocks jb of 64 columns, LB = ceil(rank / 64),
 //   chunk(rb, jb) at byte (rb * LB + jb) * 4096: bytes [1024 t + 16 l, +16) = the eight values
-//   L[32 rb + c, 64 jb + 32 h + 8 t + e], e in the order (0,4,1,5,2,6,3,7), those with odd e multiplied by 16 (the
-//   kernels stage the activations of odd columns divided by 16, see skinny_tiled.hip); zero past the rank and past N.
+//   L[32 rb + c, 64 jb + 32 h + 8 t + e], e = 0..7, those with e in {2, 3, 6, 7} multiplied by 16 (the kernels stage
+//   r with those pairs divided by 16, as the raw-code kernel stages all its activations: skinny_tiled.hip); zero past
+//   the rank and past N.
 #pragma once
 
 #include <stddef.h>

@@ -106,6 +106,11 @@ def tiled_enabled() -> bool:
     return os.environ.get("GLOWQ_TILED", "1").lower() not in {"0", "false", "no", "off"}
 
 
+# The raw handle of torch's current stream of a device: the accessor behind `torch.cuda.current_stream(dev).cuda_stream`,
+# without building the Stream object (a forward makes this call once).
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda idx: torch.cuda.current_stream(idx).cuda_stream)
+
+
 def _check(cond: bool, msg: str) -> None:
     if not cond:
         raise RuntimeError(msg)
@@ -130,7 +135,8 @@ class W4A16Extension:
 
     @staticmethod
     def _stream(dev: torch.device) -> int:
-        return torch.cuda.current_stream(dev).cuda_stream
+        idx = dev.index
+        return _raw_stream(idx if idx is not None else torch.cuda.current_device())
 
     WORKSPACE_BYTES = 64 << 20
 
@@ -308,8 +314,12 @@ class W4A16Extension:
     def wants_tiled(self, M: int, K: int, N_total: int, group_size: int, ldw_i32: int) -> bool:
         """Whether a group of this shape would take the route that reads the tiled copies: they are built (and kept in device
         memory beside the canonical buffers) only for such groups."""
-        return (M >= TILED_MIN_ROWS and tiled_enabled()
-                and self.lib.glowq_w4a16_route_tiled(int(M), int(K), int(N_total), int(group_size), int(ldw_i32)) == 8)
+        if M < TILED_MIN_ROWS or not tiled_enabled():
+            return False
+        route = self.lib.glowq_w4a16_route_tiled(int(M), int(K), int(N_total), int(group_size), int(ldw_i32))
+        # 8: the kernel that streams the copy at 5..64 rows; 2: the MFMA GEMM, which takes its B operand from the copy where
+        # the layout applies (its lane order is the matrix instruction's)
+        return route == 8 or (route == 2 and self.lib.glowq_tiled_bytes(int(N_total), int(K), int(group_size)) > 0)
 
     def _set_tiled(self, e, qw, sc, qz, L, in_features: int, group_size: int):
         """Fills the tiled fields of descriptor `e`; returns what has to stay alive with it."""
@@ -638,48 +648,64 @@ class PreparedGroup:
             self.keep.append((qw, sc, qz, L, bias, side))
         self.corrected = corrected
         self._tiled_keep = None  # the tiled copies of the members' weights: built by the first call with five token rows or more
+        self._n_total = sum(self.Ns)
 
     def run(self, x: torch.Tensor, r: Optional[torch.Tensor] = None, outs: Optional[List[torch.Tensor]] = None,
             project: bool = True) -> List[torch.Tensor]:
         """x [M, K] contiguous fp16 on the group's device.  With a right factor and `project`, r = x R^T is computed by
         the call (into `r`, allocated when not given, and kept as `self.last_r`); otherwise `r` is an input (needed when
         the group is corrected).  Returns the members' [M, N_i] outputs (`outs` when given)."""
-        _check(x.is_cuda and x.dtype == torch.float16 and x.dim() == 2 and x.size(1) == self.K and x.is_contiguous(),
-               "inputs must be contiguous CUDA fp16 [M, IC]")
+        if not (x.is_cuda and x.dtype is torch.float16 and x.dim() == 2 and x.size(1) == self.K and x.is_contiguous()):
+            raise RuntimeError("inputs must be contiguous CUDA fp16 [M, IC]")
         M = x.size(0)
-        if self._tiled_keep is None and self.ext.wants_tiled(M, self.K, sum(self.Ns), self.group_size, self.arr[0].ldw_i32):
+        dev = x.device
+        if self._tiled_keep is None and M >= TILED_MIN_ROWS and self.ext.wants_tiled(M, self.K, self._n_total, self.group_size,
+                                                                                    self.arr[0].ldw_i32):
             self._tiled_keep = [self.ext._set_tiled(e, k[0], k[1], k[2], k[3] if self.corrected else None, self.K, self.group_size)
                                 for e, k in zip(self.arr, self.keep)]
+        Ns = self.Ns
         if outs is None:
-            outs = [torch.empty((M, N), dtype=torch.float16, device=x.device) for N in self.Ns]
-        for e, y, N in zip(self.arr, outs, self.Ns):
-            _check(y.dtype == torch.float16 and tuple(y.shape) == (M, N) and y.stride(1) == 1, "output must be CUDA fp16 [M, OC]")
-            e.y, e.ldy = y.data_ptr(), y.stride(0)
+            outs = [torch.empty((M, N), dtype=torch.float16, device=dev) for N in Ns]
+            for e, y in zip(self.arr, outs):
+                e.y, e.ldy = y.data_ptr(), y.stride(0)
+        else:
+            for e, y, N in zip(self.arr, outs, Ns):
+                _check(y.dtype == torch.float16 and tuple(y.shape) == (M, N) and y.stride(1) == 1, "output must be CUDA fp16 [M, OC]")
+                e.y, e.ldy = y.data_ptr(), y.stride(0)
         if M == 0:
             return outs
         fused = project and self.R is not None
-        if (fused or self.corrected) and r is None:
-            _check(fused, "group: a corrected group needs r (or a right factor to compute it from)")
-            r = torch.empty((M, self.rank), dtype=torch.float16, device=x.device)
-        if r is not None:
-            _check(r.dtype == torch.float16 and tuple(r.shape) == (M, self.rank) and r.is_contiguous(), "r must be fp16 [M, rank]")
+        if r is None:
+            if fused or self.corrected:
+                _check(fused, "group: a corrected group needs r (or a right factor to compute it from)")
+                r = torch.empty((M, self.rank), dtype=torch.float16, device=dev)
+        elif not (r.dtype is torch.float16 and r.dim() == 2 and r.size(0) == M and r.size(1) == self.rank and r.is_contiguous()):
+            raise RuntimeError("r must be fp16 [M, rank]")
         self.last_r = r
         ext = self.ext
-        with torch.cuda.device(x.device):
-            ws, ws_bytes = ext._workspace(x.device, M)
+        idx = dev.index
+        # the library launches on the current device: switch only when the tensors live on another one
+        ctx = None
+        if idx is not None and idx != torch.cuda.current_device():
+            ctx = torch.cuda.device(dev)
+            ctx.__enter__()
+        try:
+            ws, ws_bytes = ext._workspace(dev, M) if M > 4 else (None, 0)
+            stream = ext._stream(dev)
             if fused:
                 rc = self.lib.glowq_w4a16_group_forward_fused_ws(
-                    x.data_ptr(), self.R.data_ptr(), r.data_ptr(), self.arr, len(self.Ns), M, self.K, self.group_size,
-                    self.rank, self.alpha, ws, ws_bytes, ext._stream(x.device))
+                    x.data_ptr(), self.R.data_ptr(), r.data_ptr(), self.arr, len(Ns), M, self.K, self.group_size,
+                    self.rank, self.alpha, ws, ws_bytes, stream)
             else:
                 rc = self.lib.glowq_w4a16_group_forward_ws(
-                    x.data_ptr(), r.data_ptr() if (r is not None and self.corrected) else None, self.arr, len(self.Ns), M,
-                    self.K, self.group_size, self.rank if self.corrected else 0, self.alpha, ws, ws_bytes,
-                    ext._stream(x.device))
+                    x.data_ptr(), r.data_ptr() if (r is not None and self.corrected) else None, self.arr, len(Ns), M,
+                    self.K, self.group_size, self.rank if self.corrected else 0, self.alpha, ws, ws_bytes, stream)
+        finally:
+            if ctx is not None:
+                ctx.__exit__(None, None, None)
         if rc:
             ext._raise(rc, "w4a16_group_forward")
         return outs
-
 
     def run_chained(self, x: torch.Tensor, prologue: int, epilogue: int, *, r: Optional[torch.Tensor] = None,
                     outs: Optional[List[Optional[torch.Tensor]]] = None, norm_weight=None, eps: float = 0.0, acc_in=None,

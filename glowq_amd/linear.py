@@ -59,6 +59,20 @@ _KNOB_ENV = ("W4A16_KERNEL_OUT_DTYPE", "MIXED_KERNEL_OUT_DTYPE", "W4A16_FORCE_GE
              "W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV", "W4A16_USE_GEMV", "W4A16_SPLIT_K_ITERS")
 
 
+# os.environ keeps its strings in a plain dict of encoded keys: reading that dict is a fifth of the cost of
+# os.environ.get (no encoding, no KeyError on a miss), and a forward reads all the switches.  Falls back to the mapping
+# itself where the interpreter has no such dict.
+_ENV_DATA = getattr(os.environ, "_data", None)
+_KNOB_KEYS = tuple(os.environ.encodekey(k) for k in _KNOB_ENV) if (_ENV_DATA is not None and hasattr(os.environ, "encodekey")) else None
+
+
+def _raw_env():
+    if _KNOB_KEYS is not None:
+        get = _ENV_DATA.get
+        return tuple([get(k) for k in _KNOB_KEYS])
+    return tuple(map(os.environ.get, _KNOB_ENV))
+
+
 class _Knobs:
     """The `W4A16_*` switches a forward depends on.  The reference reads them from the environment on every forward
     (linear.py:172-177); here they are parsed once and a forward only compares the raw strings with the ones it parsed
@@ -71,7 +85,7 @@ class _Knobs:
         self.read()
 
     def read(self) -> None:
-        self._raw = tuple(map(os.environ.get, _KNOB_ENV))
+        self._raw = _raw_env()
         self.out_dtype = _get_kernel_out_dtype()
         self.force_gemm = _env_flag("W4A16_FORCE_GEMM", "CUDA_MIXED_FORCE_GEMM")
         self.force_gemv = _env_flag("W4A16_FORCE_GEMV", "CUDA_MIXED_FORCE_GEMV")
@@ -79,7 +93,7 @@ class _Knobs:
         self.split_k_iters = _env_number("W4A16_SPLIT_K_ITERS", default=1)
 
     def sync(self) -> None:
-        if tuple(map(os.environ.get, _KNOB_ENV)) != self._raw:
+        if _raw_env() != self._raw:
             self.read()
 
 

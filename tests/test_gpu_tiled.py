@@ -24,7 +24,7 @@ def every_shape_on_the_tiled_route(ext):
 def _untile_weights(blob, N, K):
     """Inverse of the tiled order, written from its definition: chunk (rb, sb), the (sb * RB + rb)-th of 4352 bytes, = 4 x 1024 bytes of codes
     (piece j = 2 g + p of lane l = 32 h + c is bytes [64 g + 32 h + 16 p, +16) of the 128-byte segment sb of row
-    32 rb + c) + per row c the pair (g = 0, 1) of side words: scale bits | fp16(-zero * 2^-16) << 16 of the half's group."""
+    32 rb + c, nibbles re-ordered inside every word) + per row c the pair (g = 0, 1) of side words: scale bits | fp16(-zero * 2^-16) << 16 of the half's group."""
     SB, RB = K // 256, (N + 31) // 32
     b = blob.reshape(SB, RB, 4352).transpose(1, 0, 2)               # [rb, sb, byte]
     codes = b[:, :, :4096].reshape(RB, SB, 2, 2, 2, 32, 16)          # [rb, sb, g, p, h, c, byte]
@@ -33,7 +33,12 @@ def _untile_weights(blob, N, K):
     side = side.transpose(0, 2, 1, 3).reshape(RB * 32, SB * 2)            # [row, 128-column half]
     scales = (side & 0xFFFF).astype(np.uint16).view(np.float16)
     zl = (side >> 16).astype(np.uint16).view(np.float16).astype(np.float64)
-    return rows.copy().view(np.int32), scales, (-zl * 65536.0).astype(np.float32)
+    # inside a word the code of column k sits in nibble (0,4,1,5,2,6,3,7)[k]
+    words = rows.copy().view(np.uint32)
+    canon = np.zeros_like(words)
+    for k, at in enumerate((0, 4, 1, 5, 2, 6, 3, 7)):
+        canon |= ((words >> np.uint32(4 * at)) & np.uint32(0xF)) << np.uint32(4 * k)
+    return canon.view(np.int32), scales, (-zl * 65536.0).astype(np.float32)
 
 
 @pytest.mark.parametrize("N,K,gs", [(64, 512, 128), (40, 1024, 128), (130, 768, 256), (7, 256, 128)])
@@ -63,14 +68,10 @@ def test_tiled_left_factor_holds_L(ext, N, rank):
     L = (torch.randn(N, rank, generator=torch.Generator().manual_seed(N + rank)) * 0.01).half()
     t = ext.pack_tiled_left(L.cuda()).cpu().numpy()
     LB, RB = (rank + 63) // 64, (N + 31) // 32
-    # chunk (rb, jb): piece t of lane 32 h + c = L[32 rb + c, 64 jb + 32 h + 8 t + (0,4,1,5,2,6,3,7)], the elements
-    # 1, 5, 3, 7 (positions 2, 3, 6, 7) times 16
+    # chunk (rb, jb): piece t of lane 32 h + c = L[32 rb + c, 64 jb + 32 h + 8 t + (0..7)], the elements 2, 3, 6, 7 times 16
     b = t.view(np.float16).reshape(RB, LB, 4, 2, 32, 8).copy()        # [rb, jb, t, h, c, e]
     b[..., [2, 3, 6, 7]] /= np.float16(16)
-    order = np.array([0, 4, 1, 5, 2, 6, 3, 7])
-    nat = np.empty_like(b)
-    nat[..., order] = b                                               # position e holds element order[e]
-    full = nat.transpose(0, 4, 1, 3, 2, 5).reshape(RB * 32, LB * 64)  # [rb, c, jb, h, t, e]
+    full = b.transpose(0, 4, 1, 3, 2, 5).reshape(RB * 32, LB * 64)    # [rb, c, jb, h, t, e]
     np.testing.assert_array_equal(full[:N, :rank].view(np.uint16), L.numpy().view(np.uint16))
     assert not full[N:].any() and not full[:, rank:].any()
 
