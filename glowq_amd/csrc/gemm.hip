@@ -546,8 +546,12 @@ constexpr int kTRow = 256;  // bytes of a staged row: 128 halves, swizzled inste
 #define GLOWQ_GDBG 0
 #endif
 
-template <int kMT, int kNT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
+// kWk = 2: eight waves on the same tile, the second four take the second half of the workgroup's K range with LDS stages
+// of their own, and the two accumulator sets meet in LDS before the epilogue.  For launches with about one tile per
+// compute unit: a SIMD then holds two waves of the one workgroup it has, instead of one wave with nothing to overlap its
+// waits with, and the K loop of a tile takes half as many steps.
+template <int kMT, int kNT, int kWk>
+__global__ __launch_bounds__(256 * kWk) __attribute__((amdgpu_waves_per_eu((kMT * kNT >= 16 ? 1 : 2), (kMT * kNT >= 16 ? 1 : 8))))
 void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
   int wg = (int)blockIdx.x, slice = (int)blockIdx.y, nslices = gg.slices, part_tile = (int)blockIdx.x, part_tiles = (int)gridDim.x;
   if (gg.tail_slices > 1) {
@@ -572,11 +576,14 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
   GLOWQ_PICK(2)
   GLOWQ_PICK(3)
 #undef GLOWQ_PICK
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
   constexpr int BM = 32 * kMT;
   constexpr int BN = 128 * kNT;
   constexpr int kAL = 2 * kMT;  // 16-byte pieces of a stage (BM rows x 256 bytes) per thread
-  const int tid = threadIdx.x;
+  static_assert(kWk == 1 || kWk == 2, "one or two K groups");
+  const int gk = kWk > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;  // K group of this wave
+  unsigned char* smem = smem_all + (size_t)gk * 2 * BM * kTRow;
+  const int tid = (int)threadIdx.x & 255;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int blk = wg - blk_base;
@@ -622,7 +629,7 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
   if (a.r != nullptr && a.lt != nullptr && slice == 0) {
     const int LB = (a.rank + 63) >> 6;
     const __amdgpu_buffer_rsrc_t rs_r = rsrc(a.r, (size_t)a.M * a.rank * 2);
-    const __amdgpu_buffer_rsrc_t rs_l = rsrc(a.lt, (size_t)RB * LB * tiled::kLChunk);
+    const __amdgpu_buffer_rsrc_t rs_l = rsrc(a.lt, gk == 0 ? (size_t)RB * LB * tiled::kLChunk : 0);  // one K group adds the correction
     const int steps = (a.rank + 127) >> 7;
     u32x4 areg[kAL];
     auto load_r = [&](int st) __attribute__((always_inline)) {
@@ -693,20 +700,25 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
   // ---- phase 2: the quantised K loop, a half of a super-block (128 columns, one quantisation group) per stage --------
   {
     const __amdgpu_buffer_rsrc_t rs_x = rsrc(a.x, (size_t)a.M * a.K * 2);
-    const __amdgpu_buffer_rsrc_t rs_w = rsrc(a.wt, (size_t)RB * SB * tiled::kChunk);
+    // this workgroup's super-blocks: all of them, or slice `slice` of `nslices`; dealt to the K groups in contiguous halves.
+    // Both groups run the same number of steps (they share the barriers): a step past a group's part reads past the end of
+    // its descriptor -- zero codes at scale zero.
+    const int sb_per = (SB + nslices - 1) / nslices;
+    const int ws0 = min(slice * sb_per, SB), ws1 = min(ws0 + sb_per, SB);
+    const int per_group = (ws1 - ws0 + kWk - 1) / kWk;
+    const int sb0 = min(ws0 + gk * per_group, ws1), sb1 = min(sb0 + per_group, ws1);
+    const int sb_end = sb0 + per_group;  // steps run up to here
+    const __amdgpu_buffer_rsrc_t rs_w = rsrc(a.wt, (size_t)RB * sb1 * tiled::kChunk);
     const uint32_t chunk_stride = (uint32_t)RB * (uint32_t)tiled::kChunk;
     uint32_t a_off[kAL], w_off[kNT];
 #pragma unroll
     for (int q = 0; q < kAL; ++q) a_off[q] = (a_row[q] * (uint32_t)a.K + (uint32_t)spiece * 8u) * 2u;
 #pragma unroll
     for (int tn = 0; tn < kNT; ++tn) w_off[tn] = (uint32_t)rb[tn] * (uint32_t)tiled::kChunk + (uint32_t)lane * 16u;
-    // this workgroup's super-blocks: all of them, or slice `slice` of `nslices`
-    const int sb_per = (SB + nslices - 1) / nslices;
-    const int sb0 = min(slice * sb_per, SB), sb1 = min(sb0 + sb_per, SB);
     // half-step hs = 2 sb + g (clamped into the slice) of the activations into stage `stg`: every wave fills the four rows
     // 16 q + 4 wave + [0, 4) of piece q, one contiguous kilobyte of LDS per load
     auto load_x = [&](int hs, int stg) __attribute__((always_inline)) {
-      const int h = min(hs, 2 * sb1 - 1);
+      const int h = min(hs, 2 * SB - 1);
       typedef __attribute__((address_space(3))) void* lds_ptr_t;
 #pragma unroll
       for (int q = 0; q < kAL; ++q)
@@ -730,7 +742,7 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
     };
     BSet b0, b1;
     const int side_off = tiled::kCodeBytes + ln * 8;
-    if (sb0 < sb1) {
+    if (ws0 < ws1) {
       load_x(2 * sb0, stage);
 #pragma unroll
       for (int tn = 0; tn < kNT; ++tn) {
@@ -745,7 +757,7 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
     // g is a compile-time constant at every call site; `cur` holds super-block sb, `nxt` receives sb + 1
     auto half_step = [&](int sb, auto g_const, const BSet& cur, BSet& nxt) __attribute__((always_inline)) {
       constexpr int g = decltype(g_const)::value;
-      const int sbn = min(sb + 1, sb1 - 1);  // the last super-block loads itself once more: a uniform number of loads per step
+      const int sbn = sb + 1;  // (behind the group's last super-block: past the end of the descriptor, zeros nobody uses)
       if (!(GLOWQ_GDBG & 8)) load_x(2 * sb + g + 1, stage ^ 1);
       if (g == 1) {
 #pragma unroll
@@ -798,16 +810,37 @@ void gemm_tiled_kernel(const GemmGroup gg, const int m_blocks) {
       stage ^= 1;
     };
     int sb = sb0;
-    for (; sb + 1 < sb1; sb += 2) {
+    for (; sb + 1 < sb_end; sb += 2) {
       half_step(sb, std::integral_constant<int, 0>{}, b0, b1);
       half_step(sb, std::integral_constant<int, 1>{}, b0, b1);
       half_step(sb + 1, std::integral_constant<int, 0>{}, b1, b0);
       half_step(sb + 1, std::integral_constant<int, 1>{}, b1, b0);
     }
-    if (sb < sb1) {
+    if (sb < sb_end) {
       half_step(sb, std::integral_constant<int, 0>{}, b0, b1);
       half_step(sb, std::integral_constant<int, 1>{}, b0, b1);
     }
+  }
+
+  // ---- the second K group hands its accumulators over through LDS (the stages are free: every wave is past the last barrier)
+  if constexpr (kWk > 1) {
+    float* red = reinterpret_cast<float*>(smem_all);
+    if (gk == 1) {
+#pragma unroll
+      for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) red[((tm * kNT + tn) * 16 + i) * 256 + tid] = acc[tm][tn][i];
+    }
+    __syncthreads();
+    if (gk == 1) return;
+#pragma unroll
+    for (int tm = 0; tm < kMT; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < kNT; ++tn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[tm][tn][i] += red[((tm * kNT + tn) * 16 + i) * 256 + tid];
   }
 
   // ---- epilogue: accumulator register i of a 32x32 tile is row 8*(i/4) + 4*lh + i%4, column ln ---------
@@ -882,16 +915,18 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmGroup gg, co
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-template <int kMT, int kNT, bool kQuant, bool kSuper = false, bool kTiled = false>
+template <int kMT, int kNT, bool kQuant, bool kSuper = false, bool kTiled = false, int kWk = 1>
 static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   static_assert(!kTiled || (kQuant && kSuper), "the tiled copy serves the super-block form");
+  static_assert(kWk == 1 || kTiled, "K groups inside a workgroup: the tiled-copy kernel");
   constexpr int BM = 32 * kMT, BN = 128 * kNT;
-  auto kern = kTiled ? gemm_tiled_kernel<kMT, kNT> : gemm_mfma_kernel<kMT, kNT, kQuant, kSuper>;
-  const size_t lds = kTiled ? (size_t)2 * BM * kTRow
-                            : (size_t)2 * BM * kARow * sizeof(half_t) + (kSuper ? (size_t)4 * (32 * kNT) * 144 : 0);
+  auto kern = kTiled ? gemm_tiled_kernel<kMT, kNT, kWk> : gemm_mfma_kernel<kMT, kNT, kQuant, kSuper>;
+  size_t lds = kTiled ? (size_t)kWk * 2 * BM * kTRow
+                      : (size_t)2 * BM * kARow * sizeof(half_t) + (kSuper ? (size_t)4 * (32 * kNT) * 144 : 0);
+  if (kWk > 1 && lds < (size_t)BM * BN * sizeof(float)) lds = (size_t)BM * BN * sizeof(float);  // the hand-over of the accumulators
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
-  note_launch(0, 0, 256, "%s<%d,%d>", kTiled ? "gemm_tiled_kernel" : "gemm_mfma_kernel", kMT, kNT);
+  note_launch(0, 0, 256 * kWk, "%s<%d,%d,%d>", kTiled ? "gemm_tiled_kernel" : "gemm_mfma_kernel", kMT, kNT, kWk);
   const int m_blocks = (gg.m[0].M + BM - 1) / BM;
   int total = 0;
   for (int i = 0; i < gg.n; ++i) {
@@ -902,12 +937,12 @@ static hipError_t launch_gemm_t(GemmGroup& gg, hipStream_t stream) {
   if (!(kQuant && kSuper) || gg.slices > 1 || gg.tail_slices < 2 || gg.full < 0 || gg.full >= total) gg.tail_slices = 0;
   if (gg.tail_slices > 1) {
     const int tail_tiles = total - gg.full;
-    hipLaunchKernelGGL(kern, dim3(gg.full + tail_tiles * gg.tail_slices, 1), dim3(256), lds, stream, gg, m_blocks);
+    hipLaunchKernelGGL(kern, dim3(gg.full + tail_tiles * gg.tail_slices, 1), dim3(256 * kWk), lds, stream, gg, m_blocks);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(tail_tiles, kMT * kNT), dim3(256), 0, stream, gg, m_blocks);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(kern, dim3(total, gg.slices), dim3(256), lds, stream, gg, m_blocks);
+  hipLaunchKernelGGL(kern, dim3(total, gg.slices), dim3(256 * kWk), lds, stream, gg, m_blocks);
   if (hipError_t e = hipGetLastError(); e != hipSuccess || gg.slices == 1) return e;
   hipLaunchKernelGGL((gemm_reduce_kernel<kMT, kNT>), dim3(total, kMT * kNT), dim3(256), 0, stream, gg, m_blocks);
   return hipGetLastError();
@@ -956,12 +991,35 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, size_t ws_bytes,
     fits32 = fits32 && rows * gg.m[i].ldw * 4 < (1ull << 32) && rows * gg.m[i].lds * 2 < (1ull << 32) && rows * gg.m[i].ldz * 4 < (1ull << 32);
   }
   const bool super = env_super != 0 && (gg.m[0].K & 255) == 0 && gg.m[0].group_size >= 128 && fits32;
+  // the tiled copy of the weights where every member brings one (and its tiled left factor where it is corrected)
+  static const int env_tiled = getenv("GLOWQ_GEMM_TILED") ? atoi(getenv("GLOWQ_GEMM_TILED")) : 1;
+  bool tiled_ok = super && env_tiled != 0 && tiled::applies(gg.m[0].K, gg.m[0].group_size);
+  for (int i = 0; i < gg.n; ++i)
+    tiled_ok = tiled_ok && gg.m[i].wt != nullptr && (gg.m[i].r == nullptr || gg.m[i].lt != nullptr) &&
+               tiled::weight_bytes(gg.m[i].N, gg.m[i].K) < (1ull << 32);
+  // About one 128 x 256 tile per compute unit and a long K (where K would otherwise be cut into slices over workgroups,
+  // with fp32 partial tiles through the workspace and a second launch for their sum): eight waves per tile, the K range
+  // dealt to two groups of four inside the workgroup (gemm_tiled_kernel's kWk = 2), the sum in LDS.  Qwen2.5-7B down_proj at
+  // 2048 rows (K = 18944, 224 tiles): 308 -> 294 us.  On short K it does not pay: o_proj (K = 3584, 224 tiles) 77.5 -> 78.6 us
+  // against two co-resident 64 x 256 workgroups per compute unit, q|k|v (288 tiles) 100.6 -> 114.9 (its tail tiles, cut
+  // along K, no longer fit beside a whole tile).
+  static const int env_wk = getenv("GLOWQ_GEMM_WK") ? atoi(getenv("GLOWQ_GEMM_WK")) : 0;
+  int wk = 1;
+  if (tiled_ok && mt_cap >= 4 && nt_cap == 2 && env_wk != 1) {
+    long tiles42 = 0;
+    for (int i = 0; i < gg.n; ++i) tiles42 += (long)((M + 127) / 128) * ((gg.m[i].N + 255) / 256);
+    if ((tiles42 * 2 >= num_cus && tiles42 < 2L * num_cus && (gg.m[0].K >> 8) >= 32) || env_wk == 2) {
+      mt = 4;
+      nt = 2;
+      wk = 2;
+    }
+  }
   // Split K through the workspace: where even the largest tile the rows allow leaves CUs idle, that tile is kept and K
   // is cut into slices of at least sixteen super-blocks until the workgroups number about two per CU.
   static const int env_split = getenv("GLOWQ_GEMM_SPLIT") ? atoi(getenv("GLOWQ_GEMM_SPLIT")) : 1;
   const int ws_slices_fit = gg.slices;  // on entry: how many slices of the whole output the workspace holds
   gg.slices = 1;
-  if (super && env_split != 0 && ws_slices_fit >= 2 && mt_cap >= 2 && nt_cap == 2) {
+  if (super && env_split != 0 && ws_slices_fit >= 2 && mt_cap >= 2 && nt_cap == 2 && wk == 1) {
     const int bmt = mt_cap >= 4 ? 4 : 2;
     long tiles = 0;
     for (int i = 0; i < gg.n; ++i) tiles += (long)((M + 32 * bmt - 1) / (32 * bmt)) * ((gg.m[i].N + 255) / 256);
@@ -1009,12 +1067,7 @@ static hipError_t launch_gemm_group(GemmGroup& gg, int num_cus, size_t ws_bytes,
       }
     }
   }
-  // the tiled copy of the weights where every member brings one (and its tiled left factor where it is corrected)
-  static const int env_tiled = getenv("GLOWQ_GEMM_TILED") ? atoi(getenv("GLOWQ_GEMM_TILED")) : 1;
-  bool tiled_ok = super && env_tiled != 0 && tiled::applies(gg.m[0].K, gg.m[0].group_size);
-  for (int i = 0; i < gg.n; ++i)
-    tiled_ok = tiled_ok && gg.m[i].wt != nullptr && (gg.m[i].r == nullptr || gg.m[i].lt != nullptr) &&
-               tiled::weight_bytes(gg.m[i].N, gg.m[i].K) < (1ull << 32);
+  if (wk == 2) return launch_gemm_t<4, 2, true, true, true, 2>(gg, stream);
 #define GLOWQ_GEMM_CASE(MT, NT)                                                            \
   if (mt == MT && nt == NT)                                                                \
     return tiled_ok ? launch_gemm_t<MT, NT, true, true, true>(gg, stream)                  \
