@@ -122,8 +122,8 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
                          const unsigned char* __restrict__ wt0, const int blk_end0, const int N0, const int cw, const TileArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
   constexpr int kMT = kRows > 32 ? 2 : 1;        // 32-row tiles per consumer wave
-  constexpr int kPQ = kRows * 32 / (64 * kPW);   // 16-byte pieces of a super-block of x per producer thread
-  static_assert(kPQ >= 1 && kPQ * 64 * kPW == kRows * 32, "the producer waves share the rows evenly");
+  constexpr int kPQ = (kRows + 2 * kPW - 1) / (2 * kPW);  // 16-byte pieces of a super-block of x per producer thread
+  constexpr bool kRagged = kPQ * 2 * kPW != kRows;       // three producer waves: the last pass covers part of the rows
   constexpr int kSigBytes = kRows * 16;          // per 128-column half: a 16-byte fragment of sums per token row
   constexpr int kStage = kRows * kRowBytes + 2 * kSigBytes;
   constexpr int kLiveRegs = kRows >= 32 ? 16 : (kRows >= 16 ? 8 : 4);  // accumulator registers of rows that exist
@@ -182,6 +182,7 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
       const h2 sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
 #pragma unroll
       for (int q = 0; q < kPQ; ++q) {
+        if (kRagged && 2 * kPW * q + prow >= kRows) break;  // (whole groups of sixteen lanes: the row reduction stays among live lanes)
         // the sixteen lanes pcol / 16 hold the 128 columns of one half of the token row: their sum, in fp32
         const h8 v = __builtin_bit_cast(h8, av[q]);
         float sum = __builtin_amdgcn_fdot2(h2{v[0], v[1]}, ones, 0.f, false);
@@ -625,8 +626,11 @@ static TiledPlan tiled_plan(const GroupDev& g, int num_cus, size_t ws_bytes) {
   int wk = (SB >= 8 && p.cw <= 4 && g.M <= 16 && tiled_tiles(g, p.cw) * 2 > num_cus) ? 2 : 1;
   if (env_wk == 1 || (env_wk == 2 && p.cw <= 4 && g.M <= 32)) wk = env_wk;
   p.pw = g.M <= 8 ? 1 : (g.M <= 16 || wk == 2 ? 2 : 4);
-  if (g.M > 32) wk = 1, p.pw = p.cw > 4 ? 2 : 4;  // two row tiles per wave: 512 threads, their registers allow no more
+  // two row tiles per wave: 512 threads, their registers allow no more -- four producer waves beside four consumers, three
+  // beside five, two beside six
+  if (g.M > 32) wk = 1, p.pw = p.cw > 5 ? 2 : (p.cw > 4 ? 3 : 4);
   if (env_pw == 2 && g.M > 8) p.pw = 2;
+  if (env_pw == 3 && g.M > 32 && p.cw <= 5) p.pw = 3;
   if (env_pw == 4 && g.M > 16 && wk == 1 && (g.M <= 32 || p.cw <= 4)) p.pw = 4;
   p.wk = wk;
   const int tiles = tiled_tiles(g, p.cw);
@@ -705,6 +709,7 @@ hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream) {
     case 3212: return launch_tiled_t<32, 1, 2>(a, g.x, stream);
     case 3214: return launch_tiled_t<32, 1, 4>(a, g.x, stream);
     case 6412: return launch_tiled_t<64, 1, 2>(a, g.x, stream);
+    case 6413: return launch_tiled_t<64, 1, 3>(a, g.x, stream);
     case 6414: return launch_tiled_t<64, 1, 4>(a, g.x, stream);
   }
   return hipErrorInvalidValue;
