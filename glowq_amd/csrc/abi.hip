@@ -114,12 +114,13 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-// r = x R^T on the one-workgroup-per-row-of-R kernel (chunks of four token rows) or on the MFMA projection with its sum
-// over K slices: the first up to 16 rows always, and up to 64 rows while M K rank stays below 60 M multiply-adds
-// (K = 4096, rank 128: 3.9 us against 6.4 at 20 rows, 4.4 against 6.6 at 32, level at 64; K = 14336: 7.2 against 8.2 at
-// 32 rows, 9.4 against 8.4 at 48; K = 17408, rank 256: level at 20 rows, 16.3 against 11.4 at 32).
+// r = x R^T on the kernel with one workgroup per row (or two rows) of R and chunk of four token rows, or on the MFMA
+// projection with its sum over K slices: the first up to 16 rows always, and up to 64 rows while M K rank stays below
+// 90 M multiply-adds (timings of both next to proj_block_shape, misc.hip).
 bool proj_on_small_kernel(int M, int K, int rank) {
-  return M <= 16 || (M <= 64 && (long)M * K * rank <= 60L * 1000 * 1000);
+  static const int force = getenv("GLOWQ_PROJ_SMALL") ? atoi(getenv("GLOWQ_PROJ_SMALL")) : -1;
+  if (force >= 0) return force != 0 && M <= 64;
+  return M <= 16 || (M <= 64 && (long)M * K * rank <= 90L * 1000 * 1000);
 }
 
 int num_cus() {

@@ -1,5 +1,7 @@
 // Small kernels around the main path: dequantisation to fp16, nibble unpacking, and the shared
 // right-factor projection r = x R^T for few token rows.
+#include <cstdlib>
+
 #include "common.hpp"
 #include "side_stream.hpp"
 
@@ -142,6 +144,74 @@ __global__ __launch_bounds__(256) void shared_proj_kernel(const half_t* __restri
   }
 }
 
+// The same for a block of kJ rows of R and kM token rows per workgroup: every 16-byte piece of x the workgroup loads meets
+// kJ rows of R and every piece of R meets kM token rows, so the bytes a workgroup pulls out of L2 per multiply-add fall
+// with both.  For the shapes on which the one-row form is bound by that traffic (many token rows, long K, rank 256).
+// K % 8 == 0, 16-byte aligned rows.
+template <int kM, int kJ>
+__global__ __launch_bounds__(256) void shared_proj_block_kernel(const half_t* __restrict__ x, const half_t* __restrict__ R,
+                                                                half_t* __restrict__ r, int M, int K, int rank) {
+  __shared__ float part[4][kM * kJ];
+  const int j0 = blockIdx.x * kJ;
+  const int m0 = blockIdx.y * kM;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  float acc[kM][kJ];
+#pragma unroll
+  for (int m = 0; m < kM; ++m)
+#pragma unroll
+    for (int j = 0; j < kJ; ++j) acc[m][j] = 0.f;
+  const int words = K >> 3;
+  constexpr int kBatch = (kM + kJ) > 8 ? 1 : 2;  // all loads of a batch are issued before the first is used
+  const h8* xrow[kM];
+  const h8* rrow[kJ];
+#pragma unroll
+  for (int m = 0; m < kM; ++m) xrow[m] = reinterpret_cast<const h8*>(x + (size_t)min(m0 + m, M - 1) * K);
+#pragma unroll
+  for (int j = 0; j < kJ; ++j) rrow[j] = reinterpret_cast<const h8*>(R + (size_t)min(j0 + j, rank - 1) * K);
+  for (int w0 = threadIdx.x; w0 < words; w0 += kBatch * blockDim.x) {
+    h8 rv[kJ][kBatch], xv[kM][kBatch];
+    float live[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int w = w0 + b * blockDim.x;
+      live[b] = w < words ? 1.f : 0.f;
+      const int wc = min(w, words - 1);
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) rv[j][b] = rrow[j][wc];
+#pragma unroll
+      for (int m = 0; m < kM; ++m) xv[m][b] = xrow[m][wc];
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+#pragma unroll
+      for (int m = 0; m < kM; ++m)
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) {
+          float d = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            d = __builtin_amdgcn_fdot2(h2{rv[j][b][2 * i], rv[j][b][2 * i + 1]}, h2{xv[m][b][2 * i], xv[m][b][2 * i + 1]}, d, false);
+          acc[m][j] = __builtin_fmaf(live[b], d, acc[m][j]);
+        }
+  }
+#pragma unroll
+  for (int m = 0; m < kM; ++m)
+#pragma unroll
+    for (int j = 0; j < kJ; ++j) {
+      const float v = wave_sum(acc[m][j]);
+      if (lane == 0) part[wave][m * kJ + j] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < kM * kJ) {
+    const int m = m0 + (int)threadIdx.x / kJ, j = j0 + (int)threadIdx.x % kJ;
+    if (m < M && j < rank) {
+      const int t = threadIdx.x;
+      r[(size_t)m * rank + j] = (half_t)((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
+    }
+  }
+}
+
 // Single token row, K up to 512 kP and a multiple of 8: one wave per row of R, up to kP 16-byte pieces of R and of x per
 // lane, all requested before the first is used; no LDS, no barrier (0.13 us per launch under the four-wave form at
 // K = 4096).
@@ -211,6 +281,19 @@ hipError_t launch_pack_side(const half_t* scales, const int32_t* qzeros, const h
   return hipGetLastError();
 }
 
+// Block shape (token rows x rows of R per workgroup, as 10 * rows + rows of R) of the projection for 3 and more token rows:
+// 41 = the one-row form, 42 = two rows of R per workgroup (half the workgroups, and every piece of x meets two rows of R).
+// One launch in a graph, us, one-row form / 4 x 2 / the MFMA projection with its reduction launch, at 8 / 16 / 32 / 64
+// token rows:  K = 4096, rank 128: 2.8 3.5 4.5 6.9 / 2.7 2.9 3.4 4.3 / 5.8 6.1 6.1 6.1;  K = 14336, rank 128: 4.0 5.0 7.4 12.3 /
+// 4.9 5.1 6.1 9.1 / 7.5 7.7 7.7 8.1;  K = 5120, rank 256: 3.6 4.6 6.9 11.2 / 3.5 4.0 5.1 7.2 / 6.1 6.2 6.3 8.0;  K = 17408,
+// rank 256: 5.8 8.8 15.4 26.7 / 5.5 6.7 9.9 16.5 / 9.0 9.0 9.2 12.3.  (4 x 4 and 8 x 2 blocks are level with 4 x 2 at 64 rows and
+// slower below; 8 x 4 and 8 x 8 leave too few workgroups.)
+static int proj_block_shape(int M, int K, int rank) {
+  if (M < 8) return 41;
+  if (K <= 8192) return 42;
+  return (rank > 128 ? M <= 16 : M > 16) ? 42 : 41;
+}
+
 hipError_t launch_shared_proj_small(const half_t* x, const half_t* R, half_t* r, int M, int K, int rank,
                                     hipStream_t stream) {
   if (M == 1 && (K & 7) == 0 && K <= 4096) {
@@ -222,9 +305,26 @@ hipError_t launch_shared_proj_small(const half_t* x, const half_t* R, half_t* r,
   } else if (M == 2) {
     hipLaunchKernelGGL(shared_proj_kernel<2>, dim3(rank, 1), dim3(256), 0, stream, x, R, r, M, K, rank);
   } else {
-    // (chunks of eight token rows -- half the workgroups, half the re-reads of a row of R -- measured 0.3 to 0.9 us slower
-    // at 12..64 rows)
-    hipLaunchKernelGGL(shared_proj_kernel<4>, dim3(rank, (M + 3) / 4), dim3(256), 0, stream, x, R, r, M, K, rank);
+    // blocks of token rows x rows of R per workgroup (GLOWQ_PROJ_BLOCK=MJ overrides, for tuning runs: 41 is the one-row form)
+    static const int env_block = getenv("GLOWQ_PROJ_BLOCK") ? atoi(getenv("GLOWQ_PROJ_BLOCK")) : 0;
+    int shape = env_block > 0 ? env_block : proj_block_shape(M, K, rank);
+    if ((K & 7) != 0 || (reinterpret_cast<uintptr_t>(x) & 15u) != 0 || (reinterpret_cast<uintptr_t>(R) & 15u) != 0) shape = 41;
+#define GLOWQ_PROJ_CASE(BM, BJ)                                                                                              \
+  case BM * 10 + BJ:                                                                                                         \
+    hipLaunchKernelGGL((shared_proj_block_kernel<BM, BJ>), dim3((rank + BJ - 1) / BJ, (M + BM - 1) / BM), dim3(256), 0, stream, x, R, r, \
+                       M, K, rank);                                                                                          \
+    break;
+    switch (shape) {
+      GLOWQ_PROJ_CASE(4, 2)
+      GLOWQ_PROJ_CASE(4, 4)
+      GLOWQ_PROJ_CASE(8, 2)
+      GLOWQ_PROJ_CASE(8, 4)
+      GLOWQ_PROJ_CASE(8, 8)
+      default:
+        // (chunks of eight token rows on the one-row form measured 0.3 to 0.9 us slower at 12..64 rows)
+        hipLaunchKernelGGL(shared_proj_kernel<4>, dim3(rank, (M + 3) / 4), dim3(256), 0, stream, x, R, r, M, K, rank);
+    }
+#undef GLOWQ_PROJ_CASE
   }
   return hipGetLastError();
 }

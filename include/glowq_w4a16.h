@@ -115,7 +115,7 @@ int glowq_shared_proj(const void* x, const void* R, void* r, int M, int K, int r
 
 /*
  * The same with a caller-provided workspace (same reference lines).  With more than 16 token rows (more than 64, or
- * M * K * rank above 60 million, from where the MFMA projection is used) the output [M, rank] is too small to fill the chip, so K is split over workgroups that leave fp32 partial tiles in `workspace`; a second
+ * M * K * rank above 90 million, from where the MFMA projection is used) the output [M, rank] is too small to fill the chip, so K is split over workgroups that leave fp32 partial tiles in `workspace`; a second
  * small launch adds them in slice order (results do not depend on scheduling) and writes r.
  * `workspace`: 16-byte aligned device memory, contents irrelevant; glowq_proj_workspace_bytes gives the size that lets
  * the split go as far as it is useful for a shape -- a smaller one splits less, NULL or 0 bytes is glowq_shared_proj.
