@@ -150,3 +150,54 @@ def test_tiled_copy_follows_in_place_updates(ext):
     torch.cuda.synchronize()
     assert not torch.equal(y0, y1)
     assert_close(y1.cpu().numpy(), oracle.linear_exact(x, m2["qweight"], m2["qzeros"], m2["scales"], 128), "after in-place update")
+
+
+# ---------------------------------------------------------------- the MFMA GEMM on the tiled copy (more than 64 token rows)
+GEMM_CASES = [
+    # M, K, Ns, rank, alpha, bias
+    (65, 512, [96], 0, 0.0, False),
+    (128, 1024, [256, 300], 72, 0.5, True),
+    (200, 2048, [512], 128, 1.0, False),
+    (300, 768, [130, 64, 31], 8, 1.0, True),
+    (1000, 3584, [512, 512], 128, 1.0, False),
+]
+
+
+@pytest.mark.parametrize("M,K,Ns,rank,alpha,bias", GEMM_CASES)
+def test_gemm_on_the_tiled_copy_matches_oracle(ext, M, K, Ns, rank, alpha, bias):
+    """Above 64 token rows the group runs on the MFMA GEMM, which takes its B operand from the tiled copy: the reference's
+    dequantise-then-matmul arithmetic (src/cuda_w4a16/csrc/gemm_w4a16.cu:46-49,132), weight rounded to fp16 once."""
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(91 + M + K + rank, M, K, Ns, rank, with_bias=bias)
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"]),
+            "L": dev(m["L"]) if rank else None, "bias": dev(m["bias"]) if bias else None} for m in members]
+    assert ext.route(M, K, sum(Ns), 128, tiled=True) == "tiled_mfma_gemm"
+    r = ext.shared_proj(dev(x), dev(R)) if rank else None
+    outs = ext.group_forward(dev(x), r, mem, 128, alpha)
+    torch.cuda.synchronize()
+    assert all(hasattr(m["qweight"], "_glowq_tiled") for m in mem)    # the call built the tiled copies
+    assert ext.last_launch()["kernel"].startswith("gemm_tiled_kernel")
+    for i, (m, y) in enumerate(zip(members, outs)):
+        if rank:
+            want = oracle.corrected_linear_rounded_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha)
+        else:
+            want = oracle.linear_rounded_exact(x, m["qweight"], m["qzeros"], m["scales"], 128)
+        if bias:
+            want = want + m["bias"].astype(np.float64)[None, :]
+        assert_close(y.cpu().numpy(), want, f"tiled GEMM member {i} M={M} K={K}")
+
+
+def test_gemm_on_the_tiled_copy_dequantises_exactly(ext):
+    """Rows of the identity select weight columns: y[m, n] must be the reference's fp16((code - zero) * scale) of column
+    m bit for bit -- the lane order of the tiled chunks, the nibble order inside a word, the side words and the swizzled
+    LDS slots of the activations, all at once."""
+    K, N, gs = 1024, 160, 128
+    _, (m,), _ = make_group(404, 1, K, [N], 0, group_size=gs)
+    cols = np.concatenate([np.arange(0, 256), np.arange(256, K, 3)])
+    x = np.zeros((len(cols), K), dtype=np.float16)
+    x[np.arange(len(cols)), cols] = 1.0
+    mem = [{"qweight": dev(m["qweight"]), "scales": dev(m["scales"]), "qzeros": dev(m["qzeros"])}]
+    y = ext.group_forward(dev(x), None, mem, gs, 0.0)[0].cpu().numpy()
+    assert ext.last_launch()["kernel"].startswith("gemm_tiled_kernel")
+    w = oracle.dequant(m["qweight"], m["qzeros"], m["scales"], K, gs)          # fp16 [N, K]
+    np.testing.assert_array_equal(y.view(np.uint16), np.ascontiguousarray(w[:, cols].T).view(np.uint16))
