@@ -316,6 +316,33 @@ bool tiled_pays(const GroupDev& g) {
   return code_bytes >= 40L * 1000 * 1000 || (g.M > 16 && code_bytes >= 24L * 1000 * 1000);
 }
 
+//   proj_in_launch  1: a single token on the stream GEMV computes r = R x inside the group launch when the call brings a
+//                   workspace for the hand-over (8 bytes per entry of r); 0: always the projection launch in front
+//                   (GLOWQ_PROJ_IN_LAUNCH); 2, for tests: as 1, but the producing waves do not hand their entries over, so
+//                   that every reader runs into the limit below and computes its entry itself
+//   proj_spin_limit polls a reader spends on an entry of r that is not there yet before it computes the entry itself
+//                   (GLOWQ_PROJ_SPIN_LIMIT; 0: never waits)
+std::atomic<int> g_proj_in_launch{clampi(env_or("GLOWQ_PROJ_IN_LAUNCH", 1), 0, 2)};
+std::atomic<int> g_proj_spin_limit{clampi(env_or("GLOWQ_PROJ_SPIN_LIMIT", 16384), 0, 1 << 24)};
+// the block the readers look at (room for rank 256) and the staging words behind it (stream_kernel.hpp)
+constexpr size_t kProjHandoverBytes = 2 * 256 * 8;
+bool proj_in_launch(const GroupDev& g) {
+  if (g.M != 1 || g_proj_in_launch.load(std::memory_order_relaxed) == 0) return false;
+  if (g.ws == nullptr || (reinterpret_cast<uintptr_t>(g.ws) & 7u) != 0 || g.ws_bytes < kProjHandoverBytes) return false;
+  if (g.rank > 256 || !proj_on_small_kernel(g.M, g.K, g.rank) || !aligned16(g.x) || !aligned16(g.R)) return false;
+  bool any_left = false;
+  long blocks = 0;
+  for (int i = 0; i < g.n_members; ++i) {
+    any_left = any_left || g.mem[i].L != nullptr;
+    blocks += (g.mem[i].N + 1) / 2;
+  }
+  // Only launches whose waves (one per row block of two rows) are all on the chip at once.  A workgroup that is done
+  // before r is there waits for it; where a later workgroup waits for its place, that wait costs the launch what the
+  // projection launch in front would have.  Both ways, us per group launch, 8B shapes: q|k|v (3072 waves) 6.9 / 7.8,
+  // o_proj (2048) 6.1 / 6.9, down_proj (2048) 11.0 / 12.6, gate|up (14336) 16.1 to 16.6 / 15.9 to 16.5.
+  return any_left && (g_proj_in_launch.load(std::memory_order_relaxed) == 2 || blocks <= 16L * num_cus());
+}
+
 int pick_route(const GroupDev& g, int force) {
   if (force < 0 && g.M >= g_tiled_min_m.load(std::memory_order_relaxed) && g.M <= g_tiled_max_m.load(std::memory_order_relaxed) &&
       skinny_tiled_supported(g) && tiled_pays(g))
@@ -361,9 +388,17 @@ int pick_route_rounded(const GroupDev& g, int force) {
 int run_group(GroupDev g, int route, hipStream_t stream) {
   const int cus = num_cus();
   hipError_t e = hipSuccess;
-  if (g.R != nullptr) {
-    // r = x R^T goes ahead as a launch of its own.  (Folding it into the group kernel was measured: the
-    // R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch costs.)
+  g.pub = nullptr;
+  if (g.R != nullptr && route == kRouteStream && proj_in_launch(g)) {
+    // single token on the stream GEMV: the first waves of the group launch produce r and hand it to the others through
+    // the workspace (stream_kernel.hpp), no launch in front
+    g.pub = static_cast<unsigned long long*>(g.ws);
+    g.pub_spin = (unsigned)g_proj_spin_limit.load(std::memory_order_relaxed);
+    g.pub_mute = g_proj_in_launch.load(std::memory_order_relaxed) == 2;
+  } else if (g.R != nullptr) {
+    // r = x R^T goes ahead as a launch of its own.  (Having every workgroup of the group kernel compute r for itself
+    // was measured: the R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch
+    // costs.)
     if (!proj_on_small_kernel(g.M, g.K, g.rank) && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
       e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream, g.ws, g.ws_bytes);
     else
@@ -374,7 +409,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   }
   // side streams are used only where every member brings one packed for the rank this launch applies
   bool packed = true;
-  for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr && g.mem[i].side_rank == (g.r ? g.rank : 0);
+  for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr && g.mem[i].side_rank == ((g.r || g.pub) ? g.rank : 0);
   if (!packed)
     for (int i = 0; i < g.n_members; ++i) g.mem[i].side = nullptr;
   static const char* const kRouteNames[] = {"wave_dot_gemv", "skinny_mfma", "tiled_mfma_gemm", "generic", "quad_mfma_gemv",
@@ -733,6 +768,7 @@ int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r
   bool any_tiled = false;
   for (int i = 0; members != nullptr && i < n_members && i < GLOWQ_MAX_MEMBERS; ++i) any_tiled = any_tiled || members[i].tiled != nullptr;
   if (any_tiled) need = std::max(need, glowq::tiled_split_workspace_bytes(M, num_cus()));
+  if (M == 1 && rank > 0) need = std::max(need, kProjHandoverBytes);  // hand-over words of the projection inside the launch
   if (need > kStaticScratchBytes)
     return fail(GLOWQ_EUNSUPPORTED, "group_forward_fused_static: this shape wants %zu bytes of scratch, the static buffer holds %zu",
                 need, kStaticScratchBytes);
@@ -814,6 +850,8 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "tiled_min_m") == 0) { slot = &g_tiled_min_m; lo = 1; hi = 64; }
   else if (strcmp(key, "tiled_max_m") == 0) { slot = &g_tiled_max_m; hi = 64; }
   else if (strcmp(key, "tiled_shape_rule") == 0) { slot = &g_tiled_shape_rule; hi = 1; }
+  else if (strcmp(key, "proj_in_launch") == 0) { slot = &g_proj_in_launch; hi = 2; }
+  else if (strcmp(key, "proj_spin_limit") == 0) { slot = &g_proj_spin_limit; hi = 1 << 24; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

@@ -45,6 +45,11 @@ struct GroupDev {
   half_t* r_out;
   void* ws;         // caller's workspace for the many-row projection (or nullptr) and its size
   size_t ws_bytes;
+  // single-token stream GEMV with the projection inside the launch (run_group decides): the hand-over words of r, one
+  // 64-bit word per entry, and the number of polls a reader spends on one before it computes the entry itself
+  unsigned long long* pub;
+  unsigned pub_spin;
+  int pub_mute;
   MemberDev mem[GLOWQ_MAX_MEMBERS];
   int task_end[GLOWQ_MAX_MEMBERS];  // exclusive prefix of per-member task counts
   int wg_end[GLOWQ_MAX_MEMBERS];    // exclusive prefix of the workgroups assigned to each member
@@ -57,7 +62,7 @@ struct GroupDev {
 namespace streamk {
 constexpr int kAccCopies = GLOWQ_CHAIN_ACC_COPIES;
 constexpr int kAccStride = GLOWQ_CHAIN_ACC_STRIDE;
-constexpr int kProPlain = 0, kProAcc = 1, kProNormAcc = 2;
+constexpr int kProPlain = 0, kProAcc = 1, kProNormAcc = 2, kProProj = 3;
 constexpr int kEpiNone = 0, kEpiResidual = 1, kEpiSwiglu = 2;
 
 struct ChainDev {
@@ -70,6 +75,12 @@ struct ChainDev {
   half_t* act;              // kEpiSwiglu: gated activations [N]
   float eps;                // kProNormAcc
   float part_limit;         // epilogues: see above
+  // kProProj: right factor [rank, K], where r goes for the caller [rank], the hand-over words [rank], polls per word
+  const half_t* proj_R;
+  half_t* proj_r_out;
+  unsigned long long* proj_pub;
+  unsigned proj_spin;
+  int proj_mute;  // producers keep their entries to themselves (a test of what readers do when no entry ever arrives)
 };
 }  // namespace streamk
 

@@ -35,11 +35,13 @@ bool stream_supported(const GroupDev& g) {
 
 namespace {
 
-template <int kKit, int kLW, int kM, bool kPacked>
+// kPro: kProPlain, or kProProj where run_group left the projection to the launch (g.pub set, g.R still there)
+template <int kKit, int kLW, int kM, bool kPacked, int kPro = kProPlain>
 hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
   {
-    auto kern = gemv_stream_kernel<kKit, kLW, kM, kPacked, kProPlain, kEpiNone, stream_xw(kKit), 0>;
-    const size_t lds = wave_dot_lds_bytes(kM, g.K, g.rank, g.r != nullptr);
+    auto kern = gemv_stream_kernel<kKit, kLW, kM, kPacked, kPro, kEpiNone, stream_xw(kKit), 0>;
+    constexpr bool kProj = kPro == kProProj;
+    const size_t lds = wave_dot_lds_bytes(kM, g.K, g.rank, g.r != nullptr || kProj);
     static LdsLimit lds_limit;
     if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
     int total = 0, grid = 0;
@@ -50,9 +52,18 @@ hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
       grid += (blocks + waves - 1) / waves;
       g.wg_end[i] = grid;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), lds, stream, g.x, g.r, g.K, g.r ? g.rank : 0, g.group_size,
-                       g.alpha, g, ChainDev{});
-    note_launch(grid, 1, waves * kWave, "gemv_stream_kernel<%d,%d,%d,%d,%d,%d,%d,%d>", kKit, kLW, kM, (int)kPacked, kProPlain, kEpiNone,
+    ChainDev ch{};
+    if constexpr (kProj) {
+      grid += proj_front_wgs(g.K >> 3, waves, g.rank);  // workgroups in front: the waves that produce r, and the collector
+      ch.proj_R = g.R;
+      ch.proj_r_out = g.r_out;
+      ch.proj_pub = g.pub;
+      ch.proj_spin = g.pub_spin;
+            ch.proj_mute = g.pub_mute;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), lds, stream, g.x, kProj ? nullptr : g.r, g.K,
+                       (g.r || kProj) ? g.rank : 0, g.group_size, g.alpha, g, ch);
+    note_launch(grid, 1, waves * kWave, "gemv_stream_kernel<%d,%d,%d,%d,%d,%d,%d,%d>", kKit, kLW, kM, (int)kPacked, kPro, kEpiNone,
                 stream_xw(kKit), 0);
     return hipGetLastError();
   }
@@ -63,7 +74,13 @@ hipError_t launch_stream_m(GroupDev& g, int waves, hipStream_t stream) {
   bool packed = true;
   for (int i = 0; i < g.n_members; ++i) packed = packed && g.mem[i].side != nullptr;
   switch (g.M) {
-    case 1: return packed ? launch_stream_p<kKit, kLW, 1, true>(g, waves, stream) : launch_stream_p<kKit, kLW, 1, false>(g, waves, stream);
+    case 1:
+      if constexpr (kLW > 0) {
+        if (g.pub != nullptr)
+          return packed ? launch_stream_p<kKit, kLW, 1, true, kProProj>(g, waves, stream)
+                        : launch_stream_p<kKit, kLW, 1, false, kProProj>(g, waves, stream);
+      }
+      return packed ? launch_stream_p<kKit, kLW, 1, true>(g, waves, stream) : launch_stream_p<kKit, kLW, 1, false>(g, waves, stream);
     case 2: return launch_stream_p<kKit, kLW, 2, false>(g, waves, stream);  // side streams serve single rows only
     case 3: return launch_stream_p<kKit, kLW, 3, false>(g, waves, stream);
     case 4: return launch_stream_p<kKit, kLW, 4, false>(g, waves, stream);
@@ -73,7 +90,7 @@ hipError_t launch_stream_m(GroupDev& g, int waves, hipStream_t stream) {
 
 template <int kKit>
 hipError_t launch_stream_lw(GroupDev& g, int waves, hipStream_t stream) {
-  const int lw = g.r ? (g.rank + 127) / 128 : 0;
+  const int lw = (g.r || g.pub) ? (g.rank + 127) / 128 : 0;
   if (lw == 0) return launch_stream_m<kKit, 0>(g, waves, stream);
   if (lw == 1) return launch_stream_m<kKit, 1>(g, waves, stream);
   if (lw == 2) return launch_stream_m<kKit, 2>(g, waves, stream);

@@ -91,6 +91,12 @@ __device__ __forceinline__ u32x2 ld_b64_nt(const void* sbase, uint32_t voff) {
   asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
   return v;
 }
+// (a relaxed atomic load of agent scope: past the caches that are private to a part of the chip)
+__device__ __forceinline__ u32x2 ld_b64_agent(const void* sbase, uint32_t voff) {
+  u32x2 v;
+  asm volatile("global_load_dwordx2 %0, %1, %2 sc1" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+  return v;
+}
 __device__ __forceinline__ u32x3 ld_b96_nt(const void* sbase, uint32_t voff) {
   u32x3 v;
   asm volatile("global_load_dwordx3 %0, %1, %2 nt" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
@@ -164,6 +170,50 @@ __device__ __forceinline__ void wait_words(u32x4 (&a)[kCount]) {
   }
 }
 
+// ---- the projection inside the launch (kProProj, single token) -----------------------------------------------------
+// r = R x is needed by every wave, but only for the last of its dot products.  Instead of a launch of its own in front
+// (2.4 to 3.4 us for 128 rows of R), the grid gets rank / waves workgroups in front that have no row block: each of
+// their waves computes one entry and hands it to everybody else through one 64-bit word per entry in device memory:
+//     bits 48..63: the fp16 value,   bits 0..47: a tag that names this launch.
+// Value and tag travel in the one word, written and read with relaxed atomics of agent scope (they pass the caches that
+// are private to a part of the chip), so a reader that sees the tag has the value and no fence is needed.  The tag is
+// built from the dispatch id of the launch -- the position of its packet in the hardware queue, which a replay of a
+// captured graph renews like any other launch -- and from the address of that queue, with the top bit set so that
+// zeroed memory never matches.  Words left by earlier launches therefore never pass for this launch's, and nothing has
+// to be cleared between launches.  Readers take their word after their weights are consumed, by which time it has long
+// been written (measured on 1792 workgroups: no reader ever polled twice, +0.4 us per launch); a reader that does not
+// find the tag polls a bounded number of times and then computes its entry itself, so every wave ends whatever the
+// order in which the workgroups were started.  Calls that share the words must not overlap.
+// The entries reach the readers in two steps.  A producer leaves its word in a staging area that only one wave reads:
+// the collector, which waits (bounded) until all entries of this launch are there and then writes the block the
+// readers look at, 512 contiguous bytes per store instruction.  Lines that thousands of readers fetch while 128
+// producers write them eight bytes at a time were measured to cost the launch 0.8 to 1.5 us (every write sends the
+// readers of all parts of the chip back to memory for the line); written once, whole, they cost nothing that shows.
+extern "C" __device__ unsigned long long glowq_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
+constexpr unsigned long long kTagMask = 0xFFFFFFFFFFFFull;
+constexpr int kProjStaging = 256;  // the staging words lie behind room for the 256 entries of the largest rank
+__device__ __forceinline__ unsigned long long launch_tag() {
+  const unsigned long long q = (unsigned long long)reinterpret_cast<uintptr_t>(__builtin_amdgcn_queue_ptr());
+  return (glowq_dispatch_id() & 0xFFFFFFFull) | (((q >> 8) & 0x7FFFFull) << 28) | (1ull << 47);
+}
+
+__device__ __forceinline__ float dot8(const h8& a, const h8& c) {
+  float d = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) d = __builtin_amdgcn_fdot2(h2{a[2 * i], a[2 * i + 1]}, h2{c[2 * i], c[2 * i + 1]}, d, false);
+  return d;
+}
+// Entries of r in the summation order of the projection launch they stand in for (misc.hip), so that both ways give the
+// same bits.  Up to 8192 columns one wave owns an entry: lane l adds the 16-byte pieces l, l + 64, ... in turn
+// (shared_proj_wave_kernel).  Above, four waves share it like the four waves of the 256-thread kernel: wave q adds the
+// pieces l + 64 q, l + 64 q + 256, ..., and the four wave totals meet as (p0 + p1) + (p2 + p3) (shared_proj_kernel<1>).
+__host__ __device__ constexpr bool proj_split(int words) { return words > 1024; }
+__host__ __device__ constexpr int proj_entries_per_wg(int words, int waves) { return proj_split(words) ? waves >> 2 : waves; }
+// workgroups in front of the grid: those that produce r, and the collector's
+__host__ __device__ constexpr int proj_front_wgs(int words, int waves, int rank) {
+  return (rank + proj_entries_per_wg(words, waves) - 1) / proj_entries_per_wg(words, waves) + 1;
+}
+
 // What a wave holds of one row block: kKit steps of two 16-byte units (32 codes of each row), and the side data.
 // From the canonical buffers: the scale and the zero-point word of one (row, group) per lane and pair of steps -- lane
 // 32 r + i has group gbase(p) + i of row r for pair p -- and kLW dwords of each row of L.  From a side stream
@@ -213,12 +263,15 @@ __host__ __device__ constexpr int stream_xw(int kit) { return stream_heavy(kit) 
 // Waves per SIMD the register allocation aims at (the bounds of amdgpu_waves_per_eu).  The plain light forms end up at
 // 64 VGPRs = 8 waves by themselves; the chained ones carry norm weights, accumulator words and the next right factor on
 // top and have to be told (left at 4 waves the gate|up launch of an 8B layer took 23.7 us instead of 13): as many waves
-// as compile without spilling -- the build refuses scratch in these kernels.
+// as compile without spilling -- the build refuses scratch in these kernels.  (The forms with the projection inside
+// the launch come out one or two registers above 64 at up to two steps, and are held to 8 waves as well where they
+// read side streams, to 7 from the canonical buffers.)
 __host__ __device__ constexpr int stream_min_waves(int kit, int lw, int al, bool chained) {
   if (stream_heavy(kit)) return 1;
   if (!chained || kit > 2) return 2;
   return lw <= 1 ? (al <= 2 ? 8 : 7) : (al <= 2 ? 6 : 2);
 }
+__host__ __device__ constexpr bool stream_chained(int pro, int epi) { return pro == kProAcc || pro == kProNormAcc || epi != kEpiNone; }
 __host__ __device__ constexpr int stream_max_waves(int kit, bool chained) { return stream_heavy(kit) ? 2 : (chained && kit <= 2 ? 8 : 4); }
 
 // LDS of the plain forms: xs [kM][4][U] units of 8 halves in nibble order, sig [kM][U], rs [kM][rank] (gemv.hip); the
@@ -246,16 +299,20 @@ __host__ __device__ constexpr int chain_acc_loads(bool w8) { return w8 ? 2 : 4; 
 // held to 128 VGPRs (4 waves per SIMD), heavy ones get 256.
 template <int kKit, int kLW, int kM, bool kPacked, int kPro, int kEpi, int kXW, int kAL>
 __global__ __launch_bounds__(stream_heavy(kKit) ? 512 : 1024)
-__attribute__((amdgpu_waves_per_eu(stream_min_waves(kKit, kLW, kAL, kPro != kProPlain || kEpi != kEpiNone),
-                                   stream_max_waves(kKit, kPro != kProPlain || kEpi != kEpiNone))))
+__attribute__((amdgpu_waves_per_eu(kPro == kProProj && kKit <= 2 ? (kPacked ? 8 : 7) : stream_min_waves(kKit, kLW, kAL, stream_chained(kPro, kEpi)),
+                                   kPro == kProProj && kKit <= 2 ? 8 : stream_max_waves(kKit, stream_chained(kPro, kEpi)))))
 void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__ r, const int K, const int rank,
                         const int group_size, const float alpha, const GroupDev g, const ChainDev ch) {
   using C = SlotCounts<kKit, kLW, kPacked, kEpi>;
   constexpr int kNP = C::kNP;
-  constexpr bool kChained = kPro != kProPlain || kEpi != kEpiNone;
-  static_assert(C::kLoads <= 63, "the wait for the activations counts every load behind them");
+  constexpr bool kChained = stream_chained(kPro, kEpi);
+  constexpr bool kAccPro = kPro == kProAcc || kPro == kProNormAcc;  // r comes out of an accumulator
+  // kProProj: each thread's first look at its entry of r goes out ahead of the wait for the last step's weights
+  constexpr int kLook = kPro == kProProj ? 1 : 0;
+  static_assert(C::kLoads + kLook <= 63, "the waits count every load behind the one they are for");
   static_assert(!kChained || (kM == 1 && !kPacked), "the chained forms serve one token from the canonical buffers");
-  static_assert(kPro == kProPlain || kLW > 0, "a chained prologue takes r from an accumulator");
+  static_assert(kPro == kProPlain || kLW > 0, "every other prologue is about r");
+  static_assert(kPro != kProProj || (kM == 1 && kEpi == kEpiNone), "the projection inside the launch serves one token, plain epilogue");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int U = K >> 5;
   const int upg_shift = __builtin_ctz(group_size >> 5);
@@ -272,15 +329,103 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int threads = blockDim.x, waves = threads >> 6;
   const int ldw_half = rank >> 1;  // dwords per row of L
-  float* part = reinterpret_cast<float*>(accp + (kPro != kProPlain ? (size_t)waves * 128 * kLW : 0));
+  float* part = reinterpret_cast<float*>(accp + (kAccPro ? (size_t)waves * 128 * kLW : 0));
+
+  const int words = K >> 3;
+  // ---- kProProj: the workgroups in front of the grid have no row block (see above).  They are the first to be started
+  // and nobody's weights wait behind their dot products.  Their waves produce one entry of r each and leave it in the
+  // staging words; wave 0 of the last of them collects the staging words and publishes the block the readers look at.
+  unsigned long long tag = 0;
+  int wg = (int)blockIdx.x;
+  if constexpr (kPro == kProProj) {
+    tag = launch_tag();
+    const int front = proj_front_wgs(words, waves, rank);
+    unsigned long long* staging = ch.proj_pub + kProjStaging;
+    if (wg < front - 1) {
+      // the row of R first (up to eight pieces per lane in flight), then x into LDS in its natural order by the whole
+      // workgroup while they travel
+      const bool split = proj_split(words);
+      const int epw = proj_entries_per_wg(words, waves);
+      const int j = __builtin_amdgcn_readfirstlane(wg * epw + (split ? wave >> 2 : wave));
+      const int q = split ? wave & 3 : 0;
+      const bool active = j < rank && (!split || wave < 4 * epw);
+      const int stride = split ? 256 : kWave, first = lane + kWave * q;
+      const int pieces = (words + stride - 1) / stride;  // of the lanes with the most
+      // (a scalar base and 32-bit byte offsets: eight 64-bit addresses per lane would cost the kernel a wave per SIMD)
+      const char* Rb = reinterpret_cast<const char*>(ch.proj_R + (size_t)(active ? j : 0) * K);
+      auto piece = [&](int w) { return *reinterpret_cast<const h8*>(Rb + ((uint32_t)min(w, words - 1) << 4)); };
+      h8* xn = reinterpret_cast<h8*>(smem);
+      float* pp = reinterpret_cast<float*>(smem + (size_t)K * sizeof(half_t));  // (split form: K > 8192, room for 16 floats)
+      h8 rv[8];
+#pragma unroll
+      for (int b = 0; b < 8; ++b) rv[b] = piece(first + stride * b);
+#pragma unroll 1
+      for (int w = (int)threadIdx.x; w < words; w += threads) xn[w] = reinterpret_cast<const h8*>(x)[w];
+      __syncthreads();
+      float acc = 0.f;
+      for (int b0 = 0; b0 < pieces; b0 += 8) {
+        if (b0 > 0) {
+#pragma unroll
+          for (int b = 0; b < 8; ++b) rv[b] = piece(first + stride * (b0 + b));
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+          const int w = first + stride * (b0 + b);
+          const float d = dot8(rv[b], xn[min(w, words - 1)]);
+          acc = w < words ? acc + d : acc;
+        }
+      }
+      float total = wave_sum(acc);
+      if (split) {
+        if (lane == 0) pp[wave] = total;
+        __syncthreads();
+        total = (pp[wave & ~3] + pp[(wave & ~3) + 1]) + (pp[(wave & ~3) + 2] + pp[(wave & ~3) + 3]);
+      }
+      if (active && q == 0 && lane == 0) {
+        const half_t v = (half_t)total;
+        ch.proj_r_out[j] = v;
+        // (proj_mute: a test of the readers' own dot product -- the caller still gets r, the readers never do)
+        if (!(ch.proj_mute & 1))
+          __hip_atomic_store(staging + j, ((unsigned long long)__builtin_bit_cast(uint16_t, v) << 48) | tag, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      }
+      return;
+    }
+    if (wg == front - 1) {
+      if (wave != 0) return;
+      // the collector: lane l takes entries l, l + 64, ...; when every entry carries the tag, each store instruction
+      // below writes 512 contiguous bytes, whole lines.  (One wave only: four that polled in turn, to find the entries
+      // sooner, wrote the block more than once and cost the launch a microsecond.)
+      unsigned long long w[4] = {0, 0, 0, 0};
+      bool all = false;
+      for (unsigned spins = 0; !all && spins <= ch.proj_spin; ++spins) {
+        bool mine = true;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (lane + kWave * q < rank) {
+            w[q] = __hip_atomic_load(staging + lane + kWave * q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            mine = mine && (w[q] & kTagMask) == tag;
+          }
+        }
+        all = __builtin_amdgcn_ballot_w64(!mine) == 0;
+        if (!all) __builtin_amdgcn_s_sleep(4);
+      }
+      if (all) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (lane + kWave * q < rank) __hip_atomic_store(ch.proj_pub + lane + kWave * q, w[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      return;  // (without all entries nothing is published: the readers run into their limit and compute r themselves)
+    }
+    wg -= front;
+  }
 
   // ---- activations first: their wait then does not cover the weight requests issued behind them
-  const int words = K >> 3;
   u32x4 xw[kM][kXW];
   u32x4 nw[kPro == kProNormAcc ? kXW : 1];
   uint32_t rw[kM];
   // accumulator: wave w takes copies w, w + waves, ...; lane l their entries 2 l, 2 l + 1 (+ 128 j)
-  u32x4 av[kPro != kProPlain ? kAL : 1][kLW > 0 ? kLW : 1];
+  u32x4 av[kAccPro ? kAL : 1][kLW > 0 ? kLW : 1];
 #pragma unroll
   for (int m = 0; m < kM; ++m) {
 #pragma unroll
@@ -293,7 +438,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
 #pragma unroll
     for (int i = 0; i < kXW; ++i) nw[i] = ld_b128(ch.norm_w, (uint32_t)min((int)threadIdx.x + i * threads, words - 1) * 16u);
   }
-  if constexpr (kPro != kProPlain) {
+  if constexpr (kAccPro) {
     // Loads and waits are unconditional (a copy past the last one is clamped to it and left out of the sum below): the
     // compiler takes the result of a load statement for present as soon as the statement has run, so a load under a
     // condition gets its result copied to the variable's register where the branches meet -- before the data is there
@@ -311,7 +456,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
   int wg_begin = 0, total_blocks = g.task_end[0];
   if constexpr (kEpi == kEpiNone) {
 #define GLOWQ_PICK(i)                                            \
-  if (g.n_members > i && (int)blockIdx.x >= g.wg_end[i - 1]) {  \
+  if (g.n_members > i && wg >= g.wg_end[i - 1]) {               \
     mem = g.mem[i];                                              \
     wg_begin = g.wg_end[i - 1];                                  \
     total_blocks = g.task_end[i] - g.task_end[i - 1];            \
@@ -321,7 +466,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
     GLOWQ_PICK(3)
 #undef GLOWQ_PICK
   }
-  const int want = ((int)blockIdx.x - wg_begin) * waves + wave;
+  const int want = (wg - wg_begin) * waves + wave;
   const bool valid = want < total_blocks;
   const int blk = valid ? want : total_blocks - 1;
   const float alpha_scaled = (mem.L != nullptr ? alpha : 0.f) * 0x1p-24f;  // accumulators carry 2^-24
@@ -379,8 +524,8 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
         }
       }
       if constexpr (kLW > 0) {
-        // a member without L reads r itself (valid memory) and is weighted by zero
-        const half_t* some = kPro == kProPlain ? r : reinterpret_cast<const half_t*>(ch.acc_in);
+        // a member without L reads r itself (valid memory; x where r is produced inside the launch) and is weighted by zero
+        const half_t* some = kPro == kProPlain ? r : kPro == kProProj ? x : reinterpret_cast<const half_t*>(ch.acc_in);
         const char* l0 = mem.L ? reinterpret_cast<const char*>(mem.L + (size_t)n0 * rank) : reinterpret_cast<const char*>(some);
         const char* l1 = (mem.L && two) ? l0 + (size_t)rank * 2 : l0;
         if constexpr (kEpi == kEpiSwiglu) l1 = reinterpret_cast<const char*>(g.mem[1].L + (size_t)n0 * rank);
@@ -490,7 +635,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
       if ((int)threadIdx.x < ldw_half) reinterpret_cast<uint32_t*>(rs + (size_t)m * rank)[threadIdx.x] = rw[m];
     }
   }
-  if constexpr (kPro != kProPlain) {
+  if constexpr (kAccPro) {
     // this wave's share of the sum over the copies, entry by entry, for every wave to pick up behind the barrier
 #pragma unroll
     for (int j = 0; j < kLW; ++j) {
@@ -510,21 +655,56 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
     }
   }
   __syncthreads();
-  if constexpr (kEpi == kEpiNone) {
+  if constexpr (kEpi == kEpiNone && kPro != kProProj) {
     if (!valid) return;  // (after the barrier; the loads still in flight land in registers nobody reads)
   }
-
+  // kProProj: thread t's first look at entry t of r (rank <= 256 <= threads) goes out ahead of the wait for the last
+  // step's weights: as late as it can without adding a round trip of its own behind them
+  u32x2 look = {0u, 0u};
   // ---- consume the row block in the order it was requested
   float tot[kSRows][kM];
 #pragma unroll
   for (int rr = 0; rr < kSRows; ++rr)
 #pragma unroll
     for (int m = 0; m < kM; ++m) tot[rr][m] = 0.f;
+  // the correction's share: [L] . [alpha r], r from LDS (or, in the accumulator forms, from the sums staged there)
+  auto apply_left = [&]() {
+#pragma unroll
+    for (int j = 0; j < kLW; ++j) {
+      const int idx = lane + kWave * j;
+      // (gate/up pair: both members carry L, checked on the host)
+      const float a = idx < ldw_half ? alpha_scaled : 0.f;
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+        h2 rv;
+        if constexpr (!kAccPro) {
+          rv = reinterpret_cast<const h2*>(rs + (size_t)m * rank)[min(idx, ldw_half - 1)];
+        } else {
+          // r = fp16(f P), P = 2^-32 * (sum over the waves' shares); an accumulator that overflowed gives NaN
+          const int li = min(idx, ldw_half - 1);
+          long long s0 = 0, s1 = 0;
+          for (int w = 0; w < waves; ++w) {
+            const long long* src = accp + ((size_t)w * kLW + (li >> 6)) * 128 + 2 * (li & 63);
+            s0 += src[0];
+            s1 += src[1];
+          }
+          const float bad = ch.acc_in[(size_t)kAccCopies * kAccStride] != 0 ? __builtin_nanf("") : 0.f;
+          rv = h2{(half_t)((float)s0 * 0x1p-32f * norm_f + bad), (half_t)((float)s1 * 0x1p-32f * norm_f + bad)};
+        }
+#pragma unroll
+        for (int rr = 0; rr < kSRows; ++rr)
+          tot[rr][m] = __builtin_fmaf(a, __builtin_amdgcn_fdot2(bitcast_u32<h2>(kPacked ? b.side(kNP + kSRows * j + rr) : b.l[rr][j]),
+                                                             rv, 0.f, false), tot[rr][m]);
+      }
+    }
+  };
+  float held_sc[kPro == kProProj ? kKit : 1][kSRows], held_v[kPro == kProProj ? kKit : 1][kSRows];
   uint32_t rec = 0;
   static_for<kKit>([&](auto IT) {
     constexpr int it = decltype(IT)::value;
     constexpr int p = it >> 1;
-    constexpr int kBehind = kSRows * (kKit - 1 - it);  // loads issued behind the weights of this step
+    constexpr int kBehind = kSRows * (kKit - 1 - it) + (it == kKit - 1 ? kLook : 0);  // loads issued behind the weights of this step
+    if constexpr (kPro == kProProj && it == kKit - 1) look = ld_b64_agent(ch.proj_pub, (uint32_t)min((int)threadIdx.x, rank - 1) * 8u);
     const int uraw = lane + it * kWave;
     const bool active = uraw < U;
     int u = active ? uraw : U - 1;
@@ -598,50 +778,60 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
         }
         float v = __builtin_fmaf(accB, 0.0625f, accA);
         v = __builtin_fmaf(-zp[rr], sg, v);
-        tot[rr][m] = __builtin_fmaf(sc[rr], v, tot[rr][m]);
-      }
-    }
-    if constexpr (it == 0 && kLW > 0) {
-#pragma unroll
-      for (int j = 0; j < kLW; ++j) {
-        const int idx = lane + kWave * j;
-        // (gate/up pair: both members carry L, checked on the host)
-        const float a = idx < ldw_half ? alpha_scaled : 0.f;
-#pragma unroll
-        for (int m = 0; m < kM; ++m) {
-          h2 rv;
-          if constexpr (kPro == kProPlain) {
-            rv = reinterpret_cast<const h2*>(rs + (size_t)m * rank)[min(idx, ldw_half - 1)];
-          } else {
-            // r = fp16(f P), P = 2^-32 * (sum over the waves' shares); an accumulator that overflowed gives NaN
-            const int li = min(idx, ldw_half - 1);
-            long long s0 = 0, s1 = 0;
-            for (int w = 0; w < waves; ++w) {
-              const long long* src = accp + ((size_t)w * kLW + (li >> 6)) * 128 + 2 * (li & 63);
-              s0 += src[0];
-              s1 += src[1];
-            }
-            const float bad = ch.acc_in[(size_t)kAccCopies * kAccStride] != 0 ? __builtin_nanf("") : 0.f;
-            rv = h2{(half_t)((float)s0 * 0x1p-32f * norm_f + bad), (half_t)((float)s1 * 0x1p-32f * norm_f + bad)};
-          }
-#pragma unroll
-          for (int rr = 0; rr < kSRows; ++rr)
-            tot[rr][m] = __builtin_fmaf(a, __builtin_amdgcn_fdot2(bitcast_u32<h2>(kPacked ? b.side(kNP + kSRows * j + rr) : b.l[rr][j]),
-                                                               rv, 0.f, false), tot[rr][m]);
+        if constexpr (kPro == kProProj && it > 0) {
+          // held back: the sums of every form add in the same order (step 0, the correction, the other steps), and here
+          // the correction has to wait for r
+          held_sc[it][rr] = sc[rr];
+          held_v[it][rr] = v;
+        } else {
+          tot[rr][m] = __builtin_fmaf(sc[rr], v, tot[rr][m]);
         }
       }
     }
+    if constexpr (it == 0 && kLW > 0 && kPro != kProProj) apply_left();
     // The step's sums are pinned here (an empty statement that "rewrites" them): left alone, the compiler sinks the whole
     // arithmetic of every step to the point of the reduction below, behind all the waits, and keeps every loaded word
     // and activation fragment of every step live until then (30 VGPRs per step and token row).
 #pragma unroll
-    for (int rr = 0; rr < kSRows; ++rr)
+    for (int rr = 0; rr < kSRows; ++rr) {
 #pragma unroll
       for (int m = 0; m < kM; ++m) asm volatile("" : "+v"(tot[rr][m]));
+      if constexpr (kPro == kProProj && it > 0) asm volatile("" : "+v"(held_v[it][rr]));
+    }
   });
+  if constexpr (kPro == kProProj) {
+    // r from the waves that produced it: thread t has looked at entry t; where the word was not there yet it looks again
+    wait_vm<0>(look);
+    if ((int)threadIdx.x < rank) {
+      unsigned long long w = ((unsigned long long)look[1] << 32) | look[0];
+      unsigned spins = 0;
+      bool seen = (w & kTagMask) == tag;
+      while (!seen && spins < ch.proj_spin) {
+        ++spins;
+        w = __hip_atomic_load(ch.proj_pub + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        seen = (w & kTagMask) == tag;
+        if (!seen) __builtin_amdgcn_s_sleep(8);
+      }
+      half_t v = __builtin_bit_cast(half_t, (uint16_t)(w >> 48));
+      if (!seen) {
+        // the producer has not been heard from within the limit: this thread's own dot product (fp32, column order)
+        const half_t* Rrow = ch.proj_R + (size_t)threadIdx.x * K;
+        float acc = 0.f;
+        for (int k = 0; k < K; ++k) acc = __builtin_fmaf((float)Rrow[k], (float)x[k], acc);
+        v = (half_t)acc;
+      }
+      rs[threadIdx.x] = v;
+    }
+    __syncthreads();
+    apply_left();
+#pragma unroll
+    for (int it = 1; it < kKit; ++it)
+#pragma unroll
+      for (int rr = 0; rr < kSRows; ++rr) tot[rr][0] = __builtin_fmaf(held_sc[it][rr], held_v[it][rr], tot[rr][0]);
+  }
   // lane rr keeps the total of row rr: one store (and one bias load) per token row
   const int n = blk * kSRows + lane;
-  const bool writer = lane < kSRows && n < mem.N;
+  const bool writer = valid && lane < kSRows && n < mem.N;
   float bias = 0.f;
   if constexpr (kEpi == kEpiNone) bias = (writer && mem.bias) ? (float)mem.bias[n] : 0.f;
   float row0 = 0.f, row1 = 0.f;

@@ -140,19 +140,24 @@ class W4A16Extension:
 
     WORKSPACE_BYTES = 64 << 20
 
+    HANDOVER_BYTES = 4096
+
     def _workspace(self, dev: torch.device, rows: int):
-        """(pointer, bytes) of the workspace of the current stream of `dev` (many-row projection, split-K of the GEMM
-        and of the skinny kernel): one per stream, because calls that share one must not overlap.  Only calls with more
-        than 4 token rows use it.  A stream that meets its first such call while it is being captured into a graph goes
-        without (the buffer would come from the graph's own memory pool)."""
-        if rows <= 4:
+        """(pointer, bytes) of the workspace of the current stream of `dev`: one per stream, because calls that share
+        one must not overlap.  Calls with more than 4 token rows get the large one (many-row projection, split-K of the
+        GEMM and of the skinny kernels); single-token calls a small one, through which a group launch that computes r
+        itself hands it from the waves that produce it to the others; two to four rows use none.  A stream that meets
+        its first such call while it is being captured into a graph goes without (the buffer would come from the
+        graph's own memory pool)."""
+        if 1 < rows <= 4:
             return None, 0
-        key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev))
+        small = rows <= 1
+        key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev), small)
         ws = self._workspaces.get(key)
         if ws is None:
             if torch.cuda.is_current_stream_capturing():
                 return None, 0
-            ws = torch.empty(self.WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+            ws = torch.zeros(self.HANDOVER_BYTES if small else self.WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
             self._workspaces[key] = ws
         return ws.data_ptr(), ws.numel()
 
@@ -690,7 +695,7 @@ class PreparedGroup:
             ctx = torch.cuda.device(dev)
             ctx.__enter__()
         try:
-            ws, ws_bytes = ext._workspace(dev, M) if M > 4 else (None, 0)
+            ws, ws_bytes = ext._workspace(dev, M)
             stream = ext._stream(dev)
             if fused:
                 rc = self.lib.glowq_w4a16_group_forward_fused_ws(
