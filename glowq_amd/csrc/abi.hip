@@ -324,23 +324,16 @@ bool tiled_pays(const GroupDev& g) {
 //                   (GLOWQ_PROJ_SPIN_LIMIT; 0: never waits)
 std::atomic<int> g_proj_in_launch{clampi(env_or("GLOWQ_PROJ_IN_LAUNCH", 1), 0, 2)};
 std::atomic<int> g_proj_spin_limit{clampi(env_or("GLOWQ_PROJ_SPIN_LIMIT", 16384), 0, 1 << 24)};
-// the block the readers look at (room for rank 256) and the staging words behind it (stream_kernel.hpp)
-constexpr size_t kProjHandoverBytes = 2 * 256 * 8;
+// the block the readers look at and, 4096 bytes behind it, the staging words, each with room for rank 256
+// (stream_kernel.hpp)
+constexpr size_t kProjHandoverBytes = 4096 + 256 * 8;
 bool proj_in_launch(const GroupDev& g) {
   if (g.M != 1 || g_proj_in_launch.load(std::memory_order_relaxed) == 0) return false;
   if (g.ws == nullptr || (reinterpret_cast<uintptr_t>(g.ws) & 7u) != 0 || g.ws_bytes < kProjHandoverBytes) return false;
   if (g.rank > 256 || !proj_on_small_kernel(g.M, g.K, g.rank) || !aligned16(g.x) || !aligned16(g.R)) return false;
   bool any_left = false;
-  long blocks = 0;
-  for (int i = 0; i < g.n_members; ++i) {
-    any_left = any_left || g.mem[i].L != nullptr;
-    blocks += (g.mem[i].N + 1) / 2;
-  }
-  // Only launches whose waves (one per row block of two rows) are all on the chip at once.  A workgroup that is done
-  // before r is there waits for it; where a later workgroup waits for its place, that wait costs the launch what the
-  // projection launch in front would have.  Both ways, us per group launch, 8B shapes: q|k|v (3072 waves) 6.9 / 7.8,
-  // o_proj (2048) 6.1 / 6.9, down_proj (2048) 11.0 / 12.6, gate|up (14336) 16.1 to 16.6 / 15.9 to 16.5.
-  return any_left && (g_proj_in_launch.load(std::memory_order_relaxed) == 2 || blocks <= 16L * num_cus());
+  for (int i = 0; i < g.n_members; ++i) any_left = any_left || g.mem[i].L != nullptr;
+  return any_left;  // (the launcher still turns down a grid that is not on the chip all at once)
 }
 
 int pick_route(const GroupDev& g, int force) {
@@ -417,6 +410,15 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   note_launch(0, 0, 0, "%s", (route >= 0 && route <= kRouteSkinnyTiled) ? kRouteNames[route] : "?");  // launchers that know more overwrite it
   if (route == kRouteStream) {
     e = launch_stream(g, cus, stream);
+    if (e == hipErrorNotReady && g.pub != nullptr) {
+      // the grid with the producers of r in front does not fit the chip in one go: the projection launch after all
+      g.pub = nullptr;
+      e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
+      if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
+      g.r = g.r_out;
+      g.R = nullptr;
+      e = launch_stream(g, cus, stream);
+    }
   } else if (route == kRouteQStream) {
     e = launch_qstream(g, cus, stream);
   } else if (route == kRouteGemm) {

@@ -172,26 +172,36 @@ __device__ __forceinline__ void wait_words(u32x4 (&a)[kCount]) {
 
 // ---- the projection inside the launch (kProProj, single token) -----------------------------------------------------
 // r = R x is needed by every wave, but only for the last of its dot products.  Instead of a launch of its own in front
-// (2.4 to 3.4 us for 128 rows of R), the grid gets rank / waves workgroups in front that have no row block: each of
-// their waves computes one entry and hands it to everybody else through one 64-bit word per entry in device memory:
+// (2.4 to 3.4 us for 128 rows of R), the grid gets workgroups in front that have no row block: their waves compute the
+// entries of r and hand them to everybody else through one 64-bit word per entry in device memory:
 //     bits 48..63: the fp16 value,   bits 0..47: a tag that names this launch.
 // Value and tag travel in the one word, written and read with relaxed atomics of agent scope (they pass the caches that
 // are private to a part of the chip), so a reader that sees the tag has the value and no fence is needed.  The tag is
 // built from the dispatch id of the launch -- the position of its packet in the hardware queue, which a replay of a
 // captured graph renews like any other launch -- and from the address of that queue, with the top bit set so that
 // zeroed memory never matches.  Words left by earlier launches therefore never pass for this launch's, and nothing has
-// to be cleared between launches.  Readers take their word after their weights are consumed, by which time it has long
-// been written (measured on 1792 workgroups: no reader ever polled twice, +0.4 us per launch); a reader that does not
+// to be cleared between launches.  A reader looks at its word when the last of its weights are due; one that does not
 // find the tag polls a bounded number of times and then computes its entry itself, so every wave ends whatever the
 // order in which the workgroups were started.  Calls that share the words must not overlap.
-// The entries reach the readers in two steps.  A producer leaves its word in a staging area that only one wave reads:
-// the collector, which waits (bounded) until all entries of this launch are there and then writes the block the
-// readers look at, 512 contiguous bytes per store instruction.  Lines that thousands of readers fetch while 128
-// producers write them eight bytes at a time were measured to cost the launch 0.8 to 1.5 us (every write sends the
-// readers of all parts of the chip back to memory for the line); written once, whole, they cost nothing that shows.
+// The entries reach the readers in two steps.  A producer leaves its word in a staging area that only the collectors
+// read: the waves of one more workgroup in front, which poll it in turn (bounded) until all entries of this launch are
+// there; one of them then writes the block the readers look at, 512 contiguous bytes per store instruction.  Lines
+// that thousands of readers fetch while 128 producers write them eight bytes at a time were measured to cost the
+// launch 0.8 to 1.5 us (every write sends the readers of all parts of the chip back to memory for the line); written
+// once, whole, they cost nothing that shows.
+// What it buys is bounded by the hand-over itself: a row of R that no cache holds is there 2 to 2.5 us after the launch
+// began, and two hops through memory (producer to collector, collector to reader) add as much again, which is about as
+// long as the launch of a small group takes without it.  Per group launch of a 32-layer sequence, projection inside /
+// projection launch in front / r given: q|k|v of an 8B layer 7.1 / 7.5 / 5.1 us, o_proj 6.5 / 6.7 / 4.3, down_proj
+// 10.8 / 11.8 / 8.5.  (Tried on the way and slower: producers that also own a row block, or that publish straight
+// into the block; a first look right behind the barrier, with or without a pause in front of it; 2 to 256 copies of
+// the block for the readers to spread over.)
 extern "C" __device__ unsigned long long glowq_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
 constexpr unsigned long long kTagMask = 0xFFFFFFFFFFFFull;
-constexpr int kProjStaging = 256;  // the staging words lie behind room for the 256 entries of the largest rank
+// The staging words lie 4096 bytes behind the block, not right behind it: next to each other, the collectors' polls and
+// the readers' meet at the same place in memory (q|k|v of an 8B layer 7.45 us against 7.15).  (The lines of the block
+// themselves 4096 bytes apart, to spread the readers: 7.35.)
+constexpr int kProjStaging = 512;
 __device__ __forceinline__ unsigned long long launch_tag() {
   const unsigned long long q = (unsigned long long)reinterpret_cast<uintptr_t>(__builtin_amdgcn_queue_ptr());
   return (glowq_dispatch_id() & 0xFFFFFFFull) | (((q >> 8) & 0x7FFFFull) << 28) | (1ull << 47);
@@ -212,6 +222,12 @@ __host__ __device__ constexpr int proj_entries_per_wg(int words, int waves) { re
 // workgroups in front of the grid: those that produce r, and the collector's
 __host__ __device__ constexpr int proj_front_wgs(int words, int waves, int rank) {
   return (rank + proj_entries_per_wg(words, waves) - 1) / proj_entries_per_wg(words, waves) + 1;
+}
+// the grid of `readers` workgroups with row blocks and `front` in front: at the head of the grid they alternate in
+// fours (see the kernel), and a front padded to a multiple of four takes as many readers between it
+__host__ __device__ constexpr int proj_grid_wgs(int readers, int front) {
+  const int padded = (front + 3) & ~3;
+  return readers > padded ? padded + readers : 2 * padded;
 }
 
 // What a wave holds of one row block: kKit steps of two 16-byte units (32 codes of each row), and the side data.
@@ -341,12 +357,24 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
     tag = launch_tag();
     const int front = proj_front_wgs(words, waves, rank);
     unsigned long long* staging = ch.proj_pub + kProjStaging;
-    if (wg < front - 1) {
+    // Of each eight workgroups at the head of the grid the first four take a role in front, the other four are readers
+    // like the rest (proj_grid_wgs): workgroup i runs on part i mod 8 of the chip, and parts 4..7 were seen to start a
+    // launch 1.1 to 1.5 us behind parts 0..3 -- entries produced there kept every reader waiting.
+    const int zone = 2 * ((front + 3) & ~3);
+    int role = -1;
+    if (wg < zone) {
+      if ((wg & 7) < 4) role = (wg >> 3) * 4 + (wg & 3);
+      else wg = (wg >> 3) * 4 + (wg & 3);
+    } else {
+      wg -= zone >> 1;
+    }
+    if (role >= front) return;
+    if (role >= 0 && role < front - 1) {
       // the row of R first (up to eight pieces per lane in flight), then x into LDS in its natural order by the whole
       // workgroup while they travel
       const bool split = proj_split(words);
       const int epw = proj_entries_per_wg(words, waves);
-      const int j = __builtin_amdgcn_readfirstlane(wg * epw + (split ? wave >> 2 : wave));
+      const int j = __builtin_amdgcn_readfirstlane(role * epw + (split ? wave >> 2 : wave));
       const int q = split ? wave & 3 : 0;
       const bool active = j < rank && (!split || wave < 4 * epw);
       const int stride = split ? 256 : kWave, first = lane + kWave * q;
@@ -356,20 +384,23 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
       auto piece = [&](int w) { return *reinterpret_cast<const h8*>(Rb + ((uint32_t)min(w, words - 1) << 4)); };
       h8* xn = reinterpret_cast<h8*>(smem);
       float* pp = reinterpret_cast<float*>(smem + (size_t)K * sizeof(half_t));  // (split form: K > 8192, room for 16 floats)
-      h8 rv[8];
+      // (one batch holds a whole share of the longest row the kernel takes: 9 pieces per lane where four waves share an
+      // entry, which are the instantiations with registers to spare)
+      constexpr int kBatch = stream_heavy(kKit) ? 9 : 8;
+      h8 rv[kBatch];
 #pragma unroll
-      for (int b = 0; b < 8; ++b) rv[b] = piece(first + stride * b);
+      for (int b = 0; b < kBatch; ++b) rv[b] = piece(first + stride * b);
 #pragma unroll 1
       for (int w = (int)threadIdx.x; w < words; w += threads) xn[w] = reinterpret_cast<const h8*>(x)[w];
       __syncthreads();
       float acc = 0.f;
-      for (int b0 = 0; b0 < pieces; b0 += 8) {
+      for (int b0 = 0; b0 < pieces; b0 += kBatch) {
         if (b0 > 0) {
 #pragma unroll
-          for (int b = 0; b < 8; ++b) rv[b] = piece(first + stride * (b0 + b));
+          for (int b = 0; b < kBatch; ++b) rv[b] = piece(first + stride * (b0 + b));
         }
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < kBatch; ++b) {
           const int w = first + stride * (b0 + b);
           const float d = dot8(rv[b], xn[min(w, words - 1)]);
           acc = w < words ? acc + d : acc;
@@ -385,20 +416,26 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
         const half_t v = (half_t)total;
         ch.proj_r_out[j] = v;
         // (proj_mute: a test of the readers' own dot product -- the caller still gets r, the readers never do)
-        if (!(ch.proj_mute & 1))
+        if (!ch.proj_mute)
           __hip_atomic_store(staging + j, ((unsigned long long)__builtin_bit_cast(uint16_t, v) << 48) | tag, __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_AGENT);
       }
       return;
     }
-    if (wg == front - 1) {
-      if (wave != 0) return;
-      // the collector: lane l takes entries l, l + 64, ...; when every entry carries the tag, each store instruction
-      // below writes 512 contiguous bytes, whole lines.  (One wave only: four that polled in turn, to find the entries
-      // sooner, wrote the block more than once and cost the launch a microsecond.)
+    if (role == front - 1) {
+      // the collectors: the waves of this workgroup poll the staging words in turn, each a fraction of a round trip
+      // behind the one before, so that the last entry is noticed soon after it lands.  The first wave to find all
+      // entries of this launch claims the block through a flag in LDS and writes it -- once: a block written twice sends
+      // the readers back to memory for it twice.  Lane l takes entries l, l + 64, ...: each store instruction below
+      // writes 512 contiguous bytes, whole lines.
+      int* claimed = reinterpret_cast<int*>(smem);
+      if (threadIdx.x == 0) *claimed = 0;
+      __syncthreads();
+      for (int i = 0; i < wave; ++i) __builtin_amdgcn_s_sleep(6);
       unsigned long long w[4] = {0, 0, 0, 0};
       bool all = false;
       for (unsigned spins = 0; !all && spins <= ch.proj_spin; ++spins) {
+        if (*reinterpret_cast<volatile int*>(claimed) != 0) return;
         bool mine = true;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -408,16 +445,18 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
           }
         }
         all = __builtin_amdgcn_ballot_w64(!mine) == 0;
-        if (!all) __builtin_amdgcn_s_sleep(4);
       }
       if (all) {
+        int first = 0;
+        if (lane == 0) first = atomicCAS(claimed, 0, 1) == 0;
+        if (__builtin_amdgcn_readfirstlane(first)) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (lane + kWave * q < rank) __hip_atomic_store(ch.proj_pub + lane + kWave * q, w[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int q = 0; q < 4; ++q)
+            if (lane + kWave * q < rank) __hip_atomic_store(ch.proj_pub + lane + kWave * q, w[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
       return;  // (without all entries nothing is published: the readers run into their limit and compute r themselves)
     }
-    wg -= front;
   }
 
   // ---- activations first: their wait then does not cover the weight requests issued behind them
@@ -810,7 +849,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
         ++spins;
         w = __hip_atomic_load(ch.proj_pub + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         seen = (w & kTagMask) == tag;
-        if (!seen) __builtin_amdgcn_s_sleep(8);
+        if (!seen) __builtin_amdgcn_s_sleep(2);
       }
       half_t v = __builtin_bit_cast(half_t, (uint16_t)(w >> 48));
       if (!seen) {

@@ -140,7 +140,7 @@ class W4A16Extension:
 
     WORKSPACE_BYTES = 64 << 20
 
-    HANDOVER_BYTES = 4096
+    HANDOVER_BYTES = 8192
 
     def _workspace(self, dev: torch.device, rows: int):
         """(pointer, bytes) of the workspace of the current stream of `dev`: one per stream, because calls that share

@@ -209,9 +209,9 @@ def test_calls_that_cannot_hand_r_over_keep_the_projection_launch(ext):
                                                    m["L"].data_ptr(), yb.data_ptr())
         e.N, e.ldw_i32, e.lds, e.ldz_i32, e.ldy = N, m["qweight"].size(1), m["scales"].size(1), m["qzeros"].size(1), N
         ys.append(yb)
-    ws = torch.zeros(4096, dtype=torch.uint8, device="cuda")     # what the hand-over takes: 256 words and 256 staging words
+    ws = torch.zeros(6144, dtype=torch.uint8, device="cuda")     # what the hand-over takes: the block, and 4096 bytes behind it 256 staging words
     stream = ext._stream(xd.device)
-    for ws_bytes, want_in in ((4095, False), (4096, True), (0, False)):
+    for ws_bytes, want_in in ((6143, False), (6144, True), (0, False)):
         r = torch.empty((1, rank), dtype=torch.float16, device="cuda")
         rc = ext.lib.glowq_w4a16_group_forward_fused_ws(xd.data_ptr(), Rd.data_ptr(), r.data_ptr(), marr, n, 1, K, 128, rank, 1.0,
                                                         ws.data_ptr() if ws_bytes else None, ws_bytes, stream)
