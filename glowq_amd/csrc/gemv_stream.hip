@@ -36,6 +36,11 @@ bool stream_supported(const GroupDev& g) {
 
 namespace {
 
+int env_int_s(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : fallback;
+}
+
 // kPro: kProPlain, or kProProj where run_group left the projection to the launch (g.pub set, g.R still there)
 template <int kKit, int kLW, int kM, bool kPacked, int kPro = kProPlain>
 hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
@@ -68,7 +73,8 @@ hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
         resident.store(per_cu, std::memory_order_relaxed);
         resident_threads.store(waves * kWave, std::memory_order_relaxed);
       }
-      if (!g.pub_mute && (long)grid > (long)per_cu * num_cus()) return hipErrorNotReady;  // the caller launches the projection
+      static const int force = env_int_s("GLOWQ_PROJ_FORCE", 0);  // (for measurements: the form on every grid)
+      if (!force && !g.pub_mute && (long)grid > (long)per_cu * num_cus()) return hipErrorNotReady;  // the caller launches the projection
       ch.proj_R = g.R;
       ch.proj_r_out = g.r_out;
       ch.proj_pub = g.pub;
@@ -109,11 +115,6 @@ hipError_t launch_stream_lw(GroupDev& g, int waves, hipStream_t stream) {
   if (lw == 1) return launch_stream_m<kKit, 1>(g, waves, stream);
   if (lw == 2) return launch_stream_m<kKit, 2>(g, waves, stream);
   return hipErrorInvalidValue;  // ranks above 256 belong to the wave-dot GEMV (stream_supported)
-}
-
-int env_int_s(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return (v && *v) ? atoi(v) : fallback;
 }
 
 }  // namespace

@@ -412,10 +412,27 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
         __syncthreads();
         total = (pp[wave & ~3] + pp[(wave & ~3) + 1]) + (pp[(wave & ~3) + 2] + pp[(wave & ~3) + 3]);
       }
+      if (!split) {
+        // one wave per entry: the workgroup's entries meet in LDS and go straight into the block the readers look at,
+        // consecutive words in one store
+        float* mine = reinterpret_cast<float*>(smem);  // (over the head of x, which every wave is done with behind the barrier)
+        __syncthreads();
+        if (lane == 0) mine[wave] = total;
+        __syncthreads();
+        if (wave == 0 && lane < epw && role * epw + lane < rank) {
+          const half_t v = (half_t)mine[lane];
+          ch.proj_r_out[role * epw + lane] = v;
+          // (proj_mute: a test of the readers' own dot product -- the caller still gets r, the readers never do)
+          if (!ch.proj_mute)
+            __hip_atomic_store(ch.proj_pub + role * epw + lane, ((unsigned long long)__builtin_bit_cast(uint16_t, v) << 48) | tag,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+      }
+      // four waves per entry: through the staging words and the collectors
       if (active && q == 0 && lane == 0) {
         const half_t v = (half_t)total;
         ch.proj_r_out[j] = v;
-        // (proj_mute: a test of the readers' own dot product -- the caller still gets r, the readers never do)
         if (!ch.proj_mute)
           __hip_atomic_store(staging + j, ((unsigned long long)__builtin_bit_cast(uint16_t, v) << 48) | tag, __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_AGENT);
@@ -423,6 +440,7 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
       return;
     }
     if (role == front - 1) {
+      if (!proj_split(words)) return;  // (one wave per entry: the producers write the block themselves)
       // the collectors: the waves of this workgroup poll the staging words in turn, each a fraction of a round trip
       // behind the one before, so that the last entry is noticed soon after it lands.  The first wave to find all
       // entries of this launch claims the block through a flag in LDS and writes it -- once: a block written twice sends

@@ -158,7 +158,8 @@ int glowq_w4a16_group_forward(const void* x, const void* r, const glowq_member_t
 /*
  * Projection and group in one call: r_out = fp16(x R^T) ([M, rank], for the caller's group cache) followed by
  * the group launch that consumes it.  Replaces the whole body of `AddSVDCorrection.forward` for a group
- * (src/step3_eval_dataset.py:470-511) with one library call (two launches on `stream`).
+ * (src/step3_eval_dataset.py:470-511) with one library call (two launches on `stream`; one where the variant with a
+ * workspace below can compute r inside the group launch).
  */
 int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, const glowq_member_t* members,
                                     int n_members, int M, int K, int group_size, int rank, float alpha, void* stream);
@@ -170,6 +171,13 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
  * 4 * roundup(M, 128) * sum_i roundup(N_i, 256) bytes; the split goes as far as the workspace holds slices.
  * The skinny MFMA route (5..64 rows) splits K the same way where its column tiles cover half of the CUs or fewer and
  * K is 12288 columns or longer (down_proj): 4 * M * sum_i roundup(N_i, 32) bytes per slice, at most 8 slices.
+ * With a workspace of 6144 bytes or more, a fused call with one token row on the stream GEMV (route 5, ranks up to 256)
+ * computes r inside the group launch where the whole grid of that launch is on the chip at once: workgroups in front
+ * of the grid produce the entries of r, write them to r_out and hand them to the others through tagged words in the
+ * workspace (the first 6144 bytes; the tags name the launch, so the words need no clearing and a replay of a captured
+ * graph is a launch like any other).  One launch instead of two, the same bits in r_out and in the outputs as the
+ * projection launch in front gives; "proj_in_launch" of glowq_set_tuning switches it off.  As everywhere, calls that
+ * share a workspace must not overlap.
  */
 int glowq_w4a16_group_forward_ws(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
                                  int K, int group_size, int rank, float alpha, void* workspace, size_t workspace_bytes,
@@ -265,10 +273,14 @@ int glowq_probe_empty_launch(int grid, int block, void* stream);
  * "tiled_min_m" / "tiled_max_m" (default 5 / 64; max 0 switches the route off): token rows served by the kernel that
  * streams the tiled copy of the weights where every member brings one; "tiled_shape_rule" (0 / 1): up to 32 rows only
  * for groups whose stream is long enough to pay for its start-up (1, the default) or for every group (0).
+ * "proj_in_launch" (0 / 1, default 1): a fused single-token call with a workspace computes r inside the group launch
+ * where that applies (glowq_w4a16_group_forward_fused_ws); 2, for tests, keeps the producing waves from handing their
+ * entries over, so that every reader runs into "proj_spin_limit" (default 16384, 0 = never waits: the number of times
+ * a reader looks again for an entry of r that is not there yet before it computes the entry itself).
  * Returns the previous value (>= 0) or GLOWQ_EINVAL.  Initial values come from GLOWQ_QUAD_M,
  * GLOWQ_QUAD_MIN_M, GLOWQ_WAVEDOT_M, GLOWQ_SKINNY_M, GLOWQ_SMALL_GROUP_MB, GLOWQ_STREAM_M, GLOWQ_STREAM_SHAPE_RULE,
- * GLOWQ_QSTREAM_M, GLOWQ_QSTREAM_SHAPE_RULE, GLOWQ_SKINNY_CODES_M, GLOWQ_TILED_MIN_M, GLOWQ_TILED_MAX_M and
- * GLOWQ_TILED_SHAPE_RULE.
+ * GLOWQ_QSTREAM_M, GLOWQ_QSTREAM_SHAPE_RULE, GLOWQ_SKINNY_CODES_M, GLOWQ_TILED_MIN_M, GLOWQ_TILED_MAX_M,
+ * GLOWQ_TILED_SHAPE_RULE, GLOWQ_PROJ_IN_LAUNCH and GLOWQ_PROJ_SPIN_LIMIT.
  */
 int glowq_set_tuning(const char* key, int value);
 
