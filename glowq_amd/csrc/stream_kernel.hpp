@@ -183,19 +183,23 @@ __device__ __forceinline__ void wait_words(u32x4 (&a)[kCount]) {
 // to be cleared between launches.  A reader looks at its word when the last of its weights are due; one that does not
 // find the tag polls a bounded number of times and then computes its entry itself, so every wave ends whatever the
 // order in which the workgroups were started.  Calls that share the words must not overlap.
-// The entries reach the readers in two steps.  A producer leaves its word in a staging area that only the collectors
-// read: the waves of one more workgroup in front, which poll it in turn (bounded) until all entries of this launch are
-// there; one of them then writes the block the readers look at, 512 contiguous bytes per store instruction.  Lines
-// that thousands of readers fetch while 128 producers write them eight bytes at a time were measured to cost the
-// launch 0.8 to 1.5 us (every write sends the readers of all parts of the chip back to memory for the line); written
-// once, whole, they cost nothing that shows.
+// How the entries reach the block the readers look at depends on how many one workgroup produces.  With one wave per
+// entry (up to 8192 columns) a workgroup's entries meet in LDS and one store writes them into the block, consecutive
+// words.  With four waves per entry (longer rows: one or two entries per workgroup) a producer leaves its word in a
+// staging area that only the collectors read: the waves of one more workgroup in front, which poll it in turn
+// (bounded) until all entries of this launch are there; one of them then writes the block, 512 contiguous bytes per
+// store instruction.  What matters is how often a line of the block is written while thousands of readers fetch it:
+// every write sends the readers of all parts of the chip back to memory for the line.  128 producers writing eight
+// bytes each straight into the block cost the launch 0.8 to 1.5 us; sixteen or eight bytes per workgroup (the long rows)
+// were slower than the detour through the collectors (13.8 against 10.8 us); 32 bytes per workgroup are faster than
+// the detour (q|k|v 6.75 against 7.05 us, o_proj 6.2 against 6.7), which costs a round trip of its own.
 // What it buys is bounded by the hand-over itself: a row of R that no cache holds is there 2 to 2.5 us after the launch
-// began, and two hops through memory (producer to collector, collector to reader) add as much again, which is about as
-// long as the launch of a small group takes without it.  Per group launch of a 32-layer sequence, projection inside /
-// projection launch in front / r given: q|k|v of an 8B layer 7.1 / 7.5 / 5.1 us, o_proj 6.5 / 6.7 / 4.3, down_proj
-// 10.8 / 11.8 / 8.5.  (Tried on the way and slower: producers that also own a row block, or that publish straight
-// into the block; a first look right behind the barrier, with or without a pause in front of it; 2 to 256 copies of
-// the block for the readers to spread over.)
+// began, and each hop through memory adds half a microsecond or more, which together is about as long as the launch of
+// a small group takes without it.  Per group launch of a 32-layer sequence, projection inside / projection launch in
+// front / r given: q|k|v of an 8B layer 6.75 / 7.5 / 5.1 us, o_proj 6.3 / 6.7 / 4.3, down_proj 10.8 / 11.85 / 8.4; the
+// whole layer 39.15 against 40.6.  (Tried on the way and slower: producers that also own a row block; a first look
+// right behind the barrier, with or without a pause in front of it; 2 to 256 copies of the block for the readers to
+// spread over; the lines of the block 4096 bytes apart.)
 extern "C" __device__ unsigned long long glowq_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
 constexpr unsigned long long kTagMask = 0xFFFFFFFFFFFFull;
 // The staging words lie 4096 bytes behind the block, not right behind it: next to each other, the collectors' polls and
