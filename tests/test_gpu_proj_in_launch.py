@@ -221,3 +221,35 @@ def test_calls_that_cannot_hand_r_over_keep_the_projection_launch(ext):
         assert torch.equal(r, r_two), ws_bytes
         for a, b in zip(ys, y_two):
             assert torch.equal(a, b), ws_bytes
+
+
+def test_two_streams_with_their_own_words(ext):
+    """Two streams run launches of the same groups at the same time; each stream has its own hand-over words (the Python
+    layer keeps them per stream), so neither picks up the other's r.  Every result is the two-launch form's."""
+    K, Ns, rank = 4096, [768, 256], 128
+    _, members, R = make_group(61, 1, K, Ns, rank)
+    _, members_b, R_b = make_group(62, 1, K, Ns, rank)
+    mem, mem_b = members_on_device(members), members_on_device(members_b)
+    Rd, Rd_b = dev(R), dev(R_b)
+    g = torch.Generator().manual_seed(8)
+    xs = [torch.randn(1, K, generator=g).half().cuda() for _ in range(8)]
+    want = [(two_launch(ext, x, Rd, mem, 1.0), two_launch(ext, x, Rd_b, mem_b, 1.0)) for x in xs]
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got = []
+    for x in xs:
+        with torch.cuda.stream(s1):
+            r1 = torch.empty((1, rank), dtype=torch.float16, device="cuda")
+            y1 = ext.group_forward(x, r1, mem, 128, 1.0, R=Rd)
+            assert in_launch(ext)
+        with torch.cuda.stream(s2):
+            r2 = torch.empty((1, rank), dtype=torch.float16, device="cuda")
+            y2 = ext.group_forward(x, r2, mem_b, 128, 1.0, R=Rd_b)
+            assert in_launch(ext)
+        got.append(((r1, y1), (r2, y2)))
+    torch.cuda.synchronize()
+    for i, (w, h) in enumerate(zip(want, got)):
+        for (rw, yw), (rg, yg) in zip(w, h):
+            assert torch.equal(rw, rg), f"token {i}"
+            for a, b in zip(yw, yg):
+                assert torch.equal(a, b), f"token {i}"

@@ -356,6 +356,13 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     with pytest.raises(ValueError):
         ext.set_tuning("no_such_key", 1)
     assert ext.route(1, 100, 8) == "generic"
+    # the switch and the poll limit of the group launch that computes r itself: defaults, ranges, round trip
+    assert ext.set_tuning("proj_in_launch", 0) == 1 and ext.set_tuning("proj_in_launch", 2) == 0
+    assert ext.set_tuning("proj_in_launch", 1) == 2
+    assert ext.set_tuning("proj_spin_limit", 0) == 16384 and ext.set_tuning("proj_spin_limit", 16384) == 0
+    for key, bad in (("proj_in_launch", 3), ("proj_spin_limit", -1), ("proj_spin_limit", (1 << 24) + 1)):
+        with pytest.raises(ValueError):
+            ext.set_tuning(key, bad)
 
 
 def test_tensor_front_end_checks():
