@@ -66,12 +66,17 @@ hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
       // launch in front would have, and the workgroups in front take places of their own (the gate|up launch of an 8B
       // layer, 7 workgroups per compute unit: 16.1 to 16.6 us against 15.9 to 16.5; the down_proj launch of a 14B
       // layer, one workgroup per compute unit and two rounds as it is: 23.9 against 19.8).
-      static std::atomic<int> resident_threads{0}, resident{0};  // (per instantiation; a workgroup size gives one answer)
-      int per_cu = resident.load(std::memory_order_relaxed);
-      if (resident_threads.load(std::memory_order_relaxed) != waves * kWave || per_cu == 0) {
+      // (asked once per instantiation, workgroup size and LDS size; the last answer is kept)
+      static std::atomic<long> asked_for{-1};
+      static std::atomic<int> resident{0};
+      const long shape = (long)lds * 4096 + waves * kWave;
+      int per_cu = 0;
+      if (asked_for.load(std::memory_order_acquire) == shape) {
+        per_cu = resident.load(std::memory_order_relaxed);
+      } else {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), waves * kWave, lds) != hipSuccess) per_cu = 0;
         resident.store(per_cu, std::memory_order_relaxed);
-        resident_threads.store(waves * kWave, std::memory_order_relaxed);
+        asked_for.store(shape, std::memory_order_release);
       }
       static const int force = env_int_s("GLOWQ_PROJ_FORCE", 0);  // (for measurements: the form on every grid)
       if (!force && !g.pub_mute && (long)grid > (long)per_cu * num_cus()) return hipErrorNotReady;  // the caller launches the projection
