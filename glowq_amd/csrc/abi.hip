@@ -336,6 +336,19 @@ bool proj_in_launch(const GroupDev& g) {
   return any_left;  // (the launcher still turns down a grid that is not on the chip all at once)
 }
 
+// The same for the skinny kernel at 5..32 token rows (skinny.hip): the head of the workspace takes the hand-over words,
+// and the producers in front compute r in the arithmetic of the small projection kernels.
+constexpr size_t kSkinnyHandoverBytes = (size_t)(512 + 512) * 8;
+bool skinny_proj_in_launch(const GroupDev& g) {
+  if (g.M < 2 || g.M > 32 || g_proj_in_launch.load(std::memory_order_relaxed) == 0) return false;
+  if (g.ws == nullptr || (reinterpret_cast<uintptr_t>(g.ws) & 15u) != 0 || g.ws_bytes < kSkinnyHandoverBytes) return false;
+  if (!proj_on_small_kernel(g.M, g.K, g.rank) || (g.K & 255) != 0 || (g.rank & 7) != 0 || !aligned16(g.x) || !aligned16(g.R)) return false;
+  if ((reinterpret_cast<uintptr_t>(g.r_out) & 15u) != 0) return false;
+  bool any_left = false;
+  for (int i = 0; i < g.n_members; ++i) any_left = any_left || g.mem[i].L != nullptr;
+  return any_left;  // (the launcher still turns down shapes and grids it does not take)
+}
+
 int pick_route(const GroupDev& g, int force) {
   if (force < 0 && g.M >= g_tiled_min_m.load(std::memory_order_relaxed) && g.M <= g_tiled_max_m.load(std::memory_order_relaxed) &&
       skinny_tiled_supported(g) && tiled_pays(g))
@@ -382,23 +395,30 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
   const int cus = num_cus();
   hipError_t e = hipSuccess;
   g.pub = nullptr;
-  if (g.R != nullptr && route == kRouteStream && proj_in_launch(g)) {
-    // single token on the stream GEMV: the first waves of the group launch produce r and hand it to the others through
-    // the workspace (stream_kernel.hpp), no launch in front
+  // r = x R^T ahead of the group as a launch of its own.  (Having every workgroup of the group kernel compute r for
+  // itself was measured: the R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra
+  // launch costs.)
+  const auto launch_projection = [&]() -> hipError_t {
+    hipError_t pe;
+    if (!proj_on_small_kernel(g.M, g.K, g.rank) && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
+      pe = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream, g.ws, g.ws_bytes);
+    else
+      pe = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
+    g.r = g.r_out;
+    g.R = nullptr;
+    g.pub = nullptr;
+    return pe;
+  };
+  const bool skinny_route = route == kRouteSkinny || route == kRouteSkinnyRaw;
+  if (g.R != nullptr && ((route == kRouteStream && proj_in_launch(g)) || (skinny_route && skinny_proj_in_launch(g)))) {
+    // single token on the stream GEMV, a handful of rows on the skinny kernel: workgroups in front of the group launch
+    // produce r and hand it to the others through the workspace (stream_kernel.hpp, skinny.hip), no launch in front
     g.pub = static_cast<unsigned long long*>(g.ws);
     g.pub_spin = (unsigned)g_proj_spin_limit.load(std::memory_order_relaxed);
     g.pub_mute = g_proj_in_launch.load(std::memory_order_relaxed) == 2;
   } else if (g.R != nullptr) {
-    // r = x R^T goes ahead as a launch of its own.  (Having every workgroup of the group kernel compute r for itself
-    // was measured: the R -> r -> L.r dependency chain then stalls the weight stream for longer than the extra launch
-    // costs.)
-    if (!proj_on_small_kernel(g.M, g.K, g.rank) && (g.K & 63) == 0 && aligned16(g.x) && aligned16(g.R))
-      e = launch_shared_proj_mfma(g.x, g.R, g.r_out, g.M, g.K, g.rank, cus, stream, g.ws, g.ws_bytes);
-    else
-      e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
+    e = launch_projection();
     if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
-    g.r = g.r_out;
-    g.R = nullptr;
   }
   // side streams are used only where every member brings one packed for the rank this launch applies
   bool packed = true;
@@ -412,11 +432,8 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     e = launch_stream(g, cus, stream);
     if (e == hipErrorNotReady && g.pub != nullptr) {
       // the grid with the producers of r in front does not fit the chip in one go: the projection launch after all
-      g.pub = nullptr;
-      e = launch_shared_proj_small(g.x, g.R, g.r_out, g.M, g.K, g.rank, stream);
+      e = launch_projection();
       if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
-      g.r = g.r_out;
-      g.R = nullptr;
       e = launch_stream(g, cus, stream);
     }
   } else if (route == kRouteQStream) {
@@ -425,8 +442,13 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     e = launch_gemm(g, cus, stream);
   } else if (route == kRouteSkinnyTiled) {
     e = launch_skinny_tiled(g, cus, stream);
-  } else if (route == kRouteSkinny || route == kRouteSkinnyRaw) {
+  } else if (skinny_route) {
     e = launch_skinny(g, cus, stream, route == kRouteSkinnyRaw);
+    if (e == hipErrorNotReady && g.pub != nullptr) {
+      e = launch_projection();
+      if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
+      e = launch_skinny(g, cus, stream, route == kRouteSkinnyRaw);
+    }
   } else {
     const int cap = (route == kRouteWaveDot) ? kWaveDotMaxM
                     : (route == kRouteQuad) ? quad_capacity(g.M, g.K, g.rank, g.r != nullptr) : 65535;
@@ -766,7 +788,8 @@ int glowq_w4a16_group_forward_fused_static(const void* x, const void* R, void* r
   // what the users of the workspace ask for at this shape: the projection's split of K, the skinny kernel's and that of
   // the kernel that streams the tiled copy (each states its own bound next to its split rule)
   size_t need = (M > 0 && K > 0 && rank > 0) ? proj_workspace_bytes(M, K, rank, num_cus()) : 0;
-  need = std::max(need, glowq::skinny_split_workspace_bytes(M, num_cus()));
+  // (the skinny kernel that computes r itself keeps its hand-over words in front of the partial tiles)
+  need = std::max(need, glowq::skinny_split_workspace_bytes(M, num_cus()) + (M >= 2 && M <= 32 ? kSkinnyHandoverBytes : 0));
   bool any_tiled = false;
   for (int i = 0; members != nullptr && i < n_members && i < GLOWQ_MAX_MEMBERS; ++i) any_tiled = any_tiled || members[i].tiled != nullptr;
   if (any_tiled) need = std::max(need, glowq::tiled_split_workspace_bytes(M, num_cus()));

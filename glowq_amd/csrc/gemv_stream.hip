@@ -60,7 +60,7 @@ hipError_t launch_stream_p(GroupDev& g, int waves, hipStream_t stream) {
     }
     ChainDev ch{};
     if constexpr (kProj) {
-      grid = proj_grid_wgs(grid, proj_front_wgs(g.K >> 3, waves, g.rank));  // with the workgroups that produce r, and the collector's
+      grid = front_grid(grid, proj_front_wgs(g.K >> 3, waves, g.rank));  // with the workgroups that produce r, and the collector's
       // Only where every workgroup of the launch is on the chip at once.  A workgroup that is done before r is there
       // waits for it; where a later workgroup waits for its place, that wait costs the launch what the projection
       // launch in front would have, and the workgroups in front take places of their own (the gate|up launch of an 8B

@@ -3,6 +3,7 @@
 #include <cstdlib>
 
 #include "common.hpp"
+#include "proj_block.hpp"
 #include "side_stream.hpp"
 
 namespace glowq {
@@ -151,65 +152,9 @@ __global__ __launch_bounds__(256) void shared_proj_kernel(const half_t* __restri
 template <int kM, int kJ>
 __global__ __launch_bounds__(256) void shared_proj_block_kernel(const half_t* __restrict__ x, const half_t* __restrict__ R,
                                                                 half_t* __restrict__ r, int M, int K, int rank) {
-  __shared__ float part[4][kM * kJ];
-  const int j0 = blockIdx.x * kJ;
-  const int m0 = blockIdx.y * kM;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
-  float acc[kM][kJ];
-#pragma unroll
-  for (int m = 0; m < kM; ++m)
-#pragma unroll
-    for (int j = 0; j < kJ; ++j) acc[m][j] = 0.f;
-  const int words = K >> 3;
-  constexpr int kBatch = (kM + kJ) > 8 ? 1 : 2;  // all loads of a batch are issued before the first is used
-  const h8* xrow[kM];
-  const h8* rrow[kJ];
-#pragma unroll
-  for (int m = 0; m < kM; ++m) xrow[m] = reinterpret_cast<const h8*>(x + (size_t)min(m0 + m, M - 1) * K);
-#pragma unroll
-  for (int j = 0; j < kJ; ++j) rrow[j] = reinterpret_cast<const h8*>(R + (size_t)min(j0 + j, rank - 1) * K);
-  for (int w0 = threadIdx.x; w0 < words; w0 += kBatch * blockDim.x) {
-    h8 rv[kJ][kBatch], xv[kM][kBatch];
-    float live[kBatch];
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b) {
-      const int w = w0 + b * blockDim.x;
-      live[b] = w < words ? 1.f : 0.f;
-      const int wc = min(w, words - 1);
-#pragma unroll
-      for (int j = 0; j < kJ; ++j) rv[j][b] = rrow[j][wc];
-#pragma unroll
-      for (int m = 0; m < kM; ++m) xv[m][b] = xrow[m][wc];
-    }
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b)
-#pragma unroll
-      for (int m = 0; m < kM; ++m)
-#pragma unroll
-        for (int j = 0; j < kJ; ++j) {
-          float d = 0.f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            d = __builtin_amdgcn_fdot2(h2{rv[j][b][2 * i], rv[j][b][2 * i + 1]}, h2{xv[m][b][2 * i], xv[m][b][2 * i + 1]}, d, false);
-          acc[m][j] = __builtin_fmaf(live[b], d, acc[m][j]);
-        }
-  }
-#pragma unroll
-  for (int m = 0; m < kM; ++m)
-#pragma unroll
-    for (int j = 0; j < kJ; ++j) {
-      const float v = wave_sum(acc[m][j]);
-      if (lane == 0) part[wave][m * kJ + j] = v;
-    }
-  __syncthreads();
-  if (threadIdx.x < kM * kJ) {
-    const int m = m0 + (int)threadIdx.x / kJ, j = j0 + (int)threadIdx.x % kJ;
-    if (m < M && j < rank) {
-      const int t = threadIdx.x;
-      r[(size_t)m * rank + j] = (half_t)((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
-    }
-  }
+  __shared__ float part[4 * kM * kJ];
+  proj_block_body<kM, kJ>(x, R, M, K, rank, (int)blockIdx.x * kJ, (int)blockIdx.y * kM, part,
+                          [&](int m, int j, float v) { r[(size_t)m * rank + j] = (half_t)v; });
 }
 
 // Single token row, K up to 512 kP and a multiple of 8: one wave per row of R, up to kP 16-byte pieces of R and of x per

@@ -12,9 +12,12 @@
 //     kNT >= 2 every A fragment feeds two MFMAs, which keeps the L1 traffic per weight byte low enough.
 // The correction is a K-extension in front: the ceil(rank/64) blocks of [r | L] are dealt to the waves first,
 // acc *= alpha, then the weight blocks accumulate on top.  The waves' partial tiles meet in LDS once.
+#include <atomic>
 #include <cstdlib>
 
 #include "common.hpp"
+#include "handover.hpp"
+#include "proj_block.hpp"
 
 namespace glowq {
 
@@ -40,7 +43,18 @@ struct SkinnyArgs {
   // tile in `partials` ([slice][workgroup][M][32 kNT]) and skinny_reduce_kernel adds the slices in order
   int slices;
   float* partials;
+  // second form, where the launch computes r = x R^T itself (kProj): workgroups in front of the grid produce blocks of
+  // four token rows by four rows of R and write them to r_out, the others apply the correction behind their weights
+  // instead of in front of them and read r_out once the word `pub[0]` says that all of it is there
+  const half_t* R;          // [rank, K]
+  half_t* r_out;            // [M, rank]
+  unsigned long long* pub;  // [0]: the ready word; [kSkinnyFlags + p]: the flag of producer p
+  unsigned spin;            // polls of the ready word before a wave computes its part of r itself
+  int producers;            // workgroups that produce r
 };
+constexpr int kSkinnyFlags = 512;          // the producers' flags lie 4096 bytes behind the ready word
+constexpr int kSkinnyMaxProducers = 512;
+constexpr size_t kSkinnyHandoverBytes = (size_t)(kSkinnyFlags + kSkinnyMaxProducers) * 8;
 
 __device__ __forceinline__ h8 nibble_order(const u32x4& v) {
   // halves (0..7) -> (0,4,1,5,2,6,3,7): two byte permutes per output dword
@@ -283,7 +297,14 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
 // code * x, and scale and zero-point are applied to that sum, y += s (sum c x - z sum x), with the fp32 sums of x per
 // token row and group taken when the activations are staged.  Five vector instructions per code word instead of
 // thirteen, and the arithmetic of the GEMV routes: weights never rounded to fp16.
-template <int kMT, int kNT, bool kBulk, bool kRaw>
+// kProj: the launch computes r = x R^T itself (SkinnyArgs).  The grid then has producers + 1 workgroups in front (roles
+// dealt as in handover.hpp).  Producer p takes the blocks p, p + producers, ... of four token rows by four rows of R with
+// its first four waves, in the arithmetic of shared_proj_block_kernel, writes them to r_out with stores that pass the caches private to a part of the
+// chip, waits until they are acknowledged and raises its flag (the launch's tag); the collector polls the flags
+// (bounded) and, when all are up, writes the ready word.  A wave with a correction block polls the ready word (bounded)
+// once its weights are done, then reads its part of r with loads that pass those caches as well; a wave that never sees
+// the word computes the part of r it needs itself, so every wave ends whatever becomes of the producers.
+template <int kMT, int kNT, bool kBulk, bool kRaw, bool kProj = false>
 __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63;
@@ -291,10 +312,64 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   const int waves = blockDim.x >> 6;
   const int ln = lane & 31, lh = lane >> 5;
 
+  int wg = (int)blockIdx.x;
+  const int tiles = g.blk_end[g.n_members - 1];  // workgroups with a column tile (per slice)
+  unsigned long long tag = 0;
+  if constexpr (kProj) {
+    tag = launch_tag();
+    const int front = g.producers + 1;
+    const int role = front_role(wg, front);
+    if (role >= 0) {
+      if (role >= front || blockIdx.y != 0) return;
+      if (role < g.producers) {
+        if (threadIdx.x >= 256) return;  // (the body's barriers count the waves that arrive)
+        float* part = reinterpret_cast<float*>(smem);
+        float* vals = part + 4 * 16;
+        const int jblocks = (g.rank + 3) >> 2, nblocks = jblocks * ((g.M + 3) >> 2);
+        // blocks of four token rows by four rows of R, dealt round robin to the producers
+        for (int b = role; b < nblocks; b += g.producers) {
+          const int bj = b % jblocks, bm = b / jblocks;
+          proj_block_body<4, 4>(g.x, g.R, g.M, g.K, g.rank, 4 * bj, 4 * bm, part,
+                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; });
+          __syncthreads();
+          // pairs of neighbouring entries of a token row go out as one 32-bit store (ranks are multiples of 8)
+          if (threadIdx.x < 8) {
+            const int mi = (int)threadIdx.x >> 1, pp = (int)threadIdx.x & 1;
+            const int m = 4 * bm + mi, j = 4 * bj + 2 * pp;
+            if (m < g.M && j < g.rank) {
+              const h2 v = {(half_t)vals[mi * 4 + 2 * pp], (half_t)vals[mi * 4 + 2 * pp + 1]};
+              __hip_atomic_store(reinterpret_cast<uint32_t*>(g.r_out + (size_t)m * g.rank + j), __builtin_bit_cast(uint32_t, v),
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+          __syncthreads();  // (part and vals are free for the next block)
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are acknowledged: r is where every reader looks
+        __syncthreads();
+        if (threadIdx.x == 0 && g.spin != 0xFFFFFFFFu)  // (that value: a test in which the flags never go up)
+          __hip_atomic_store(g.pub + kSkinnyFlags + role, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+      }
+      // the collector: one wave, lane l takes flags l, l + 64, ...
+      if (wave != 0) return;
+      bool all = false;
+      for (unsigned spins = 0; !all && spins <= g.spin && g.spin != 0xFFFFFFFFu; ++spins) {
+        bool mine = true;
+        for (int p = lane; p < g.producers; p += 64)
+          mine = mine && (__hip_atomic_load(g.pub + kSkinnyFlags + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kTagMask) == tag;
+        all = __builtin_amdgcn_ballot_w64(!mine) == 0;
+        if (!all) __builtin_amdgcn_s_sleep(2);
+      }
+      if (all && lane == 0) __hip_atomic_store(g.pub, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (wg >= tiles) return;  // (a front larger than the grid behind it leaves places between its workgroups empty)
+  }
+
   SkinnyMember mem = g.mem[0];
   int blk_base = 0;
 #define GLOWQ_PICK(i)                                          \
-  if (g.n_members > i && (int)blockIdx.x >= g.blk_end[i - 1]) { \
+  if (g.n_members > i && wg >= g.blk_end[i - 1]) {             \
     mem = g.mem[i];                                            \
     blk_base = g.blk_end[i - 1];                               \
   }
@@ -302,7 +377,7 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   GLOWQ_PICK(2)
   GLOWQ_PICK(3)
 #undef GLOWQ_PICK
-  const int n0 = ((int)blockIdx.x - blk_base) * (32 * kNT);
+  const int n0 = (wg - blk_base) * (32 * kNT);
 
   int ncol[kNT];
 #pragma unroll
@@ -327,11 +402,12 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   unsigned char* atile = smem + (size_t)wave * (kATile + kBTile + kSig);
   unsigned char* btile = atile + kATile;
   float* asig = reinterpret_cast<float*>(btile + kBTile);
-  const bool corrected = mem.L != nullptr && g.r != nullptr && blockIdx.y == 0;  // the first slice carries the correction
-  if (corrected) {
-    // A 64-column block of [r | L] reaches the operands like the weights below: its 128-byte row segments are loaded in
-    // memory order, 8 lanes per segment, into the wave's LDS tiles and read back in MFMA lane order.
-    const int lblocks = (g.rank + 63) >> 6;  // ranks are multiples of 8: the last block may be partial
+  const bool corrected = mem.L != nullptr && (kProj || g.r != nullptr) && blockIdx.y == 0;  // the first slice carries the correction
+  const int lblocks = (g.rank + 63) >> 6;  // ranks are multiples of 8: the last block may be partial
+  // A 64-column block of [r | L] reaches the operands like the weights below: its 128-byte row segments are loaded in
+  // memory order, 8 lanes per segment, into the wave's LDS tiles and read back in MFMA lane order.
+  // r_there (kProj): r_out holds r; else the lane computes the octets of r it would have loaded (fp32, column order).
+  auto correction = [&](const bool r_there) {
     for (int jb = wave; jb < lblocks; jb += waves) {
       // octets past the rank: r counts as zero there, L is read from the row's last octet (finite values)
       const int k = jb * 64 + (lane & 7) * 8;
@@ -340,7 +416,28 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
       u32x4 lreg[kNT * 4], rreg[kMT * 4];
 #pragma unroll
       for (int q = 0; q < kMT * 4; ++q) {
-        rreg[q] = *reinterpret_cast<const u32x4*>(g.r + (size_t)min(q * 8 + (lane >> 3), g.M - 1) * g.rank + kc);
+        const int m = min(q * 8 + (lane >> 3), g.M - 1);
+        if constexpr (kProj) {
+          if (r_there) {
+            // (64-bit loads of agent scope: they pass the caches that the producers' stores passed)
+            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(g.r_out + (size_t)m * g.rank + kc);
+            const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            rreg[q] = u32x4{(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+          } else {
+            h8 own;
+            for (int e = 0; e < 8; ++e) {
+              const half_t* Rrow = g.R + (size_t)(kc + e) * g.K;
+              const half_t* xrow = g.x + (size_t)m * g.K;
+              float a = 0.f;
+              for (int kk = 0; kk < g.K; ++kk) a = __builtin_fmaf((float)Rrow[kk], (float)xrow[kk], a);
+              own[e] = (half_t)a;
+            }
+            rreg[q] = __builtin_bit_cast(u32x4, own);
+          }
+        } else {
+          rreg[q] = *reinterpret_cast<const u32x4*>(g.r + (size_t)m * g.rank + kc);
+        }
         if (!live) rreg[q] = u32x4{0u, 0u, 0u, 0u};
       }
 #pragma unroll
@@ -371,13 +468,19 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
         }
       }
     }
-    if (g.alpha != 1.0f) {
+  };
+  const auto scale_acc = [&](const float f) {
 #pragma unroll
-      for (int tm = 0; tm < kMT; ++tm)
+    for (int tm = 0; tm < kMT; ++tm)
 #pragma unroll
-        for (int tn = 0; tn < kNT; ++tn)
+      for (int tn = 0; tn < kNT; ++tn)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= g.alpha;
+        for (int i = 0; i < 16; ++i) acc[tm][tn][i] *= f;
+  };
+  if constexpr (!kProj) {
+    if (corrected) {
+      correction(true);
+      if (g.alpha != 1.0f) scale_acc(g.alpha);
     }
   }
 
@@ -638,6 +741,22 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     if constexpr (kRaw) compute_raw(1); else { compute(i, 2); compute(i, 3); }
   }
 #undef GLOWQ_PIN_LOADS
+  if constexpr (kProj) {
+    // the correction behind the weights: acc_w + alpha (r . L^T) = alpha (acc_w / alpha + r . L^T)
+    if (corrected && wave < lblocks) {
+      int seen = 0;
+      if (lane == 0) {
+        for (unsigned spins = 0; !seen && spins <= g.spin && g.spin != 0xFFFFFFFFu; ++spins) {
+          seen = (__hip_atomic_load(g.pub, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kTagMask) == tag;
+          if (!seen) __builtin_amdgcn_s_sleep(2);
+        }
+      }
+      seen = __builtin_amdgcn_readfirstlane(seen);
+      if (g.alpha != 1.0f) scale_acc(1.0f / g.alpha);
+      correction(seen != 0);
+      if (g.alpha != 1.0f) scale_acc(g.alpha);
+    }
+  }
   __syncthreads();  // the reduction buffer below overlays the staging tiles
 
   // ---- the waves' partial tiles meet in LDS: [wave][tm][tn][16 regs][64 lanes] floats; only registers and slots of
@@ -663,7 +782,7 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
     for (int w = 0; w < waves; ++w) v += red[(size_t)w * kTile + at];
     const int n = n0 + col;
     if (g.slices > 1) {
-      g.partials[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * g.M + m) * (32 * kNT) + col] = v;
+      g.partials[(((size_t)blockIdx.y * tiles + wg) * g.M + m) * (32 * kNT) + col] = v;
     } else if (n < mem.N) {
       const float b = mem.bias ? (float)mem.bias[n] : 0.f;
       mem.y[(size_t)m * mem.ldy + n] = (half_t)(v + b);
@@ -745,9 +864,10 @@ static bool skinny_bulk_runs(const SkinnyArgs& a, int waves) {
 // ws_bytes: room behind a.partials (0: none).  The second form cuts K into slices through it where the column tiles
 // alone leave half of the CUs or more without a workgroup and every wave still keeps three super-blocks and more
 // (4096 outputs of K = 14336: 128 workgroups -> 2 x 128; 8 rows 16.6 -> about 14.5 us, 64 rows 41 -> about 28).
-template <int kMT, int kNT, bool kGroupForm, bool kRaw = false>
+template <int kMT, int kNT, bool kGroupForm, bool kRaw = false, bool kProj = false>
 static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t ws_bytes, hipStream_t stream) {
   static_assert(kGroupForm || !kRaw, "the raw-code form is a variant of the second form");
+  static_assert(kGroupForm || !kProj, "only the second form computes r itself");
   int total = 0;
   for (int i = 0; i < a.n_members; ++i) {
     total += (a.mem[i].N + 32 * kNT - 1) / (32 * kNT);
@@ -766,13 +886,46 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
   }
   const bool bulk = kGroupForm && skinny_bulk_runs(a, waves);
   auto kern = !kGroupForm ? skinny_mfma_kernel<kMT, kNT>
-              : bulk ? skinny_group_kernel<kMT, kNT, true, kRaw> : skinny_group_kernel<kMT, kNT, false, kRaw>;
+              : bulk ? skinny_group_kernel<kMT, kNT, true, kRaw, kProj> : skinny_group_kernel<kMT, kNT, false, kRaw, kProj>;
   size_t lds = (size_t)waves * kMT * kNT * 16 * 64 * sizeof(float);
   const size_t staging = (size_t)waves * ((kMT * 64 + kNT * 32) * 144 + (kRaw ? kMT * 32 * sizeof(float) : 0));
   if (kGroupForm && lds < staging) lds = staging;
   static LdsLimit lds_limit[2];  // one per kernel this site launches
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit[bulk]); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(total, a.slices), dim3(waves * 64), lds, stream, a);
+  int grid_x = total;
+  if constexpr (kProj) {
+    static std::atomic<long> asked_for[2] = {{-1}, {-1}};
+    static std::atomic<int> resident[2] = {{0}, {0}};
+    const long shape = (long)lds * 4096 + waves * 64;
+    int per_cu = 0;
+    if (asked_for[bulk].load(std::memory_order_acquire) == shape) {
+      per_cu = resident[bulk].load(std::memory_order_relaxed);
+    } else {
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), waves * 64, lds) != hipSuccess) per_cu = 0;
+      resident[bulk].store(per_cu, std::memory_order_relaxed);
+      asked_for[bulk].store(shape, std::memory_order_release);
+    }
+    // The workgroups in front take the places the launch leaves free on the chip (its staging tiles allow one workgroup
+    // per compute unit), and only where those are enough for about one block of r per producer: every workgroup
+    // of the launch then starts at once, the producers are done long before the first wave asks for r, and no workgroup
+    // with a column tile waits for a place (one that does adds its whole run time to the launch: q|k|v of an 8B layer at
+    // eight rows with 257 workgroups for 256 places 11.25 us against 11.05 with the projection launch in front; fewer
+    // producers with more blocks each: down_proj 32 us against 19).
+    const long capacity = (long)per_cu * num_cus;
+    long want = ((capacity - (long)total * a.slices) & ~3L) - 1;  // (the front is padded to a multiple of four: handover.hpp)
+    static const int env_producers = getenv("GLOWQ_SKINNY_PRODUCERS") ? atoi(getenv("GLOWQ_SKINNY_PRODUCERS")) : 0;
+    if (env_producers > 0) want = env_producers;
+    const int nblocks = ((a.rank + 3) / 4) * ((a.M + 3) / 4);  // blocks of r: four token rows by four rows of R
+    if (want > nblocks) want = nblocks;
+    if (want > kSkinnyMaxProducers) want = kSkinnyMaxProducers;
+    // (a few producers with two blocks are as far as it goes: 4 x 8 blocks, two to a producer, on o_proj of a 14B layer
+    // at 16 rows: 16.4 us against 14.3 with the projection launch)
+    if (want < 1 || (9 * want < 8 * nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
+    a.producers = (int)want;
+    grid_x = front_grid(total, a.producers + 1);
+  }
+  hipLaunchKernelGGL(kern, dim3(grid_x, a.slices), dim3(waves * 64), lds, stream, a);
+  if constexpr (kProj) note_launch(grid_x, a.slices, waves * 64, "skinny_group_kernel<%d,%d,%d,%d,1>", kMT, kNT, (int)bulk, (int)kRaw);
   if (hipError_t e = hipGetLastError(); e != hipSuccess || a.slices == 1) return e;
   hipLaunchKernelGGL(skinny_reduce_kernel<kNT>, dim3(total), dim3(256), 0, stream, a);
   return hipGetLastError();
@@ -796,7 +949,21 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw)
   a.slices = 1;
   const bool ws_ok = g.ws != nullptr && (reinterpret_cast<uintptr_t>(g.ws) & 15u) == 0;
   a.partials = ws_ok ? static_cast<float*>(g.ws) : nullptr;
-  const size_t ws_bytes = ws_ok ? g.ws_bytes : 0;
+  size_t ws_bytes = ws_ok ? g.ws_bytes : 0;
+  // the launch computes r itself (run_group set g.pub to the head of the workspace): the partial tiles lie behind the
+  // hand-over words
+  const bool proj = g.pub != nullptr;
+  a.R = g.R;
+  a.r_out = g.r_out;
+  a.pub = g.pub;
+  a.spin = g.pub_mute ? 0xFFFFFFFFu : g.pub_spin;
+  a.producers = 0;
+  if (proj) {
+    if (!ws_ok || ws_bytes < kSkinnyHandoverBytes) return hipErrorNotReady;
+    a.r = nullptr;
+    a.partials = reinterpret_cast<float*>(static_cast<unsigned char*>(g.ws) + kSkinnyHandoverBytes);
+    ws_bytes -= kSkinnyHandoverBytes;
+  }
   for (int i = 0; i < g.n_members; ++i) {
     const MemberDev& m = g.mem[i];
     SkinnyMember& s = a.mem[i];
@@ -823,6 +990,12 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw)
     if (env_waves < 1) waves = wide ? 4 : (g.M <= 32 ? 8 : 6);  // staging tiles: 18 / 13.5 / 22.5 KB of LDS per wave
     if (waves > (g.K >> 8)) waves = g.K >> 8;
     if (raw && !skinny_raw_form(g)) return hipErrorInvalidValue;
+    if (proj) {
+      // (the narrow tile at up to 32 rows, four waves and more: the shapes whose launch leaves room on the chip)
+      if (g.M > 32 || wide || waves < 4) return hipErrorNotReady;
+      return raw ? launch_skinny_t<1, 1, true, true, true>(a, waves, num_cus, ws_bytes, stream)
+                 : launch_skinny_t<1, 1, true, false, true>(a, waves, num_cus, ws_bytes, stream);
+    }
     if (g.M <= 32) {
       if (raw) return wide ? launch_skinny_t<1, 2, true, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true, true>(a, waves, num_cus, ws_bytes, stream);
       return wide ? launch_skinny_t<1, 2, true>(a, waves, num_cus, ws_bytes, stream) : launch_skinny_t<1, 1, true>(a, waves, num_cus, ws_bytes, stream);
@@ -845,6 +1018,7 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw)
     return hipSuccess;
   }
   if (raw) return hipErrorInvalidValue;
+  if (proj) return hipErrorNotReady;
   const int kblocks = g.K >> 6;
   if (waves > kblocks) waves = kblocks;
   if (g.M <= 32) return launch_skinny_t<1, 2, false>(a, waves, num_cus, ws_bytes, stream);

@@ -22,6 +22,7 @@
 #include <utility>
 
 #include "common.hpp"
+#include "handover.hpp"
 #include "side_stream.hpp"
 
 namespace glowq {
@@ -200,17 +201,10 @@ __device__ __forceinline__ void wait_words(u32x4 (&a)[kCount]) {
 // whole layer 39.15 against 40.6.  (Tried on the way and slower: producers that also own a row block; a first look
 // right behind the barrier, with or without a pause in front of it; 2 to 256 copies of the block for the readers to
 // spread over; the lines of the block 4096 bytes apart.)
-extern "C" __device__ unsigned long long glowq_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
-constexpr unsigned long long kTagMask = 0xFFFFFFFFFFFFull;
 // The staging words lie 4096 bytes behind the block, not right behind it: next to each other, the collectors' polls and
 // the readers' meet at the same place in memory (q|k|v of an 8B layer 7.45 us against 7.15).  (The lines of the block
 // themselves 4096 bytes apart, to spread the readers: 7.35.)
 constexpr int kProjStaging = 512;
-__device__ __forceinline__ unsigned long long launch_tag() {
-  const unsigned long long q = (unsigned long long)reinterpret_cast<uintptr_t>(__builtin_amdgcn_queue_ptr());
-  return (glowq_dispatch_id() & 0xFFFFFFFull) | (((q >> 8) & 0x7FFFFull) << 28) | (1ull << 47);
-}
-
 __device__ __forceinline__ float dot8(const h8& a, const h8& c) {
   float d = 0.f;
 #pragma unroll
@@ -226,12 +220,6 @@ __host__ __device__ constexpr int proj_entries_per_wg(int words, int waves) { re
 // workgroups in front of the grid: those that produce r, and the collector's
 __host__ __device__ constexpr int proj_front_wgs(int words, int waves, int rank) {
   return (rank + proj_entries_per_wg(words, waves) - 1) / proj_entries_per_wg(words, waves) + 1;
-}
-// the grid of `readers` workgroups with row blocks and `front` in front: at the head of the grid they alternate in
-// fours (see the kernel), and a front padded to a multiple of four takes as many readers between it
-__host__ __device__ constexpr int proj_grid_wgs(int readers, int front) {
-  const int padded = (front + 3) & ~3;
-  return readers > padded ? padded + readers : 2 * padded;
 }
 
 // What a wave holds of one row block: kKit steps of two 16-byte units (32 codes of each row), and the side data.
@@ -361,17 +349,8 @@ void gemv_stream_kernel(const half_t* __restrict__ x, const half_t* __restrict__
     tag = launch_tag();
     const int front = proj_front_wgs(words, waves, rank);
     unsigned long long* staging = ch.proj_pub + kProjStaging;
-    // Of each eight workgroups at the head of the grid the first four take a role in front, the other four are readers
-    // like the rest (proj_grid_wgs): workgroup i runs on part i mod 8 of the chip, and parts 4..7 were seen to start a
-    // launch 1.1 to 1.5 us behind parts 0..3 -- entries produced there kept every reader waiting.
-    const int zone = 2 * ((front + 3) & ~3);
-    int role = -1;
-    if (wg < zone) {
-      if ((wg & 7) < 4) role = (wg >> 3) * 4 + (wg & 3);
-      else wg = (wg >> 3) * 4 + (wg & 3);
-    } else {
-      wg -= zone >> 1;
-    }
+    // (roles in front go to the workgroup indices that start first: handover.hpp)
+    const int role = front_role(wg, front);
     if (role >= front) return;
     if (role >= 0 && role < front - 1) {
       // the row of R first (up to eight pieces per lane in flight), then x into LDS in its natural order by the whole

@@ -253,3 +253,97 @@ def test_two_streams_with_their_own_words(ext):
             assert torch.equal(rw, rg), f"token {i}"
             for a, b in zip(yw, yg):
                 assert torch.equal(a, b), f"token {i}"
+
+
+# ---- the skinny kernel at a handful of token rows ----------------------------------------------------------------------
+# (M, K, member rows, rank, alpha): the raw-code form (up to 8 rows) and the dequantising form, one and two column-tile
+# members, a member without L, K slices through the workspace (few column tiles, long K), rank 256, a scale on the
+# correction
+SKINNY_CASES = [(8, 4096, [1024, 256, 256], 128, 1.0), (16, 5120, [640, 320], 128, 1.0), (8, 5120, [640, 320], 256, 1.0), (5, 1024, [96, 64], 64, 0.5),
+                (8, 14336, [512], 128, 1.0), (12, 2048, [200], 32, 2.0), (32, 4096, [512, 128], 128, 1.0)]
+
+
+def skinny_in_launch(ext) -> bool:
+    return ext.last_launch()["kernel"].startswith("skinny_group_kernel<") and ext.last_launch()["kernel"].endswith(",1>")
+
+
+@pytest.fixture
+def skinny_routes(ext):
+    """The skinny kernel on the canonical buffers serves these launches (not the kernel that streams the tiled copy)."""
+    with tuning(ext, tiled_max_m=0):
+        yield
+
+
+@pytest.mark.parametrize("M,K,Ns,rank,alpha", SKINNY_CASES)
+def test_skinny_kernel_computes_r_itself(ext, skinny_routes, M, K, Ns, rank, alpha):
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(70 + M + K + rank, M, K, Ns, rank, with_bias=True)
+    mem = members_on_device(members, drop_left=1 if len(Ns) > 1 else None, with_bias=True)
+    xd, Rd = dev(x), dev(R)
+    with tuning(ext, proj_in_launch=0):
+        r_two = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+        y_two = ext.group_forward(xd, r_two, mem, 128, alpha, R=Rd)
+        assert not skinny_in_launch(ext)
+    for rep in range(3):
+        r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        y = ext.group_forward(xd, r, mem, 128, alpha, R=Rd)
+        assert skinny_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+        assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, f"r, launch {rep}")
+        for i, (m, got) in enumerate(zip(members, y)):
+            want = (oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128) if mem[i]["L"] is None else
+                    oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha))
+            assert_close(got.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"member {i}, launch {rep}")
+            # and next to the two-launch form: the same weights' sums, the correction added behind instead of in front
+            assert np.abs(got.float().cpu().numpy() - y_two[i].float().cpu().numpy()).max() <= 4e-3 * max(1.0, float(np.abs(want).max()))
+
+
+def test_skinny_launches_and_replays_see_their_own_r(ext, skinny_routes):
+    """Launch after launch and replay after replay through the same workspace, each with other activations."""
+    M, K, Ns, rank = 8, 4096, [768, 256], 128
+    _, members, R = make_group(81, M, K, Ns, rank)
+    mem = members_on_device(members)
+    Rd = dev(R)
+    g = torch.Generator().manual_seed(9)
+    xs = torch.randn(M, K, generator=g).half().cuda()
+    r = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+        assert skinny_in_launch(ext)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+            again = ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+        assert skinny_in_launch(ext)
+    torch.cuda.synchronize()
+    for rep in range(5):
+        xs.copy_(torch.randn(M, K, generator=g).half())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        xn = xs.cpu().numpy()
+        assert_close(r.cpu().numpy(), xn.astype(np.float64) @ R.astype(np.float64).T, f"r, replay {rep}")
+        for m, a, b in zip(members, outs, again):
+            want = oracle.corrected_linear_exact(xn, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0)
+            assert_close(a.cpu().numpy(), want, f"replay {rep}")
+            assert torch.equal(a, b), f"replay {rep}: two launches of one replay"
+
+
+def test_skinny_waves_that_never_see_the_ready_word(ext, skinny_routes):
+    """With the producers' flags held down no wave ever sees the ready word: each computes the part of r it needs
+    itself; the caller still gets r from the producers."""
+    M, K, Ns, rank = 6, 1024, [96, 32], 64
+    x, members, R = make_group(91, M, K, Ns, rank)
+    mem = members_on_device(members)
+    xd, Rd = dev(x), dev(R)
+    with tuning(ext, proj_in_launch=2):
+        r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        y = ext.group_forward(xd, r, mem, 128, 1.0, R=Rd)
+        assert skinny_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+    assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
+    for m, got in zip(members, y):
+        assert_close(got.cpu().numpy(), oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0), "own r")
