@@ -11,7 +11,8 @@
 //     most and lives in L2), permuted in registers into the order the nibble masks deliver the codes.  With
 //     kNT >= 2 every A fragment feeds two MFMAs, which keeps the L1 traffic per weight byte low enough.
 // The correction is a K-extension in front: the ceil(rank/64) blocks of [r | L] are dealt to the waves first,
-// acc *= alpha, then the weight blocks accumulate on top.  The waves' partial tiles meet in LDS once.
+// acc *= alpha, then the weight blocks accumulate on top.  The waves' partial tiles meet in LDS once.  (Where the launch
+// computes r itself -- the second form's kProj -- the correction comes behind the weights instead.)
 #include <atomic>
 #include <cstdlib>
 
