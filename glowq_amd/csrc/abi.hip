@@ -410,7 +410,7 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     return pe;
   };
   const bool skinny_route = route == kRouteSkinny || route == kRouteSkinnyRaw;
-  if (g.R != nullptr && ((route == kRouteStream && proj_in_launch(g)) || (skinny_route && skinny_proj_in_launch(g)))) {
+  if (g.R != nullptr && ((route == kRouteStream && proj_in_launch(g)) || ((skinny_route || route == kRouteSkinnyTiled) && skinny_proj_in_launch(g)))) {
     // single token on the stream GEMV, a handful of rows on the skinny kernel: workgroups in front of the group launch
     // produce r and hand it to the others through the workspace (stream_kernel.hpp, skinny.hip), no launch in front
     g.pub = static_cast<unsigned long long*>(g.ws);
@@ -442,6 +442,11 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     e = launch_gemm(g, cus, stream);
   } else if (route == kRouteSkinnyTiled) {
     e = launch_skinny_tiled(g, cus, stream);
+    if (e == hipErrorNotReady && g.pub != nullptr) {
+      e = launch_projection();
+      if (e != hipSuccess) return fail(GLOWQ_ELAUNCH, "shared_proj launch failed: %s", hipGetErrorString(e));
+      e = launch_skinny_tiled(g, cus, stream);
+    }
   } else if (skinny_route) {
     e = launch_skinny(g, cus, stream, route == kRouteSkinnyRaw);
     if (e == hipErrorNotReady && g.pub != nullptr) {

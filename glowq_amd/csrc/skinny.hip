@@ -883,6 +883,10 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
     if (s > 8) s = 8;
     const size_t per_slice = (size_t)total * a.M * (32 * kNT) * sizeof(float);
     if (per_slice > 0 && (size_t)s > ws_bytes / per_slice) s = (int)(ws_bytes / per_slice);
+    // (a launch that computes r itself is not cut in two: the workgroups a second slice would bring are worth less than
+    // the projection launch and the reduction launch together -- down_proj of an 8B layer, 128 column tiles, two slices
+    // with both launches 20.6 us at 8 rows and 23.9 at 16, one slice with 64 / 127 producers in front 18.5 and 21.1)
+    if (kProj && s == 2) s = 1;
     if (s >= 2) a.slices = s;
   }
   const bool bulk = kGroupForm && skinny_bulk_runs(a, waves);

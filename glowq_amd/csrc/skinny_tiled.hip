@@ -29,14 +29,24 @@
 // The correction is a K-extension behind the weights: in the last rotation the sets are refilled with the blocks of
 // the tiled left factor (fp16, already in B-operand order), r follows the last super-block through the stages, and
 // acc += alpha * (r . L^T) from an accumulator of its own.
+// kProj: the launch computes r = x R^T itself.  Workgroups in front of the grid (roles dealt as in handover.hpp) produce
+// blocks of four token rows by four rows of R in the arithmetic of shared_proj_block_kernel and write them to r_out with
+// stores that pass the caches private to a part of the chip, each raises its flag when its stores are acknowledged, a
+// collector turns the flags into one ready word.  The producer waves of the other workgroups look for that word when
+// they are about to send r through the stages -- during the last super-block, so the producers in front have the whole
+// weight stream to get there -- and read r with loads that pass those caches; one that does not see the word within its
+// bound computes the pieces of r it would have loaded, so every wave ends whatever becomes of the workgroups in front.
 // Few column tiles (o_proj, down_proj): K is also cut into gridDim.y slices, each workgroup leaves its fp32 tile in the
 // caller's workspace and skinny_tiled_reduce_kernel adds the slices in order.  More than 32 token rows: two row tiles
 // per wave, every code word feeds two matrix instructions.
+#include <atomic>
 #include <cstdlib>
 
 #include <type_traits>
 
 #include "common.hpp"
+#include "handover.hpp"
+#include "proj_block.hpp"
 #include "tiled.hpp"
 
 namespace glowq {
@@ -62,7 +72,20 @@ struct TileArgs {
   int ldp;
   int tiles;        // column tiles of the whole group: the grid's x extent
   int cw;           // consumer waves per K group: a tile is 32 cw columns
+  // kProj (the launch computes r itself; `r` then points at r_out)
+  const half_t* R;          // [rank, K]
+  half_t* r_out;            // [M, rank]
+  unsigned long long* pub;  // [0]: the ready word; [kTiledFlags + p]: the flag of producer p
+  unsigned spin;            // polls of the ready word before a producer wave computes its pieces of r itself
+  int producers;            // workgroups in front that produce r
 };
+constexpr int kTiledFlags = 512;  // the producers' flags lie 4096 bytes behind the ready word
+constexpr int kTiledMaxProducers = 512;
+constexpr size_t kTiledHandoverBytes = (size_t)(kTiledFlags + kTiledMaxProducers) * 8;
+// blocks of r a producer in front may have to compute (gate|up of a 14B layer, rank 256, 35 producers: 3.7 blocks each at
+// eight rows 26.8 us against 30.9 with the projection launch, 5.5 at twelve 27.4 against 31.3, 7.3 at sixteen 30.5 to 31.5
+// against 31.5)
+constexpr int kTiledProjBlocks = 6;
 
 namespace {
 
@@ -116,7 +139,7 @@ __device__ unsigned long long g_tstamps[65536 * 32];
 constexpr int tiled_max_cw(int rows, int wk, int pw) { return wk > 1 ? 4 : (rows > 32 ? 8 - pw : 12 - pw); }
 constexpr int tiled_max_threads(int rows, int wk, int pw) { return (tiled_max_cw(rows, wk, pw) + pw) * 64 * wk; }
 
-template <int kRows, int kWk, int kPW>
+template <int kRows, int kWk, int kPW, bool kProj = false>
 __global__ __launch_bounds__(tiled_max_threads(kRows, kWk, kPW))
 void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K, const int slices,
                          const unsigned char* __restrict__ wt0, const int blk_end0, const int N0, const int cw, const TileArgs g) {
@@ -138,7 +161,62 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
   unsigned char* smem = smem_all + gk * 2 * kStage;
   GLOWQ_STAMP(0);
 
-  const int tile = (int)blockIdx.x;
+  int tile = (int)blockIdx.x;
+  unsigned long long tag = 0;
+  if constexpr (kProj) {
+    tag = launch_tag();
+    const int front = g.producers + 1;
+    const int role = front_role(tile, front);
+    if (role >= 0) {
+      if (role >= front || blockIdx.y != 0) return;
+      if (role < g.producers) {
+        if (threadIdx.x >= 256) return;  // (the body's barriers count the waves that arrive)
+        float* part = reinterpret_cast<float*>(smem_all);
+        const int jblocks = (g.rank + 3) >> 2;
+        float* vals = part + 4 * 16;
+        const int nblocks = jblocks * ((M + 3) >> 2);
+        // blocks of four token rows by four rows of R, dealt round robin to the producers.  (Blocks of eight token rows,
+        // half as many: 21.5 against 20.1 us at 12 rows on gate|up of an 8B layer, 32.0 against 27.5 on a 14B layer's;
+        // three 16-byte pieces of every row in flight per thread instead of two, a row of 5120 columns in one round trip:
+        // no difference.)
+        for (int b = role; b < nblocks; b += g.producers) {
+          const int bj = b % jblocks, bm = b / jblocks;
+          proj_block_body<4, 4>(x, g.R, M, K, g.rank, 4 * bj, 4 * bm, part,
+                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; });
+          __syncthreads();
+          // pairs of neighbouring entries of a token row go out as one 32-bit store (ranks are multiples of 8)
+          if (threadIdx.x < 8) {
+            const int mi = (int)threadIdx.x >> 1, pp = (int)threadIdx.x & 1;
+            const int m = 4 * bm + mi, j = 4 * bj + 2 * pp;
+            if (m < M && j < g.rank) {
+              const h2 v = {(half_t)vals[mi * 4 + 2 * pp], (half_t)vals[mi * 4 + 2 * pp + 1]};
+              __hip_atomic_store(reinterpret_cast<uint32_t*>(g.r_out + (size_t)m * g.rank + j), __builtin_bit_cast(uint32_t, v),
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+          __syncthreads();  // (part and vals are free for the next block)
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are acknowledged: r is where every reader looks
+        __syncthreads();
+        if (threadIdx.x == 0 && g.spin != 0xFFFFFFFFu)  // (that value: a test in which the flags never go up)
+          __hip_atomic_store(g.pub + kTiledFlags + role, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+      }
+      // the collector: one wave, lane l takes flags l, l + 64, ...
+      if (threadIdx.x >= 64) return;
+      bool all = false;
+      for (unsigned spins = 0; !all && spins <= g.spin && g.spin != 0xFFFFFFFFu; ++spins) {
+        bool mine = true;
+        for (int p = (int)threadIdx.x; p < g.producers; p += 64)
+          mine = mine && (__hip_atomic_load(g.pub + kTiledFlags + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kTagMask) == tag;
+        all = __builtin_amdgcn_ballot_w64(!mine) == 0;
+        if (!all) __builtin_amdgcn_s_sleep(2);
+      }
+      if (all && threadIdx.x == 0) __hip_atomic_store(g.pub, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (tile >= g.tiles) return;  // (a front larger than the grid behind it leaves places between its workgroups empty)
+  }
   const int SB = K >> 8;
   // The workgroup's super-blocks (slice blockIdx.y of K) are dealt to its K groups in contiguous parts of `pg`; every
   // group runs the same number of steps, a whole number of rotations of the register sets.  Steps past the end of a
@@ -204,15 +282,67 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
         }
       }
     };
+    // kProj: the first 256 columns of r from r_out once the ready word is up (loads that pass the caches the producers'
+    // stores passed); without the word within the bound, the thread computes the eight entries of each of its pieces
+    // `polls`: how often the wave looks before it gives up (one look where it may come back later).  True: the loads
+    // are out.
+    auto ask_r_handed = [&](unsigned polls) __attribute__((always_inline)) -> bool {
+      int seen = 0;
+      if (lane == 0) {
+        for (unsigned spins = 0; !seen && spins < polls && g.spin != 0xFFFFFFFFu; ++spins) {
+          seen = (__hip_atomic_load(g.pub, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & kTagMask) == tag;
+          if (!seen && spins + 1 < polls) __builtin_amdgcn_s_sleep(2);
+        }
+      }
+      seen = __builtin_amdgcn_readfirstlane(seen);
+      if (seen) {
+#pragma unroll
+        for (int q = 0; q < kPQ; ++q) {
+          const uint32_t row = (uint32_t)min(2 * kPW * q + prow, M - 1);
+          av[q] = __builtin_amdgcn_raw_buffer_load_b128(rs_r, (int)((row * (uint32_t)g.rank + (uint32_t)pcol * 8u) * 2u), 0, 16);
+        }
+      }
+      return seen != 0;
+    };
+    auto load_r_handed = [&]() __attribute__((always_inline)) {
+      if (ask_r_handed(g.spin == 0xFFFFFFFFu ? 0u : g.spin + 1u)) return;
+      for (int q = 0; q < kPQ; ++q) {
+        const int row = min(2 * kPW * q + prow, M - 1);
+        h8 own;
+        for (int e = 0; e < 8; ++e) {
+          const int j = pcol * 8 + e;
+          float a = 0.f;
+          if (j < g.rank) {
+            const half_t* Rrow = g.R + (size_t)j * K;
+            const half_t* xrow = x + (size_t)row * K;
+            for (int kk = 0; kk < K; ++kk) a = __builtin_fmaf((float)Rrow[kk], (float)xrow[kk], a);
+          }
+          own[e] = (half_t)a;
+        }
+        av[q] = __builtin_bit_cast(u32x4, own);
+      }
+    };
     load_a(false, min(sb0, SB - 1));
     store_a(0);
     load_a(false, min(sb0 + 1, SB - 1));
     __syncthreads();
+    bool have_r = false;
     for (int i = 0; i < steps; ++i) {
 #if !(GLOWQ_TDBG & 8)
+      if constexpr (kProj) {
+        // r that was not there a step earlier is waited for during the last super-block, for the stage that super-block
+        // does not read
+        if (i + 1 == steps && wg_corr && gk == 0 && !have_r) load_r_handed();
+      }
       store_a((i + 1) & 1);                                   // step i + 1's activations (or r after the last step)
       const bool next_r = i + 2 >= steps;
-      load_a(next_r, next_r ? 0 : min(sb0 + i + 2, SB - 1));  // (past the last step: r once more, never stored)
+      if constexpr (kProj) {
+        if (!next_r) load_a(false, min(sb0 + i + 2, SB - 1));
+        // where the other form asks for r, one look: as a rule the workgroups in front are long done
+        else if (i + 2 == steps && wg_corr && gk == 0) have_r = ask_r_handed(1u);
+      } else {
+        load_a(next_r, next_r ? 0 : min(sb0 + i + 2, SB - 1));  // (past the last step: r once more, never stored)
+      }
 #endif
       __syncthreads();
     }
@@ -650,9 +780,9 @@ static TiledPlan tiled_plan(const GroupDev& g, int num_cus, size_t ws_bytes) {
 // groups have tiles of four consumer waves (128 columns): one 128-column fp32 tile per token row for each of them.
 size_t tiled_split_workspace_bytes(int M, int num_cus) { return M > 4 ? (size_t)num_cus * (size_t)M * 128 * sizeof(float) : 0; }
 
-template <int kRows, int kWk, int kPW>
-static hipError_t launch_tiled_t(const TileArgs& a, const half_t* x, hipStream_t stream) {
-  auto kern = skinny_tiled_kernel<kRows, kWk, kPW>;
+template <int kRows, int kWk, int kPW, bool kProj = false>
+static hipError_t launch_tiled_t(TileArgs& a, const half_t* x, int num_cus, hipStream_t stream) {
+  auto kern = skinny_tiled_kernel<kRows, kWk, kPW, kProj>;
   constexpr int kMT = kRows > 32 ? 2 : 1;
   size_t lds = (size_t)kWk * 2 * (kRows * kRowBytes + 2 * kRows * 16);
   const size_t red = (size_t)(kWk - 1) * a.cw * kMT * 16 * 64 * sizeof(float);
@@ -660,9 +790,43 @@ static hipError_t launch_tiled_t(const TileArgs& a, const half_t* x, hipStream_t
   static LdsLimit lds_limit;
   if (hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, lds_limit); e != hipSuccess) return e;
   if (a.cw < 1 || a.cw > tiled_max_cw(kRows, kWk, kPW)) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(kern, dim3(a.tiles, a.slices), dim3((a.cw + kPW) * 64 * kWk), lds, stream, x, a.M, a.K, a.slices, a.mem[0].wt,
+  const int threads = (a.cw + kPW) * 64 * kWk;
+  int grid_x = a.tiles;
+  if constexpr (kProj) {
+    // The workgroups in front take places the launch leaves free on the chip, so that every workgroup starts at once and
+    // none with a column tile waits behind a producer.  The readers ask for r during their last super-block, so a
+    // producer has most of the launch for its blocks: up to `per_producer` of them (GLOWQ_TILED_PROJ_BLOCKS).
+    static std::atomic<long> asked_for{-1};
+    static std::atomic<int> resident{0};
+    const long shape = (long)lds * 4096 + threads;
+    int per_cu = 0;
+    if (asked_for.load(std::memory_order_acquire) == shape) {
+      per_cu = resident.load(std::memory_order_relaxed);
+    } else {
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), threads, lds) != hipSuccess) per_cu = 0;
+      resident.store(per_cu, std::memory_order_relaxed);
+      asked_for.store(shape, std::memory_order_release);
+    }
+    static const int env_blocks = getenv("GLOWQ_TILED_PROJ_BLOCKS") ? atoi(getenv("GLOWQ_TILED_PROJ_BLOCKS")) : 0;
+    static const int env_producers = getenv("GLOWQ_TILED_PRODUCERS") ? atoi(getenv("GLOWQ_TILED_PRODUCERS")) : 0;
+    const int per_producer = env_blocks > 0 ? env_blocks : kTiledProjBlocks;
+    // (one workgroup per compute unit, whatever the occupancy allows: two that share a compute unit share its LDS
+    // bandwidth and matrix cores, and the launch gets longer -- gate|up of a 14B layer at eight rows with 131 producers
+    // beside 218 tiles 42 us against 30.5)
+    const long capacity = per_cu >= 1 ? num_cus : 0;
+    long want = ((capacity - (long)a.tiles) & ~3L) - 1;  // (the front is padded to a multiple of four: handover.hpp)
+    if (env_producers > 0) want = env_producers;
+    const int nblocks = ((a.rank + 3) / 4) * ((a.M + 3) / 4);  // blocks of r: four token rows by four rows of R
+    if (want > nblocks) want = nblocks;
+    if (want > kTiledMaxProducers) want = kTiledMaxProducers;
+    if (threads < 256 || want < 1 || ((long)per_producer * want < nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
+    a.producers = (int)want;
+    grid_x = front_grid(a.tiles, a.producers + 1);
+  }
+  hipLaunchKernelGGL(kern, dim3(grid_x, a.slices), dim3(threads), lds, stream, x, a.M, a.K, a.slices, a.mem[0].wt,
                      a.blk_end[0], a.mem[0].N, a.cw, a);
-  note_launch(a.tiles, a.slices, (a.cw + kPW) * 64 * kWk, "skinny_tiled_kernel<%d,%d,%d> with %d consumer waves", kRows, kWk, kPW, a.cw);
+  note_launch(grid_x, a.slices, threads, kProj ? "skinny_tiled_kernel<%d,%d,%d,1> with %d consumer waves" : "skinny_tiled_kernel<%d,%d,%d> with %d consumer waves",
+              kRows, kWk, kPW, a.cw);
   if (hipError_t e = hipGetLastError(); e != hipSuccess || a.slices == 1) return e;
   hipLaunchKernelGGL(skinny_tiled_reduce_kernel, dim3((a.ldp / 4 + 255) / 256, a.M), dim3(256), 0, stream, a);
   return hipGetLastError();
@@ -671,6 +835,19 @@ static hipError_t launch_tiled_t(const TileArgs& a, const half_t* x, hipStream_t
 hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream) {
   TileArgs a;
   a.r = g.r;
+  // the launch computes r itself (run_group set g.pub to the head of the workspace): up to 16 token rows and rank 256 (r
+  // goes through the stages in one pass), K whole, nothing else in the workspace (no slices)
+  const bool proj = g.pub != nullptr;
+  a.R = g.R;
+  a.r_out = g.r_out;
+  a.pub = g.pub;
+  a.spin = g.pub_mute ? 0xFFFFFFFFu : g.pub_spin;
+  a.producers = 0;
+  if (proj) {
+    if (g.M > 16 || g.rank > 256 || (g.rank & 7) != 0 || (g.K & 7) != 0 || g.R == nullptr || g.r_out == nullptr || g.ws_bytes < kTiledHandoverBytes)
+      return hipErrorNotReady;
+    a.r = g.r_out;
+  }
   a.n_members = g.n_members;
   a.M = g.M;
   a.K = g.K;
@@ -686,7 +863,7 @@ hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream) {
     const MemberDev& m = g.mem[i];
     TileMember& t = a.mem[i];
     t.wt = static_cast<const unsigned char*>(m.tiled);
-    t.lt = (m.L != nullptr && g.r != nullptr) ? static_cast<const unsigned char*>(m.tiled_L) : nullptr;
+    t.lt = (m.L != nullptr && (g.r != nullptr || proj)) ? static_cast<const unsigned char*>(m.tiled_L) : nullptr;
     t.bias = m.bias;
     t.y = m.y;
     t.N = m.N;
@@ -700,17 +877,27 @@ hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream) {
   a.tiles = tiles;
   a.ldp = col;
   const int key = (g.M <= 8 ? 8 : g.M <= 16 ? 16 : g.M <= 32 ? 32 : 64) * 100 + plan.wk * 10 + plan.pw;
+  if (proj) {
+    if (a.slices != 1) return hipErrorNotReady;
+    switch (key) {
+      case 821: return launch_tiled_t<8, 2, 1, true>(a, g.x, num_cus, stream);
+      case 811: return launch_tiled_t<8, 1, 1, true>(a, g.x, num_cus, stream);
+      case 1622: return launch_tiled_t<16, 2, 2, true>(a, g.x, num_cus, stream);
+      case 1612: return launch_tiled_t<16, 1, 2, true>(a, g.x, num_cus, stream);
+    }
+    return hipErrorNotReady;
+  }
   switch (key) {
-    case 821: return launch_tiled_t<8, 2, 1>(a, g.x, stream);
-    case 811: return launch_tiled_t<8, 1, 1>(a, g.x, stream);
-    case 1622: return launch_tiled_t<16, 2, 2>(a, g.x, stream);
-    case 1612: return launch_tiled_t<16, 1, 2>(a, g.x, stream);
-    case 3222: return launch_tiled_t<32, 2, 2>(a, g.x, stream);
-    case 3212: return launch_tiled_t<32, 1, 2>(a, g.x, stream);
-    case 3214: return launch_tiled_t<32, 1, 4>(a, g.x, stream);
-    case 6412: return launch_tiled_t<64, 1, 2>(a, g.x, stream);
-    case 6413: return launch_tiled_t<64, 1, 3>(a, g.x, stream);
-    case 6414: return launch_tiled_t<64, 1, 4>(a, g.x, stream);
+    case 821: return launch_tiled_t<8, 2, 1>(a, g.x, num_cus, stream);
+    case 811: return launch_tiled_t<8, 1, 1>(a, g.x, num_cus, stream);
+    case 1622: return launch_tiled_t<16, 2, 2>(a, g.x, num_cus, stream);
+    case 1612: return launch_tiled_t<16, 1, 2>(a, g.x, num_cus, stream);
+    case 3222: return launch_tiled_t<32, 2, 2>(a, g.x, num_cus, stream);
+    case 3212: return launch_tiled_t<32, 1, 2>(a, g.x, num_cus, stream);
+    case 3214: return launch_tiled_t<32, 1, 4>(a, g.x, num_cus, stream);
+    case 6412: return launch_tiled_t<64, 1, 2>(a, g.x, num_cus, stream);
+    case 6413: return launch_tiled_t<64, 1, 3>(a, g.x, num_cus, stream);
+    case 6414: return launch_tiled_t<64, 1, 4>(a, g.x, num_cus, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -2,6 +2,8 @@
 the grid produce the entries, the others pick them up through tagged words in the caller's workspace.  The results have
 to be the bits of the two-launch form (projection launch in front, group launch on the r it left), on every launch and
 every replay of a captured graph, whatever the words still hold from earlier launches."""
+import re
+
 import numpy as np
 import pytest
 import torch
@@ -347,3 +349,116 @@ def test_skinny_waves_that_never_see_the_ready_word(ext, skinny_routes):
     assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
     for m, got in zip(members, y):
         assert_close(got.cpu().numpy(), oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0), "own r")
+
+
+# ---- the kernel that streams the tiled copy (5..16 token rows, groups whose column tiles fill the chip without K slices) ----
+# (M, K, member rows, rank, alpha): one and two K groups per workgroup (K of four super-blocks / eight and more), one to
+# three members with a ragged last tile, a member without L, rank 256, a scale on the correction
+TILED_CASES = [(8, 1024, [12288, 4608], 64, 1.0), (5, 2048, [16640], 128, 1.0), (12, 1024, [9000, 9000], 32, 2.0),
+               (16, 2048, [20000], 256, 1.0), (9, 4096, [8192, 8192, 1000], 128, 0.5)]
+
+
+def tiled_in_launch(ext) -> bool:
+    return re.match(r"skinny_tiled_kernel<\d+,\d+,\d+,1> ", ext.last_launch()["kernel"]) is not None
+
+
+@pytest.fixture
+def tiled_routes(ext):
+    """The kernel that streams the tiled copy serves these launches whatever the length of the stream."""
+    with tuning(ext, tiled_shape_rule=0):
+        yield
+
+
+@pytest.mark.parametrize("M,K,Ns,rank,alpha", TILED_CASES)
+def test_tiled_kernel_computes_r_itself(ext, tiled_routes, M, K, Ns, rank, alpha):
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(170 + M + K + rank, M, K, Ns, rank, with_bias=True)
+    mem = members_on_device(members, drop_left=1 if len(Ns) > 1 else None, with_bias=True)
+    xd, Rd = dev(x), dev(R)
+    with tuning(ext, proj_in_launch=0):
+        r_two = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+        y_two = ext.group_forward(xd, r_two, mem, 128, alpha, R=Rd)
+        assert ext.last_launch()["kernel"].startswith("skinny_tiled_kernel<") and not tiled_in_launch(ext), ext.last_launch()
+    for rep in range(3):
+        r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        y = ext.group_forward(xd, r, mem, 128, alpha, R=Rd)
+        assert tiled_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+        # the producers in front add an entry of r up like the projection launch, and the correction is applied in the
+        # same place: the same bits
+        assert torch.equal(r, r_two), f"r, launch {rep}"
+        for a, b in zip(y, y_two):
+            assert torch.equal(a, b), f"launch {rep}"
+    assert_close(r_two.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
+    for i, (m, got) in enumerate(zip(members, y_two)):
+        want = (oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128) if mem[i]["L"] is None else
+                oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], alpha))
+        assert_close(got.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"member {i}")
+
+
+def test_tiled_launches_and_replays_see_their_own_r(ext, tiled_routes):
+    """Launch after launch and replay after replay through the same workspace, each with other activations."""
+    M, K, Ns, rank = 8, 1024, [16384, 2048], 128
+    _, members, R = make_group(181, M, K, Ns, rank)
+    mem = members_on_device(members)
+    Rd = dev(R)
+    g = torch.Generator().manual_seed(19)
+    xs = torch.randn(M, K, generator=g).half().cuda()
+    r = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+        assert tiled_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+            again = ext.group_forward(xs, r, mem, 128, 1.0, R=Rd)
+        assert tiled_in_launch(ext)
+    torch.cuda.synchronize()
+    for rep in range(5):
+        xs.copy_(torch.randn(M, K, generator=g).half())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        xn = xs.cpu().numpy()
+        assert_close(r.cpu().numpy(), xn.astype(np.float64) @ R.astype(np.float64).T, f"r, replay {rep}")
+        for m, a, b in zip(members, outs, again):
+            want = oracle.corrected_linear_exact(xn, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0)
+            assert_close(a.cpu().numpy(), want, f"replay {rep}")
+            assert torch.equal(a, b), f"replay {rep}: two launches of one replay"
+
+
+@pytest.mark.parametrize("spin", [None, 0])
+def test_tiled_waves_that_never_see_the_ready_word(ext, tiled_routes, spin):
+    """With the producers' flags held down (or no patience at all) the waves that stage r for their workgroup compute
+    the pieces they would have loaded themselves; the caller still gets r from the producers in front."""
+    M, K, Ns, rank = 7, 512, [16640], 64
+    x, members, R = make_group(191, M, K, Ns, rank)
+    mem = members_on_device(members)
+    xd, Rd = dev(x), dev(R)
+    knobs = {"proj_in_launch": 2} if spin is None else {"proj_spin_limit": spin}
+    with tuning(ext, **knobs):
+        r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        y = ext.group_forward(xd, r, mem, 128, 1.0, R=Rd)
+        assert tiled_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+    assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
+    for m, got in zip(members, y):
+        assert_close(got.cpu().numpy(), oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0), "own r")
+
+
+def test_tiled_launch_that_leaves_no_room_keeps_the_projection_launch(ext, tiled_routes):
+    """Column tiles for every compute unit, K slices through the workspace, more than 16 rows: the projection launch goes
+    ahead as before, with the same results."""
+    for M, K, Ns, rank in [(8, 512, [40000], 64), (8, 4096, [2048], 64), (24, 1024, [16640], 64)]:
+        x, members, R = make_group(201 + M, M, K, Ns, rank)
+        mem = members_on_device(members)
+        r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+        y = ext.group_forward(dev(x), r, mem, 128, 1.0, R=dev(R))
+        assert ext.last_launch()["kernel"].startswith("skinny_tiled_kernel<") and not tiled_in_launch(ext), ext.last_launch()
+        torch.cuda.synchronize()
+        assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
+        for m, got in zip(members, y):
+            assert_close(got.cpu().numpy(), oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0), f"M={M} K={K}")
