@@ -185,7 +185,12 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
  * their weights instead of in front of them -- read r_out once they see that word.  The head of the workspace (8192
  * bytes) holds flags and ready word, the partial tiles of a split of K lie behind it.  Outputs agree with the
  * two-launch form to rounding (the correction is added last instead of first), r_out in the arithmetic of the small
- * projection kernels.
+ * projection kernels.  A launch that computes r itself is not cut into two slices of K (down_proj of an 8B layer: one
+ * launch instead of three).
+ * The kernel that streams the tiled copy does it at 5..16 token rows and ranks up to 256 where its grid is not cut into
+ * slices of K and leaves compute units free (gate|up): producers in front as above, and the waves that stage the
+ * activations of each workgroup look for the ready word when r is due in the stages, behind the last columns of K.  Same
+ * 8192 bytes at the head of the workspace; the same bits in r_out and in the outputs as the two-launch form.
  */
 int glowq_w4a16_group_forward_ws(const void* x, const void* r, const glowq_member_t* members, int n_members, int M,
                                  int K, int group_size, int rank, float alpha, void* workspace, size_t workspace_bytes,
