@@ -911,7 +911,7 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
       asked_for[bulk].store(shape, std::memory_order_release);
     }
     // The workgroups in front take the places the launch leaves free on the chip (its staging tiles allow one workgroup
-    // per compute unit), and only where those are enough for about one block of r per producer: every workgroup
+    // per compute unit), and only where those are enough for one to one and a half blocks of r per producer: every workgroup
     // of the launch then starts at once, the producers are done long before the first wave asks for r, and no workgroup
     // with a column tile waits for a place (one that does adds its whole run time to the launch: q|k|v of an 8B layer at
     // eight rows with 257 workgroups for 256 places 11.25 us against 11.05 with the projection launch in front; fewer
@@ -925,7 +925,10 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
     if (want > kSkinnyMaxProducers) want = kSkinnyMaxProducers;
     // (a few producers with two blocks are as far as it goes: 4 x 8 blocks, two to a producer, on o_proj of a 14B layer
     // at 16 rows: 16.4 us against 14.3 with the projection launch; 4 x 4 blocks, 2.7 to a producer: 16.1)
-    if (want < 1 || (9 * want < 8 * nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
+    // (up to about one and a half blocks per producer pay -- 8B shapes: q|k|v at 12 rows, 96 blocks for 63 producers, 11.0
+    // us against 11.7 with the projection launch; o_proj at 24 rows, 192 for 127, 11.2 against 12.4 -- two do not: q|k|v at
+    // 16 rows, 128 for 63, 13.2 against 12.0)
+    if (want < 1 || (13 * want < 8 * nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
     a.producers = (int)want;
     grid_x = front_grid(total, a.producers + 1);
   }
