@@ -8,12 +8,19 @@
 
 namespace glowq {
 
-// part: 4 x kM x kJ floats of LDS.  `store(m, j, value)` is called by thread m * kJ + j of the workgroup for the
-// entries inside [M, rank].  Threads 256 and up must not call this (the barrier inside counts the waves that arrive).
+// part: 4 x kM x kJ floats of LDS.  `store(m, j, value)` is called by thread m * kJ + j of the team for the
+// entries inside [M, rank].  A team is 256 threads, `tid` the thread's index in it: by default the first 256 threads of
+// the workgroup (threads 256 and up must then not call this: the barrier inside counts the waves that arrive).  Several
+// teams of one workgroup may each take a block of their own at the same time, with a `part` of their own; all of them
+// then have to call this equally often, a team without a block with `active` false (it only meets the barrier).
 template <int kM, int kJ, typename Store>
 __device__ __forceinline__ void proj_block_body(const half_t* __restrict__ x, const half_t* __restrict__ R, int M, int K, int rank,
-                                                int j0, int m0, float* part, Store&& store) {
-  const int tid = threadIdx.x;
+                                                int j0, int m0, float* part, Store&& store, int tid = (int)threadIdx.x,
+                                                bool active = true) {
+  if (!active) {
+    __syncthreads();
+    return;
+  }
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   float acc[kM][kJ];

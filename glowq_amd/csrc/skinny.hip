@@ -52,6 +52,7 @@ struct SkinnyArgs {
   unsigned long long* pub;  // [0]: the ready word; [kSkinnyFlags + p]: the flag of producer p
   unsigned spin;            // polls of the ready word before a wave computes its part of r itself
   int producers;            // workgroups that produce r
+  int teams;                // blocks of r a producer works on at a time: teams of four waves (1 or 2)
 };
 constexpr int kSkinnyFlags = 512;          // the producers' flags lie 4096 bytes behind the ready word
 constexpr int kSkinnyMaxProducers = 512;
@@ -298,11 +299,11 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(const SkinnyArgs g) {
 // code * x, and scale and zero-point are applied to that sum, y += s (sum c x - z sum x), with the fp32 sums of x per
 // token row and group taken when the activations are staged.  Five vector instructions per code word instead of
 // thirteen, and the arithmetic of the GEMV routes: weights never rounded to fp16.
-// kProj: the launch computes r = x R^T itself (SkinnyArgs).  The grid then has producers + 1 workgroups in front (roles
-// dealt as in handover.hpp).  Producer p takes the blocks p, p + producers, ... of four token rows by four rows of R with
-// its first four waves, in the arithmetic of shared_proj_block_kernel, writes them to r_out with stores that pass the caches private to a part of the
-// chip, waits until they are acknowledged and raises its flag (the launch's tag); the collector polls the flags
-// (bounded) and, when all are up, writes the ready word.  A wave with a correction block polls the ready word (bounded)
+// kProj: the launch computes r = x R^T itself (SkinnyArgs).  The grid then has `producers` workgroups in front (roles
+// dealt as in handover.hpp).  A producer's teams of four waves (one or two) each take every (producers x teams)-th block of
+// four token rows by four rows of R, in the arithmetic of shared_proj_block_kernel; the producer writes them to r_out with
+// stores that pass the caches private to a part of the chip, waits until they are acknowledged and raises its flag (the
+// launch's tag); the first producer then polls all flags (bounded) and, when all are up, writes the ready word.  A wave with a correction block polls the ready word (bounded)
 // once its weights are done, then reads its part of r with loads that pass those caches as well; a wave that never sees
 // the word computes the part of r it needs itself, so every wave ends whatever becomes of the producers.
 template <int kMT, int kNT, bool kBulk, bool kRaw, bool kProj = false>
@@ -318,24 +319,30 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
   unsigned long long tag = 0;
   if constexpr (kProj) {
     tag = launch_tag();
-    const int front = g.producers + 1;
+    const int front = g.producers;
     const int role = front_role(wg, front);
     if (role >= 0) {
       if (role >= front || blockIdx.y != 0) return;
-      if (role < g.producers) {
-        if (threadIdx.x >= 256) return;  // (the body's barriers count the waves that arrive)
-        float* part = reinterpret_cast<float*>(smem);
+      {
+        // teams of 256 threads, each with a block of its own at a time: two where the workgroup has eight waves (the
+        // round trips of two blocks overlap; the compute unit has nothing else to do)
+        const int teams = g.teams;
+        if ((int)threadIdx.x >= 256 * teams) return;  // (the body's barriers count the waves that arrive)
+        const int team = (int)threadIdx.x >> 8, tid = (int)threadIdx.x & 255;
+        float* part = reinterpret_cast<float*>(smem) + team * (4 * 16 + 16);
         float* vals = part + 4 * 16;
         const int jblocks = (g.rank + 3) >> 2, nblocks = jblocks * ((g.M + 3) >> 2);
-        // blocks of four token rows by four rows of R, dealt round robin to the producers
-        for (int b = role; b < nblocks; b += g.producers) {
+        // blocks of four token rows by four rows of R, dealt round robin to the teams of the producers
+        for (int b0 = role * teams; b0 < nblocks; b0 += g.producers * teams) {
+          const int b = b0 + team;
+          const bool active = b < nblocks;
           const int bj = b % jblocks, bm = b / jblocks;
           proj_block_body<4, 4>(g.x, g.R, g.M, g.K, g.rank, 4 * bj, 4 * bm, part,
-                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; });
+                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; }, tid, active);
           __syncthreads();
           // pairs of neighbouring entries of a token row go out as one 32-bit store (ranks are multiples of 8)
-          if (threadIdx.x < 8) {
-            const int mi = (int)threadIdx.x >> 1, pp = (int)threadIdx.x & 1;
+          if (active && tid < 8) {
+            const int mi = tid >> 1, pp = tid & 1;
             const int m = 4 * bm + mi, j = 4 * bj + 2 * pp;
             if (m < g.M && j < g.rank) {
               const h2 v = {(half_t)vals[mi * 4 + 2 * pp], (half_t)vals[mi * 4 + 2 * pp + 1]};
@@ -349,10 +356,10 @@ __global__ __launch_bounds__(512) void skinny_group_kernel(const SkinnyArgs g) {
         __syncthreads();
         if (threadIdx.x == 0 && g.spin != 0xFFFFFFFFu)  // (that value: a test in which the flags never go up)
           __hip_atomic_store(g.pub + kSkinnyFlags + role, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return;
       }
-      // the collector: one wave, lane l takes flags l, l + 64, ...
-      if (wave != 0) return;
+      // the first producer is also the collector: one wave, lane l takes flags l, l + 64, ...  (a workgroup of its own
+      // for this takes a place that a producer can use: 64 blocks of r for 64 free compute units)
+      if (role != 0 || wave != 0) return;
       bool all = false;
       for (unsigned spins = 0; !all && spins <= g.spin && g.spin != 0xFFFFFFFFu; ++spins) {
         bool mine = true;
@@ -917,7 +924,7 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
     // eight rows with 257 workgroups for 256 places 11.25 us against 11.05 with the projection launch in front; fewer
     // producers with more blocks each: down_proj 32 us against 19).
     const long capacity = (long)per_cu * num_cus;
-    long want = ((capacity - (long)total * a.slices) & ~3L) - 1;  // (the front is padded to a multiple of four: handover.hpp)
+    long want = (capacity - (long)total * a.slices) & ~3L;  // (the front is padded to a multiple of four: handover.hpp)
     static const int env_producers = getenv("GLOWQ_SKINNY_PRODUCERS") ? atoi(getenv("GLOWQ_SKINNY_PRODUCERS")) : 0;
     if (env_producers > 0) want = env_producers;
     const int nblocks = ((a.rank + 3) / 4) * ((a.M + 3) / 4);  // blocks of r: four token rows by four rows of R
@@ -928,9 +935,16 @@ static hipError_t launch_skinny_t(SkinnyArgs& a, int waves, int num_cus, size_t 
     // (up to about one and a half blocks per producer pay -- 8B shapes: q|k|v at 12 rows, 96 blocks for 63 producers, 11.0
     // us against 11.7 with the projection launch; o_proj at 24 rows, 192 for 127, 11.2 against 12.4 -- two do not: q|k|v at
     // 16 rows, 128 for 63, 13.2 against 12.0)
-    if (want < 1 || (13 * want < 8 * nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
+    // Blocks a producer works on at a time (teams of four waves): one where there is a producer for every block; two, in
+    // a workgroup of eight waves, where that brings all blocks of r under way at once; else, one at a time, up to about
+    // one and a half per producer.  8B shapes, us, inside the launch / projection launch in front: q|k|v at 12 rows (96
+    // blocks, 64 places) 9.4 / 11.7, o_proj at 24 rows (192, 128) 9.6 / 12.4; two rounds do not pay: q|k|v at 16 rows
+    // with 126 slots for 128 blocks 12.4 / 11.8, o_proj of a 14B layer at 16 rows (256 blocks, 190 slots) 15.4 / 14.4.
+    const int teams = (nblocks > want && waves >= 8 && nblocks <= 2 * want) ? 2 : 1;
+    if (want < 1 || (nblocks > want * teams && 13 * want < 8 * nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
+    a.teams = teams;
     a.producers = (int)want;
-    grid_x = front_grid(total, a.producers + 1);
+    grid_x = front_grid(total, a.producers);
   }
   hipLaunchKernelGGL(kern, dim3(grid_x, a.slices), dim3(waves * 64), lds, stream, a);
   if constexpr (kProj) note_launch(grid_x, a.slices, waves * 64, "skinny_group_kernel<%d,%d,%d,%d,1>", kMT, kNT, (int)bulk, (int)kRaw);
@@ -966,6 +980,7 @@ hipError_t launch_skinny(GroupDev& g, int num_cus, hipStream_t stream, bool raw)
   a.pub = g.pub;
   a.spin = g.pub_mute ? 0xFFFFFFFFu : g.pub_spin;
   a.producers = 0;
+  a.teams = 1;
   if (proj) {
     if (!ws_ok || ws_bytes < kSkinnyHandoverBytes) return hipErrorNotReady;
     a.r = nullptr;

@@ -31,8 +31,9 @@
 // acc += alpha * (r . L^T) from an accumulator of its own.
 // kProj: the launch computes r = x R^T itself.  Workgroups in front of the grid (roles dealt as in handover.hpp) produce
 // blocks of four token rows by four rows of R in the arithmetic of shared_proj_block_kernel and write them to r_out with
-// stores that pass the caches private to a part of the chip, each raises its flag when its stores are acknowledged, a
-// collector turns the flags into one ready word.  The producer waves of the other workgroups look for that word when
+// stores that pass the caches private to a part of the chip (two blocks at a time where the workgroup has eight waves
+// and more), each raises its flag when its stores are acknowledged, and the first of them turns the flags into one ready
+// word.  The producer waves of the other workgroups look for that word when
 // they are about to send r through the stages -- during the last super-block, so the producers in front have the whole
 // weight stream to get there -- and read r with loads that pass those caches; one that does not see the word within its
 // bound computes the pieces of r it would have loaded, so every wave ends whatever becomes of the workgroups in front.
@@ -78,6 +79,7 @@ struct TileArgs {
   unsigned long long* pub;  // [0]: the ready word; [kTiledFlags + p]: the flag of producer p
   unsigned spin;            // polls of the ready word before a producer wave computes its pieces of r itself
   int producers;            // workgroups in front that produce r
+  int teams;                // blocks of r a producer works on at a time: teams of four waves (1 or 2)
 };
 constexpr int kTiledFlags = 512;  // the producers' flags lie 4096 bytes behind the ready word
 constexpr int kTiledMaxProducers = 512;
@@ -165,13 +167,16 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
   unsigned long long tag = 0;
   if constexpr (kProj) {
     tag = launch_tag();
-    const int front = g.producers + 1;
+    const int front = g.producers;
     const int role = front_role(tile, front);
     if (role >= 0) {
       if (role >= front || blockIdx.y != 0) return;
-      if (role < g.producers) {
-        if (threadIdx.x >= 256) return;  // (the body's barriers count the waves that arrive)
-        float* part = reinterpret_cast<float*>(smem_all);
+      {
+        // teams of four waves, each with a block of its own at a time
+        const int teams = g.teams;
+        if ((int)threadIdx.x >= 256 * teams) return;  // (the body's barriers count the waves that arrive)
+        const int team = (int)threadIdx.x >> 8, ttid = (int)threadIdx.x & 255;
+        float* part = reinterpret_cast<float*>(smem_all) + team * (4 * 16 + 16);
         const int jblocks = (g.rank + 3) >> 2;
         float* vals = part + 4 * 16;
         const int nblocks = jblocks * ((M + 3) >> 2);
@@ -179,14 +184,16 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
         // half as many: 21.5 against 20.1 us at 12 rows on gate|up of an 8B layer, 32.0 against 27.5 on a 14B layer's;
         // three 16-byte pieces of every row in flight per thread instead of two, a row of 5120 columns in one round trip:
         // no difference.)
-        for (int b = role; b < nblocks; b += g.producers) {
+        for (int b0 = role * teams; b0 < nblocks; b0 += g.producers * teams) {
+          const int b = b0 + team;
+          const bool active = b < nblocks;
           const int bj = b % jblocks, bm = b / jblocks;
           proj_block_body<4, 4>(x, g.R, M, K, g.rank, 4 * bj, 4 * bm, part,
-                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; });
+                                [&](int m, int j, float v) { vals[(m - 4 * bm) * 4 + (j - 4 * bj)] = v; }, ttid, active);
           __syncthreads();
           // pairs of neighbouring entries of a token row go out as one 32-bit store (ranks are multiples of 8)
-          if (threadIdx.x < 8) {
-            const int mi = (int)threadIdx.x >> 1, pp = (int)threadIdx.x & 1;
+          if (active && ttid < 8) {
+            const int mi = ttid >> 1, pp = ttid & 1;
             const int m = 4 * bm + mi, j = 4 * bj + 2 * pp;
             if (m < M && j < g.rank) {
               const h2 v = {(half_t)vals[mi * 4 + 2 * pp], (half_t)vals[mi * 4 + 2 * pp + 1]};
@@ -200,10 +207,9 @@ void skinny_tiled_kernel(const half_t* __restrict__ x, const int M, const int K,
         __syncthreads();
         if (threadIdx.x == 0 && g.spin != 0xFFFFFFFFu)  // (that value: a test in which the flags never go up)
           __hip_atomic_store(g.pub + kTiledFlags + role, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return;
       }
-      // the collector: one wave, lane l takes flags l, l + 64, ...
-      if (threadIdx.x >= 64) return;
+      // the first producer is also the collector: one wave, lane l takes flags l, l + 64, ...
+      if (role != 0 || threadIdx.x >= 64) return;
       bool all = false;
       for (unsigned spins = 0; !all && spins <= g.spin && g.spin != 0xFFFFFFFFu; ++spins) {
         bool mine = true;
@@ -814,14 +820,15 @@ static hipError_t launch_tiled_t(TileArgs& a, const half_t* x, int num_cus, hipS
     // bandwidth and matrix cores, and the launch gets longer -- gate|up of a 14B layer at eight rows with 131 producers
     // beside 218 tiles 42 us against 30.5)
     const long capacity = per_cu >= 1 ? num_cus : 0;
-    long want = ((capacity - (long)a.tiles) & ~3L) - 1;  // (the front is padded to a multiple of four: handover.hpp)
+    long want = (capacity - (long)a.tiles) & ~3L;  // (the front is padded to a multiple of four: handover.hpp)
     if (env_producers > 0) want = env_producers;
     const int nblocks = ((a.rank + 3) / 4) * ((a.M + 3) / 4);  // blocks of r: four token rows by four rows of R
     if (want > nblocks) want = nblocks;
     if (want > kTiledMaxProducers) want = kTiledMaxProducers;
     if (threads < 256 || want < 1 || ((long)per_producer * want < nblocks && a.spin != 0xFFFFFFFFu)) return hipErrorNotReady;
     a.producers = (int)want;
-    grid_x = front_grid(a.tiles, a.producers + 1);
+    a.teams = (nblocks > want && threads >= 512) ? 2 : 1;  // two blocks at a time where the workgroup has the waves
+    grid_x = front_grid(a.tiles, a.producers);
   }
   hipLaunchKernelGGL(kern, dim3(grid_x, a.slices), dim3(threads), lds, stream, x, a.M, a.K, a.slices, a.mem[0].wt,
                      a.blk_end[0], a.mem[0].N, a.cw, a);
@@ -843,6 +850,7 @@ hipError_t launch_skinny_tiled(GroupDev& g, int num_cus, hipStream_t stream) {
   a.pub = g.pub;
   a.spin = g.pub_mute ? 0xFFFFFFFFu : g.pub_spin;
   a.producers = 0;
+  a.teams = 1;
   if (proj) {
     if (g.M > 16 || g.rank > 256 || (g.rank & 7) != 0 || (g.K & 7) != 0 || g.R == nullptr || g.r_out == nullptr || g.ws_bytes < kTiledHandoverBytes)
       return hipErrorNotReady;
