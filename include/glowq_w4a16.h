@@ -179,9 +179,9 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
  * projection launch in front gives; "proj_in_launch" of glowq_set_tuning switches it off.  As everywhere, calls that
  * share a workspace must not overlap.
  * The skinny MFMA route does the same at 2..32 token rows where its launch leaves enough compute units free for the
- * workgroups that produce r (one workgroup per block of four token rows by four rows of R; o_proj of an 8B layer at 8 and
- * 16 rows, q|k|v at 8): they write r_out with stores that pass the caches private to a part of the chip and raise a
- * tagged flag each, a collector turns the flags into one ready word, and the waves that apply the correction -- behind
+ * workgroups that produce r (a workgroup per one or two blocks of four token rows by four rows of R; every group of an 8B
+ * layer at 8 and 16 rows): they write r_out with stores that pass the caches private to a part of the chip and raise a
+ * tagged flag each, the first of them turns the flags into one ready word, and the waves that apply the correction -- behind
  * their weights instead of in front of them -- read r_out once they see that word.  The head of the workspace (8192
  * bytes) holds flags and ready word, the partial tiles of a split of K lie behind it.  Outputs agree with the
  * two-launch form to rounding (the correction is added last instead of first), r_out in the arithmetic of the small
