@@ -324,6 +324,10 @@ bool tiled_pays(const GroupDev& g) {
 //                   (GLOWQ_PROJ_SPIN_LIMIT; 0: never waits)
 std::atomic<int> g_proj_in_launch{clampi(env_or("GLOWQ_PROJ_IN_LAUNCH", 1), 0, 2)};
 std::atomic<int> g_proj_spin_limit{clampi(env_or("GLOWQ_PROJ_SPIN_LIMIT", 16384), 0, 1 << 24)};
+//   small_rows_in_launch  1: a fused call with three or four token rows and a workspace goes to the skinny kernel where its
+//                   launch computes r itself (GLOWQ_SMALL_ROWS_IN_LAUNCH; 0: always the 2..4-row kernels behind a
+//                   projection launch)
+std::atomic<int> g_small_rows_in_launch{clampi(env_or("GLOWQ_SMALL_ROWS_IN_LAUNCH", 1), 0, 1)};
 // the block the readers look at and, 4096 bytes behind it, the staging words, each with room for rank 256
 // (stream_kernel.hpp)
 constexpr size_t kProjHandoverBytes = 4096 + 256 * 8;
@@ -409,6 +413,25 @@ int run_group(GroupDev g, int route, hipStream_t stream) {
     g.pub = nullptr;
     return pe;
   };
+  // Three and four token rows of a fused call with a workspace: the skinny kernel in its raw-code form where its launch
+  // takes r along (one launch instead of the projection launch and the launch of the 2..4-row kernels); where it turns
+  // the shape down (gate|up: no compute units left for the producers of r), the route chosen above.  Group call, us, this /
+  // the route above, at 4 rows: 8B shapes q|k|v 8.6 / 10.0, o_proj 8.2 / 8.1, down_proj 15.9 / 15.8 (16.4 / 15.7 at three
+  // rows: the stream-scheduled kernel keeps a long K); 14B shapes (rank 256) q|k|v 12.2 / 13.1, o_proj 9.6 / 11.4,
+  // down_proj (on the 4x4x4 kernel) 20.7 / 26.7.
+  if (g.R != nullptr && g.M >= 3 && g.M <= 4 && g_small_rows_in_launch.load(std::memory_order_relaxed) != 0 &&
+      (route == kRouteQuad || route == kRouteStream || route == kRouteWaveDot || (route == kRouteQStream && g.K <= 8192)) && skinny_supported(g) &&
+      skinny_raw_form(g) && skinny_proj_in_launch(g)) {
+    g.pub = static_cast<unsigned long long*>(g.ws);
+    g.pub_spin = (unsigned)g_proj_spin_limit.load(std::memory_order_relaxed);
+    g.pub_mute = g_proj_in_launch.load(std::memory_order_relaxed) == 2;
+    note_launch(0, 0, 0, "%s", "skinny_codes_mfma");
+    e = launch_skinny(g, cus, stream, true);
+    if (e == hipSuccess) return GLOWQ_OK;
+    if (e != hipErrorNotReady) return fail(GLOWQ_ELAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+    e = hipSuccess;
+    g.pub = nullptr;
+  }
   const bool skinny_route = route == kRouteSkinny || route == kRouteSkinnyRaw;
   if (g.R != nullptr && ((route == kRouteStream && proj_in_launch(g)) || ((skinny_route || route == kRouteSkinnyTiled) && skinny_proj_in_launch(g)))) {
     // single token on the stream GEMV, a handful of rows on the skinny kernel: workgroups in front of the group launch
@@ -882,6 +905,7 @@ int glowq_set_tuning(const char* key, int value) {
   else if (strcmp(key, "tiled_shape_rule") == 0) { slot = &g_tiled_shape_rule; hi = 1; }
   else if (strcmp(key, "proj_in_launch") == 0) { slot = &g_proj_in_launch; hi = 2; }
   else if (strcmp(key, "proj_spin_limit") == 0) { slot = &g_proj_spin_limit; hi = 1 << 24; }
+  else if (strcmp(key, "small_rows_in_launch") == 0) { slot = &g_small_rows_in_launch; hi = 1; }
   if (slot == nullptr) return fail(GLOWQ_EINVAL, "unknown tuning key '%s'", key);
   if (value < lo || value > hi) return fail(GLOWQ_EINVAL, "tuning key '%s': value %d outside [%d, %d]", key, value, lo, hi);
   return slot->exchange(value);

@@ -144,12 +144,13 @@ class W4A16Extension:
 
     def _workspace(self, dev: torch.device, rows: int):
         """(pointer, bytes) of the workspace of the current stream of `dev`: one per stream, because calls that share
-        one must not overlap.  Calls with more than 4 token rows get the large one (many-row projection, split-K of the
-        GEMM and of the skinny kernels); single-token calls a small one, through which a group launch that computes r
-        itself hands it from the waves that produce it to the others; two to four rows use none.  A stream that meets
+        one must not overlap.  Calls with more than 2 token rows get the large one (many-row projection, split-K of the
+        GEMM and of the skinny kernels, hand-over words of the launches that compute r themselves); single-token calls
+        a small one, through which a group launch that computes r itself hands it from the waves that produce it to the
+        others; two rows use none.  A stream that meets
         its first such call while it is being captured into a graph goes without (the buffer would come from the
         graph's own memory pool)."""
-        if 1 < rows <= 4:
+        if rows == 2:
             return None, 0
         small = rows <= 1
         key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev), small)

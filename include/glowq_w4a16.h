@@ -186,7 +186,9 @@ int glowq_w4a16_group_forward_fused(const void* x, const void* R, void* r_out, c
  * bytes) holds flags and ready word, the partial tiles of a split of K lie behind it.  Outputs agree with the
  * two-launch form to rounding (the correction is added last instead of first), r_out in the arithmetic of the small
  * projection kernels.  A launch that computes r itself is not cut into two slices of K (down_proj of an 8B layer: one
- * launch instead of three).
+ * launch instead of three).  A fused call with three or four token rows and such a workspace takes this kernel too where
+ * its launch computes r itself (q|k|v, o_proj, down_proj; "small_rows_in_launch" of glowq_set_tuning switches that off),
+ * instead of the projection launch and the launch of the 2..4-row kernels.
  * The kernel that streams the tiled copy does it at 5..16 token rows and ranks up to 256 where its grid is not cut into
  * slices of K and leaves compute units free (gate|up): producers in front as above, and the waves that stage the
  * activations of each workgroup look for the ready word when r is due in the stages, behind the last columns of K.  Same

@@ -462,3 +462,26 @@ def test_tiled_launch_that_leaves_no_room_keeps_the_projection_launch(ext, tiled
         assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
         for m, got in zip(members, y):
             assert_close(got.cpu().numpy(), oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0), f"M={M} K={K}")
+
+
+# ---- three and four token rows: the fused call takes the skinny kernel where its launch computes r itself ------------------
+@pytest.mark.parametrize("M,K,Ns,rank", [(4, 4096, [1024, 256, 256], 128), (3, 5120, [640, 320], 256), (4, 14336, [512], 64)])
+def test_three_and_four_rows_take_the_launch_that_computes_r(ext, M, K, Ns, rank):
+    print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
+    x, members, R = make_group(270 + M + K + rank, M, K, Ns, rank, with_bias=True)
+    mem = members_on_device(members, drop_left=1 if len(Ns) > 1 else None, with_bias=True)
+    xd, Rd = dev(x), dev(R)
+    with tuning(ext, small_rows_in_launch=0):
+        r_two = torch.empty((M, rank), dtype=torch.float16, device="cuda")
+        y_two = ext.group_forward(xd, r_two, mem, 128, 1.0, R=Rd)
+        assert not skinny_in_launch(ext), ext.last_launch()
+    r = torch.full((M, rank), float("nan"), dtype=torch.float16, device="cuda")
+    y = ext.group_forward(xd, r, mem, 128, 1.0, R=Rd)
+    assert skinny_in_launch(ext), ext.last_launch()
+    torch.cuda.synchronize()
+    assert_close(r.cpu().numpy(), x.astype(np.float64) @ R.astype(np.float64).T, "r")
+    for i, (m, got) in enumerate(zip(members, y)):
+        want = (oracle.linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128) if mem[i]["L"] is None else
+                oracle.corrected_linear_exact(x, m["qweight"], m["qzeros"], m["scales"], 128, R, m["L"], 1.0))
+        assert_close(got.cpu().numpy(), want + m["bias"].astype(np.float64)[None, :], f"member {i}")
+        assert np.abs(got.float().cpu().numpy() - y_two[i].float().cpu().numpy()).max() <= 4e-3 * max(1.0, float(np.abs(want).max()))

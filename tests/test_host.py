@@ -360,7 +360,8 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     assert ext.set_tuning("proj_in_launch", 0) == 1 and ext.set_tuning("proj_in_launch", 2) == 0
     assert ext.set_tuning("proj_in_launch", 1) == 2
     assert ext.set_tuning("proj_spin_limit", 0) == 16384 and ext.set_tuning("proj_spin_limit", 16384) == 0
-    for key, bad in (("proj_in_launch", 3), ("proj_spin_limit", -1), ("proj_spin_limit", (1 << 24) + 1)):
+    assert ext.set_tuning("small_rows_in_launch", 0) == 1 and ext.set_tuning("small_rows_in_launch", 1) == 0
+    for key, bad in (("proj_in_launch", 3), ("proj_spin_limit", -1), ("proj_spin_limit", (1 << 24) + 1), ("small_rows_in_launch", 2)):
         with pytest.raises(ValueError):
             ext.set_tuning(key, bad)
 
