@@ -465,7 +465,7 @@ def test_tiled_launch_that_leaves_no_room_keeps_the_projection_launch(ext, tiled
 
 
 # ---- three and four token rows: the fused call takes the skinny kernel where its launch computes r itself ------------------
-@pytest.mark.parametrize("M,K,Ns,rank", [(4, 4096, [1024, 256, 256], 128), (3, 5120, [640, 320], 256), (4, 14336, [512], 64)])
+@pytest.mark.parametrize("M,K,Ns,rank", [(4, 4096, [4096, 1024, 1024], 128), (3, 5120, [5120], 256), (3, 4096, [4096], 64)])
 def test_three_and_four_rows_take_the_launch_that_computes_r(ext, M, K, Ns, rank):
     print(f"case M={M} K={K} Ns={Ns} rank={rank}", flush=True)
     x, members, R = make_group(270 + M + K + rank, M, K, Ns, rank, with_bias=True)
