@@ -298,7 +298,7 @@ int pick_route_rounded(const GroupDev& g, int force);
 
 //   tiled_min_m / tiled_max_m  token rows served by the matrix-core kernel that reads the tiled copy of the weights, where
 //                   every member of the group brings one (GLOWQ_TILED_MIN_M, GLOWQ_TILED_MAX_M; max 0 switches it off)
-std::atomic<int> g_tiled_min_m{clampi(env_or("GLOWQ_TILED_MIN_M", 5), 1, 64)};
+std::atomic<int> g_tiled_min_m{clampi(env_or("GLOWQ_TILED_MIN_M", 2), 1, 64)};
 std::atomic<int> g_tiled_max_m{clampi(env_or("GLOWQ_TILED_MAX_M", 64), 0, 64)};
 //   tiled_shape_rule  1: up to 32 rows only groups whose stream is long enough to pay for the kernel's start-up take the
 //                   tiled route, the others stay on the skinny kernel (GLOWQ_TILED_SHAPE_RULE; 0: every group that can).
@@ -313,6 +313,10 @@ bool tiled_pays(const GroupDev& g) {
   long rows = 0;
   for (int i = 0; i < g.n_members; ++i) rows += g.mem[i].N;
   const long code_bytes = rows * (long)g.K / 2;
+  // two to four rows: only the longest streams (gate|up of a 14B layer, 89 MB: 24.0 to 24.2 us against 26.1 to 27.6 on the
+  // 4x4x4 stream kernel with r given, 25.0 against 30.1 with the projection, which the launch then takes along; gate|up of
+  // an 8B layer, 59 MB: 17.5 against 14.8 to 15.8 with r given)
+  if (g.M < 5) return code_bytes >= 80L * 1000 * 1000;
   return code_bytes >= 40L * 1000 * 1000 || (g.M > 16 && code_bytes >= 24L * 1000 * 1000);
 }
 

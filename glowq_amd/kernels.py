@@ -98,7 +98,7 @@ _SIGNATURES = {
 
 
 # Calls with this many token rows and more bring the tiled copy of the weights along when they build descriptors per call.
-TILED_MIN_ROWS = 5
+TILED_MIN_ROWS = 2
 
 
 def tiled_enabled() -> bool:
@@ -144,14 +144,12 @@ class W4A16Extension:
 
     def _workspace(self, dev: torch.device, rows: int):
         """(pointer, bytes) of the workspace of the current stream of `dev`: one per stream, because calls that share
-        one must not overlap.  Calls with more than 2 token rows get the large one (many-row projection, split-K of the
+        one must not overlap.  Calls with two and more token rows get the large one (many-row projection, split-K of the
         GEMM and of the skinny kernels, hand-over words of the launches that compute r themselves); single-token calls
         a small one, through which a group launch that computes r itself hands it from the waves that produce it to the
-        others; two rows use none.  A stream that meets
+        others.  A stream that meets
         its first such call while it is being captured into a graph goes without (the buffer would come from the
         graph's own memory pool)."""
-        if rows == 2:
-            return None, 0
         small = rows <= 1
         key = (dev.index if dev.index is not None else torch.cuda.current_device(), self._stream(dev), small)
         ws = self._workspaces.get(key)

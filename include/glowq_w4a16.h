@@ -285,9 +285,10 @@ int glowq_probe_empty_launch(int grid, int block, void* stream);
  * was measured faster on (1, the default) or for every shape it can take (0).
  * "skinny_codes_max_m" (0..64, default 8): token rows up to which the skinny MFMA kernel runs in its raw-code form
  * (route 7) where that applies; above it is slower than dequantising first (the work on the sums grows with the rows).
- * "tiled_min_m" / "tiled_max_m" (default 5 / 64; max 0 switches the route off): token rows served by the kernel that
+ * "tiled_min_m" / "tiled_max_m" (default 2 / 64; max 0 switches the route off): token rows served by the kernel that
  * streams the tiled copy of the weights where every member brings one; "tiled_shape_rule" (0 / 1): up to 32 rows only
- * for groups whose stream is long enough to pay for its start-up (1, the default) or for every group (0).
+ * for groups whose stream is long enough to pay for its start-up (1, the default: 80 MB of codes up to 4 rows, 40 MB up to
+ * 16, 24 MB up to 32) or for every group (0).
  * "proj_in_launch" (0 / 1, default 1): a fused single-token call with a workspace computes r inside the group launch
  * where that applies (glowq_w4a16_group_forward_fused_ws); 2, for tests, keeps the producing waves from handing their
  * entries over, so that every reader runs into "proj_spin_limit" (default 16384, 0 = never waits: the number of times

@@ -306,8 +306,10 @@ def test_abi_rejects_bad_arguments_without_a_gpu():
     # 16384 columns; at two rows not where the last 2048-column slice of a short group's rows is mostly empty
     assert ext.route(2, 4096, 28672) == "quad_stream_gemv" and ext.route(4, 4096, 4096) == "quad_stream_gemv"
     assert ext.route(3, 14336, 4096) == "quad_stream_gemv" and ext.route(4, 8192, 10240) == "quad_stream_gemv"
-    assert ext.route(2, 5120, 5120) != "quad_stream_gemv" and ext.route(2, 5120, 34816) == "quad_stream_gemv"
-    assert ext.route(4, 5120, 5120) == "quad_stream_gemv" and ext.route(4, 6144, 28672) == "quad_stream_gemv"
+    assert ext.route(2, 5120, 5120) != "quad_stream_gemv" and ext.route(2, 5120, 34816, tiled=False) == "quad_stream_gemv"
+    # with the tiled copy the longest streams (80 MB of codes and more) go to the kernel that streams it from two rows on
+    assert ext.route(2, 5120, 34816, tiled=True) == "skinny_tiled_mfma" and ext.route(4, 4096, 28672, tiled=True) == "quad_stream_gemv"
+    assert ext.route(4, 5120, 5120) == "quad_stream_gemv" and ext.route(4, 6144, 28672, tiled=False) == "quad_stream_gemv"
     assert ext.route(1, 4096, 4096) != "quad_stream_gemv" and ext.route(5, 4096, 4096) != "quad_stream_gemv"
     assert ext.route(4, 4096, 4096, group_size=64) != "quad_stream_gemv" and ext.route(4, 17408, 5120) != "quad_stream_gemv"
     rule = ext.set_tuning("qstream_shape_rule", 0)
