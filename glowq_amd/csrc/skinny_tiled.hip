@@ -1,4 +1,4 @@
-// Matrix-core kernel for a handful of token rows (5..64) on members that bring the tiled copy of their weights
+// Matrix-core kernel for a handful of token rows (5..64, from 2 on the longest streams) on members that bring the tiled copy of their weights
 // (tiled.hpp): the weights are streamed once, every 16-byte load of a wave is one contiguous kilobyte and lands in
 // the lanes' registers as the B operand of v_mfma_f32_32x32x16_f16 -- no pass through LDS, no per-lane scale and
 // zero-point gather (both ride in the stream).

@@ -321,7 +321,7 @@ class W4A16Extension:
         if M < TILED_MIN_ROWS or not tiled_enabled():
             return False
         route = self.lib.glowq_w4a16_route_tiled(int(M), int(K), int(N_total), int(group_size), int(ldw_i32))
-        # 8: the kernel that streams the copy at 5..64 rows; 2: the MFMA GEMM, which takes its B operand from the copy where
+        # 8: the kernel that streams the copy at 5..64 rows (2..4 on the longest streams); 2: the MFMA GEMM, which takes its B operand from the copy where
         # the layout applies (its lane order is the matrix instruction's)
         return route == 8 or (route == 2 and self.lib.glowq_tiled_bytes(int(N_total), int(K), int(group_size)) > 0)
 

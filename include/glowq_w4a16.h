@@ -202,7 +202,7 @@ int glowq_w4a16_group_forward_fused_ws(const void* x, const void* R, void* r_out
                                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Tiled copy of a member's weights for the matrix-core routes (5..64 token rows): the codes of 32 output rows and 256
+ * Tiled copy of a member's weights for the matrix-core routes (5..64 token rows, from 2 on groups of 80 MB of codes and more): the codes of 32 output rows and 256
  * input columns at a time in the order in which one coalesced 16-byte-per-lane load hands every lane the B operand of
  * the 32x32x16 matrix instruction, with each lane's scale and -(1024 + zero-point) behind them (4352 bytes per
  * (row block, super-block); layout in glowq_amd/csrc/tiled.hpp).  A deterministic function of the canonical buffers,
